@@ -1,0 +1,25 @@
+"""Shared fixtures.  Tests marked `gpu` need an MI355X and the built HIP library; everything else
+runs on the CPU (oracle pins, host logic, C-ABI symbol checks)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture
+def rng():
+    return np.random.default_rng(0)
+
+
+def f16(a):
+    """fp32 -> fp16 with IEEE round-to-nearest-even (what the device conversion does)."""
+    return np.asarray(a, dtype=np.float32).astype(np.float16)

@@ -1,0 +1,145 @@
+// Shared device/host helpers for the gfx950 kernels of libaxhip.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "axhip.h"
+
+namespace axhip {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+inline hipStream_t as_stream(axhip_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Maps a launch error to a Status value.
+inline int launch_status() {
+  return hipGetLastError() == hipSuccess ? AXHIP_OK : AXHIP_DEVICE_ERROR;
+}
+
+inline bool is_float_dtype(int dt) { return dt == AXHIP_FLOAT16 || dt == AXHIP_FLOAT32; }
+
+// ---- 16-byte vector access ---------------------------------------------------------------------
+struct alignas(16) Vec16 {
+  uint32_t w[4];
+};
+
+__device__ __forceinline__ Vec16 ld16(const void *p) { return *reinterpret_cast<const Vec16 *>(p); }
+__device__ __forceinline__ void st16(void *p, const Vec16 &v) { *reinterpret_cast<Vec16 *>(p) = v; }
+
+__device__ __forceinline__ half2_t as_half2(uint32_t w) { return __builtin_bit_cast(half2_t, w); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+// Eight consecutive elements of T as fp32.
+template <typename T>
+struct Row8;
+
+template <>
+struct Row8<__half> {
+  // 8 halves = one 16-byte load
+  static __device__ __forceinline__ void load(const __half *p, float (&f)[8]) {
+    const Vec16 v = ld16(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const half2_t h = as_half2(v.w[i]);
+      f[2 * i] = static_cast<float>(h.x);
+      f[2 * i + 1] = static_cast<float>(h.y);
+    }
+  }
+  static __device__ __forceinline__ void store(__half *p, const float (&f)[8]) {
+    Vec16 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      half2_t h;
+      h.x = static_cast<_Float16>(f[2 * i]);  // round-to-nearest-even
+      h.y = static_cast<_Float16>(f[2 * i + 1]);
+      v.w[i] = as_u32(h);
+    }
+    st16(p, v);
+  }
+};
+
+template <>
+struct Row8<float> {
+  static __device__ __forceinline__ void load(const float *p, float (&f)[8]) {
+    const Vec16 a = ld16(p), b = ld16(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[i] = __builtin_bit_cast(float, a.w[i]);
+      f[4 + i] = __builtin_bit_cast(float, b.w[i]);
+    }
+  }
+  static __device__ __forceinline__ void store(float *p, const float (&f)[8]) {
+    Vec16 a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a.w[i] = __builtin_bit_cast(uint32_t, f[i]);
+      b.w[i] = __builtin_bit_cast(uint32_t, f[4 + i]);
+    }
+    st16(p, a);
+    st16(p + 4, b);
+  }
+};
+
+// Scalar element access as fp32 (tails, odd sizes).
+__device__ __forceinline__ float ldf(const __half *p) { return __half2float(*p); }
+__device__ __forceinline__ float ldf(const float *p) { return *p; }
+__device__ __forceinline__ void stf(__half *p, float v) { *p = __float2half_rn(v); }
+__device__ __forceinline__ void stf(float *p, float v) { *p = v; }
+
+// ---- cross-lane sums with DPP (no LDS traffic) -------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over aligned groups of LANES consecutive lanes (LANES in {1,2,4,8,16,32,64}); every lane of a
+// group ends with the same bits because each step adds the same two partner values.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float x) {
+  if constexpr (LANES >= 2) x += dpp_f32<0xB1>(x);   // quad_perm [1,0,3,2]
+  if constexpr (LANES >= 4) x += dpp_f32<0x4E>(x);   // quad_perm [2,3,0,1]
+  if constexpr (LANES >= 8) x += dpp_f32<0x141>(x);  // row_half_mirror
+  if constexpr (LANES >= 16) x += dpp_f32<0x140>(x); // row_mirror
+  if constexpr (LANES >= 32) x += __shfl_xor(x, 16, 64);
+  if constexpr (LANES >= 64) x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+template <int LANES>
+__device__ __forceinline__ float group_max(float x) {
+  if constexpr (LANES >= 2) x = fmaxf(x, dpp_f32<0xB1>(x));
+  if constexpr (LANES >= 4) x = fmaxf(x, dpp_f32<0x4E>(x));
+  if constexpr (LANES >= 8) x = fmaxf(x, dpp_f32<0x141>(x));
+  if constexpr (LANES >= 16) x = fmaxf(x, dpp_f32<0x140>(x));
+  if constexpr (LANES >= 32) x = fmaxf(x, __shfl_xor(x, 16, 64));
+  if constexpr (LANES >= 64) x = fmaxf(x, __shfl_xor(x, 32, 64));
+  return x;
+}
+
+// Block-wide sum for blocks of NWAVES wavefronts; `smem` holds NWAVES floats.
+template <int NWAVES>
+__device__ __forceinline__ float block_sum(float x, float *smem) {
+  x = group_sum<64>(x);
+  if constexpr (NWAVES == 1) return x;
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) smem[wave] = x;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NWAVES; ++i) t += smem[i];
+  __syncthreads();
+  return t;
+}
+
+}  // namespace axhip

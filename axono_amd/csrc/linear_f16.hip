@@ -1,0 +1,398 @@
+// fp16 Linear: out[M,N] = x[M,K] . W[N,K]^T (+ bias), fp32 accumulation on the matrix cores.
+//
+// Both operands are K-contiguous, which is what the MFMA register layouts want: for
+// v_mfma_f32_16x16x32_f16 every lane supplies 8 consecutive K elements of one row, i.e. exactly one
+// 16-byte load.  Which 8 elements of the 32-wide K step a lane takes does not matter as long as the
+// W fragment and the x fragment agree, so the lanes are assigned so that the four lanes serving a
+// row read 64 consecutive bytes per load and 256 consecutive bytes per unrolled step.
+//
+// Skinny M (decode, M <= 32): the weight matrix is streamed from HBM exactly once and the work is
+// HBM-bound.  A wavefront owns NT*16 rows of W and a K slice, with the W rows as the MFMA "A"
+// operand and the (few) x rows as "B", so the output fragment holds out^T.  Nothing is staged
+// through LDS: x is small and stays in L2.  The four wavefronts of a workgroup take four K slices
+// of the same rows and add their fragments through LDS; further K splitting across workgroups
+// (needed to fill 256 CUs when N is small) goes through fp32 partial sums in a workspace and a
+// small reduction kernel.
+//
+// Larger M runs a tiled GEMM (128x128 output tile per workgroup, 32x32x16 MFMA, operands staged
+// through LDS with register double buffering); it is MFMA-bound once M reaches a few hundred rows.
+#include "common.hpp"
+
+namespace axhip {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kMaxOuterSplits = 8;
+constexpr int kSkinnyMaxM = 32;
+
+struct LinearTuning {
+  int target_waves = 2048;  // wavefronts to aim for in the skinny kernel (256 CUs x 8)
+  int force_nt = 0;         // > 0: rows-of-16 per wavefront (1, 2 or 4)
+  int force_ks_outer = 0;   // > 0: K splits across workgroups
+};
+LinearTuning g_lin;
+
+struct SkinnyPlan {
+  int nt, mt, ks_outer, k_per_wave;
+};
+
+SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
+  SkinnyPlan p;
+  p.mt = M <= 16 ? 1 : 2;
+  if (g_lin.force_nt > 0)
+    p.nt = g_lin.force_nt;
+  else if (p.mt == 2)
+    p.nt = 2;
+  else
+    p.nt = N >= 32768 ? 4 : (N >= 8192 ? 2 : 1);
+  if (p.mt == 2 && p.nt > 2) p.nt = 2;
+  const int64_t ntiles = (N + p.nt * 16 - 1) / (p.nt * 16);
+  int64_t ks = g_lin.force_ks_outer > 0
+                   ? g_lin.force_ks_outer
+                   : (g_lin.target_waves + ntiles * kWaves - 1) / (ntiles * kWaves);
+  const int64_t cap = K / (kWaves * 256);  // at least 256 of K per wavefront
+  if (ks > cap) ks = cap;
+  if (ks > kMaxOuterSplits) ks = kMaxOuterSplits;
+  if (ks < 1) ks = 1;
+  int64_t kpw = (K + kWaves * ks - 1) / (kWaves * ks);
+  kpw = (kpw + 127) / 128 * 128;
+  p.ks_outer = static_cast<int>((K + kWaves * kpw - 1) / (kWaves * kpw));
+  p.k_per_wave = static_cast<int>(kpw);
+  return p;
+}
+
+__device__ __forceinline__ half8_t zero_h8() {
+  half8_t z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = static_cast<_Float16>(0.0f);
+  return z;
+}
+
+__device__ __forceinline__ half8_t load_h8(const __half *p) {
+  return __builtin_bit_cast(half8_t, ld16(p));
+}
+
+// 8 fp32 activations -> fp16 round-to-nearest-even (the conversion the reference applies to x
+// before its GEMM)
+__device__ __forceinline__ half8_t load_h8(const float *p) {
+  const Vec16 a = ld16(p), b = ld16(p + 4);
+  half8_t h;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    h[i] = static_cast<_Float16>(__builtin_bit_cast(float, a.w[i]));
+    h[4 + i] = static_cast<_Float16>(__builtin_bit_cast(float, b.w[i]));
+  }
+  return h;
+}
+
+struct LinearArgs {
+  const void *x;
+  const __half *w;
+  const __half *bias;
+  void *out;
+  float *partial;  // [ks_outer, M, N] when ks_outer > 1
+  int M, K, N;
+  int k_per_wave, ks_outer, out_f16;
+};
+
+// Final store of 4 consecutive n for one m (bias added here when this is the last reduction).
+__device__ __forceinline__ void store_out4(const LinearArgs &a, int m, int n, const float (&v)[4],
+                                           bool add_bias) {
+  if (m >= a.M) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    if (n + r >= a.N) continue;
+    float y = v[r];
+    if (add_bias && a.bias) y += __half2float(a.bias[n + r]);
+    const int64_t o = static_cast<int64_t>(m) * a.N + n + r;
+    if (a.out_f16)
+      static_cast<__half *>(a.out)[o] = __float2half_rn(y);
+    else
+      static_cast<float *>(a.out)[o] = y;
+  }
+}
+
+template <int NT, int MT, typename XT>
+__global__ __launch_bounds__(kThreads) void linear_skinny_kernel(LinearArgs a) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n_base = blockIdx.x * (NT * 16);
+  const int kso = blockIdx.y;
+  const int m_base = blockIdx.z * (MT * 16);
+  const int k_begin = (kso * kWaves + wave) * a.k_per_wave;
+  const int k_end = min(k_begin + a.k_per_wave, a.K);
+  const XT *x = static_cast<const XT *>(a.x);
+
+  float4_t acc[NT][MT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const __half *wrow[NT];
+  bool wok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int row = n_base + t * 16 + r;
+    wok[t] = row < a.N;
+    wrow[t] = a.w + static_cast<int64_t>(wok[t] ? row : 0) * a.K;
+  }
+  const XT *xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) {
+    const int m = m_base + u * 16 + r;
+    xok[u] = m < a.M;
+    xrow[u] = x + static_cast<int64_t>(xok[u] ? m : 0) * a.K;
+  }
+
+  for (int kk = k_begin; kk < k_end; kk += 128) {
+    half8_t af[NT][4], bf[MT][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kc = kk + (j * 4 + g) * 8;
+      const bool kin = kc < k_end;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) af[t][j] = (kin && wok[t]) ? load_h8(wrow[t] + kc) : zero_h8();
+#pragma unroll
+      for (int u = 0; u < MT; ++u) bf[u][j] = (kin && xok[u]) ? load_h8(xrow[u] + kc) : zero_h8();
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int u = 0; u < MT; ++u)
+          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t][j], bf[u][j], acc[t][u], 0, 0, 0);
+  }
+
+  // add the four K slices of this workgroup
+  __shared__ float4_t red[kWaves - 1][NT * MT][64];
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int u = 0; u < MT; ++u) red[wave - 1][t * MT + u][lane] = acc[t][u];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+      float4_t s = acc[t][u];
+#pragma unroll
+      for (int w = 0; w < kWaves - 1; ++w) s += red[w][t * MT + u][lane];
+      // fragment layout: this lane holds out[m = m_base + u*16 + r][n = n_base + t*16 + 4g + 0..3]
+      const int m = m_base + u * 16 + r;
+      const int n = n_base + t * 16 + 4 * g;
+      const float v[4] = {s[0], s[1], s[2], s[3]};
+      if (a.ks_outer == 1) {
+        store_out4(a, m, n, v, true);
+      } else if (m < a.M) {
+        float *dst = a.partial + (static_cast<int64_t>(kso) * a.M + m) * a.N + n;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (n + q < a.N) dst[q] = v[q];
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void linear_reduce_kernel(LinearArgs a) {
+  const int64_t total = static_cast<int64_t>(a.M) * a.N;
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= total) return;
+  float s = 0.f;
+  for (int k = 0; k < a.ks_outer; ++k) s += a.partial[static_cast<int64_t>(k) * total + i];
+  if (a.bias) s += __half2float(a.bias[i % a.N]);
+  if (a.out_f16)
+    static_cast<__half *>(a.out)[i] = __float2half_rn(s);
+  else
+    static_cast<float *>(a.out)[i] = s;
+}
+
+template <int NT, int MT, typename XT>
+void launch_skinny(const LinearArgs &a, hipStream_t st) {
+  const dim3 grid((a.N + NT * 16 - 1) / (NT * 16), a.ks_outer, (a.M + MT * 16 - 1) / (MT * 16));
+  hipLaunchKernelGGL((linear_skinny_kernel<NT, MT, XT>), grid, dim3(kThreads), 0, st, a);
+}
+
+template <typename XT>
+void dispatch_skinny(const LinearArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  if (p.mt == 1) {
+    if (p.nt == 4)
+      launch_skinny<4, 1, XT>(a, st);
+    else if (p.nt == 2)
+      launch_skinny<2, 1, XT>(a, st);
+    else
+      launch_skinny<1, 1, XT>(a, st);
+  } else {
+    if (p.nt == 2)
+      launch_skinny<2, 2, XT>(a, st);
+    else
+      launch_skinny<1, 2, XT>(a, st);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Tiled GEMM for M > 32.  Workgroup tile 128 (m) x 128 (n), K step 32; four wavefronts in a 2x2
+// arrangement, each computing 64x64 with 2x2 MFMA 32x32x16 tiles.  Operands go global -> registers
+// -> LDS (rows padded by 16 bytes against bank conflicts) -> MFMA fragments; the global loads of
+// step k+1 are issued before the MFMAs of step k.
+// ------------------------------------------------------------------------------------------------
+constexpr int kTM = 128, kTN = 128, kTK = 32;
+constexpr int kLdsRow = kTK + 8;  // halves per LDS row (64 B data + 16 B pad)
+
+template <typename XT>
+__global__ __launch_bounds__(kThreads) void linear_gemm_kernel(LinearArgs a) {
+  __shared__ __attribute__((aligned(16))) _Float16 sx[kTM][kLdsRow];
+  __shared__ __attribute__((aligned(16))) _Float16 sw[kTN][kLdsRow];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int m0 = blockIdx.y * kTM, n0 = blockIdx.x * kTN;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const XT *x = static_cast<const XT *>(a.x);
+
+  // global -> register staging: 128 rows x 32 halves = 512 16-byte chunks per operand, 2 per thread
+  const int lr = tid >> 2;        // 0..63 (+64 for the second chunk)
+  const int lc = (tid & 3) * 8;   // k offset of the chunk
+  half8_t gx[2], gw[2];
+  auto load_global = [&](int kk) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int row = lr + h * 64;
+      const int kc = kk + lc;
+      const bool kin = kc < a.K;
+      gx[h] = (kin && m0 + row < a.M) ? load_h8(x + static_cast<int64_t>(m0 + row) * a.K + kc) : zero_h8();
+      gw[h] = (kin && n0 + row < a.N) ? load_h8(a.w + static_cast<int64_t>(n0 + row) * a.K + kc) : zero_h8();
+    }
+  };
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      *reinterpret_cast<half8_t *>(&sx[lr + h * 64][lc]) = gx[h];
+      *reinterpret_cast<half8_t *>(&sw[lr + h * 64][lc]) = gw[h];
+    }
+  };
+
+  float16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int fr = lane & 31, fk = (lane >> 5) * 8;  // fragment row / k offset within a 16-wide K step
+  load_global(0);
+  for (int kk = 0; kk < a.K; kk += kTK) {
+    __syncthreads();  // previous step's fragment reads are done
+    store_lds();
+    __syncthreads();
+    if (kk + kTK < a.K) load_global(kk + kTK);
+#pragma unroll
+    for (int ks = 0; ks < kTK; ks += 16) {
+      half8_t fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const half8_t *>(&sw[wn + i * 32 + fr][ks + fk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const half8_t *>(&sx[wm + j * 32 + fr][ks + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // 32x32 fragment: rows are W rows (n), columns are x rows (m); lane holds column lane%32 and rows
+  // 8*blk + 4*(lane/32)... : element e -> row 8*(e/4) + (lane/32)*4 + e%4
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = m0 + wm + j * 32 + (lane & 31);
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk) {
+        const int n = n0 + wn + i * 32 + blk * 8 + (lane >> 5) * 4;
+        const float v[4] = {acc[i][j][blk * 4], acc[i][j][blk * 4 + 1], acc[i][j][blk * 4 + 2],
+                            acc[i][j][blk * 4 + 3]};
+        store_out4(a, m, n, v, true);
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace axhip
+
+using namespace axhip;
+
+extern "C" {
+
+// Measurement hook for sweeps (0 restores a default).
+AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_ks_outer) {
+  g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
+  g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
+  g_lin.force_ks_outer = force_ks_outer > 0 ? force_ks_outer : 0;
+}
+
+AXHIP_API size_t axhip_linear_f16_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+  if (M <= 0 || K <= 0 || N <= 0 || M > kSkinnyMaxM) return 0;
+  // enough for any split count the skinny kernel may choose
+  return static_cast<size_t>(kMaxOuterSplits) * M * N * sizeof(float);
+}
+
+AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const void *bias, void *out,
+                               int out_dtype, int64_t M, int64_t K, int64_t N, void *workspace,
+                               size_t workspace_bytes, axhip_stream stream) {
+  if (!is_float_dtype(x_dtype) || !is_float_dtype(out_dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (M < 0 || K <= 0 || N <= 0 || K % 8 != 0) return AXHIP_INVALID_ARGUMENT;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+  if (M == 0) return AXHIP_OK;
+  if (!x || !w || !out) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return AXHIP_INVALID_PTR;
+  hipStream_t st = as_stream(stream);
+  LinearArgs a;
+  a.x = x;
+  a.w = static_cast<const __half *>(w);
+  a.bias = static_cast<const __half *>(bias);
+  a.out = out;
+  a.partial = nullptr;
+  a.M = static_cast<int>(M);
+  a.K = static_cast<int>(K);
+  a.N = static_cast<int>(N);
+  a.out_f16 = out_dtype == AXHIP_FLOAT16;
+  a.ks_outer = 1;
+  a.k_per_wave = 0;
+
+  if (M <= kSkinnyMaxM) {
+    const SkinnyPlan p = plan_skinny(M, K, N);
+    a.ks_outer = p.ks_outer;
+    a.k_per_wave = p.k_per_wave;
+    if (p.ks_outer > 1) {
+      const size_t need = static_cast<size_t>(p.ks_outer) * M * N * sizeof(float);
+      if (!workspace || workspace_bytes < need) return AXHIP_INVALID_ARGUMENT;
+      a.partial = static_cast<float *>(workspace);
+    }
+    if (x_dtype == AXHIP_FLOAT16)
+      dispatch_skinny<__half>(a, p, st);
+    else
+      dispatch_skinny<float>(a, p, st);
+    if (p.ks_outer > 1) {
+      const int64_t total = M * N;
+      hipLaunchKernelGGL(linear_reduce_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
+                         dim3(kThreads), 0, st, a);
+    }
+    return launch_status();
+  }
+  const dim3 grid((a.N + kTN - 1) / kTN, (a.M + kTM - 1) / kTM);
+  if (grid.y > 65535) return AXHIP_INVALID_ARGUMENT;
+  if (x_dtype == AXHIP_FLOAT16)
+    hipLaunchKernelGGL((linear_gemm_kernel<__half>), grid, dim3(kThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL((linear_gemm_kernel<float>), grid, dim3(kThreads), 0, st, a);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,690 @@
+// Bandwidth-bound row-wise and elementwise operators of the decode step: add_rms_norm, rms_norm,
+// silu_mul, add, fp16<->fp32 cast, the rotary family, KV-cache append, concat, embedding, argmax.
+//
+// All of them move each byte once with 16-byte accesses (8 fp16 or 2x4 fp32 elements per lane),
+// compute in fp32 and round once at the final store.  At decode sizes (tens of rows) they are
+// launch-latency bound; the layouts are chosen so the same kernels stream at HBM speed when the
+// row count is large (prefill).
+#include <cmath>
+
+#include "common.hpp"
+
+namespace axhip {
+namespace {
+
+constexpr int kBlock = 256;
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+inline unsigned blocks_for(int64_t items, int per_block) {
+  return static_cast<unsigned>((items + per_block - 1) / per_block);
+}
+
+// ------------------------------------------------------------------------------------------------
+// add_rms_norm / rms_norm.  TPR threads cooperate on one row (64: one wavefront, for short rows
+// such as per-head q/k norm; 256: the whole workgroup).  Each thread owns 8-element chunks at
+// stride TPR*8 and keeps up to kRegChunks of them in registers between the two passes.
+// ------------------------------------------------------------------------------------------------
+constexpr int kRegChunks = 4;
+
+template <typename T, typename WT, int TPR, bool ADD>
+__global__ __launch_bounds__(kBlock) void rms_norm_kernel(const T *__restrict__ x,
+                                                          const T *__restrict__ res,
+                                                          const WT *__restrict__ w, float eps,
+                                                          T *__restrict__ y, T *__restrict__ out,
+                                                          int64_t rows, int hidden, int vec_ok) {
+  constexpr int RPB = kBlock / TPR;
+  __shared__ float red[kBlock / 64];
+  const int lane = threadIdx.x % TPR;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * RPB + threadIdx.x / TPR;
+  const bool live = row < rows;
+  const int64_t off = (live ? row : 0) * hidden;
+  // whole 8-element chunks (only when rows start on 16-byte boundaries); the rest goes element by element
+  const int nvec = vec_ok ? hidden / 8 : 0;
+
+  float keep[kRegChunks][8];
+  float ss = 0.0f;
+  if (live) {
+    int c = 0;
+    for (int i = lane; i < nvec; i += TPR, ++c) {
+      float a[8];
+      Row8<T>::load(x + off + i * 8, a);
+      if (ADD) {
+        float r[8];
+        Row8<T>::load(res + off + i * 8, r);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] += r[j];
+        Row8<T>::store(y + off + i * 8, a);  // the only rounding of y; the norm uses the fp32 sum
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(a[j], a[j], ss);
+      if (c < kRegChunks) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) keep[c][j] = a[j];
+      }
+    }
+    for (int i = nvec * 8 + lane; i < hidden; i += TPR) {
+      float a = ldf(x + off + i);
+      if (ADD) {
+        a += ldf(res + off + i);
+        stf(y + off + i, a);
+      }
+      ss = __builtin_fmaf(a, a, ss);
+    }
+  }
+  if (TPR == 64)
+    ss = group_sum<64>(ss);
+  else
+    ss = block_sum<kBlock / 64>(ss, red);
+  if (!live) return;
+  const float rms = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
+  int c = 0;
+  for (int i = lane; i < nvec; i += TPR, ++c) {
+    float a[8], o[8];
+    if (c < kRegChunks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a[j] = keep[c][j];
+    } else {  // recompute the fp32 sum rather than read back the rounded y
+      Row8<T>::load(x + off + i * 8, a);
+      if (ADD) {
+        float r[8];
+        Row8<T>::load(res + off + i * 8, r);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] += r[j];
+      }
+    }
+    if (w) {
+      float wv[8];
+      Row8<WT>::load(w + i * 8, wv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = a[j] * rms * wv[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = a[j] * rms;
+    }
+    Row8<T>::store(out + off + i * 8, o);
+  }
+  for (int i = nvec * 8 + lane; i < hidden; i += TPR) {
+    float a = ldf(x + off + i);
+    if (ADD) a += ldf(res + off + i);
+    stf(out + off + i, w ? a * rms * ldf(w + i) : a * rms);
+  }
+}
+
+template <typename T, typename WT, bool ADD>
+int launch_rms(const void *x, const void *res, const void *w, float eps, void *y, void *out,
+               int64_t rows, int64_t hidden, hipStream_t st) {
+  const int vec_ok = (hidden * sizeof(T)) % 16 == 0;  // else every element goes through the scalar path
+  const T *xp = static_cast<const T *>(x), *rp = static_cast<const T *>(res);
+  const WT *wp = static_cast<const WT *>(w);
+  T *yp = static_cast<T *>(y), *op = static_cast<T *>(out);
+  if (hidden <= 512) {
+    hipLaunchKernelGGL((rms_norm_kernel<T, WT, 64, ADD>), dim3(blocks_for(rows, kBlock / 64)),
+                       dim3(kBlock), 0, st, xp, rp, wp, eps, yp, op, rows, static_cast<int>(hidden), vec_ok);
+  } else {
+    hipLaunchKernelGGL((rms_norm_kernel<T, WT, kBlock, ADD>), dim3(static_cast<unsigned>(rows)),
+                       dim3(kBlock), 0, st, xp, rp, wp, eps, yp, op, rows, static_cast<int>(hidden), vec_ok);
+  }
+  return launch_status();
+}
+
+template <bool ADD>
+int dispatch_rms(const void *x, const void *res, const void *w, float eps, void *y, void *out,
+                 int dtype, int w_dtype, int64_t rows, int64_t hidden, hipStream_t st) {
+  if (!is_float_dtype(dtype) || (w && !is_float_dtype(w_dtype))) return AXHIP_UNSUPPORTED_TYPE;
+  if (rows < 0 || hidden <= 0 || hidden > (1 << 24)) return AXHIP_INVALID_ARGUMENT;
+  if (rows == 0) return AXHIP_OK;
+  if (!x || !out || (ADD && (!res || !y))) return AXHIP_INVALID_PTR;
+  // 16-byte row accesses need aligned bases and rows that start on 16-byte boundaries
+  const int64_t esz = dtype == AXHIP_FLOAT16 ? 2 : 4;
+  if (!aligned16(x) || !aligned16(out) || (ADD && (!aligned16(res) || !aligned16(y))) ||
+      (w && !aligned16(w)))
+    return AXHIP_INVALID_ARGUMENT;
+  (void)esz;
+  const bool wh = w && w_dtype == AXHIP_FLOAT16;
+  if (dtype == AXHIP_FLOAT16)
+    return wh ? launch_rms<__half, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st)
+              : launch_rms<__half, float, ADD>(x, res, w, eps, y, out, rows, hidden, st);
+  return wh ? launch_rms<float, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st)
+            : launch_rms<float, float, ADD>(x, res, w, eps, y, out, rows, hidden, st);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Flat elementwise kernels: 8 elements per thread, scalar tail.
+// ------------------------------------------------------------------------------------------------
+struct SiluMulOp {
+  static __device__ __forceinline__ float apply(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+};
+struct AddOp {
+  static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+
+template <typename T, typename OP>
+__global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
+                                                        const T *__restrict__ b,
+                                                        T *__restrict__ y, int64_t n) {
+  const int64_t nvec = n / 8;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
+    float fa[8], fb[8], fy[8];
+    Row8<T>::load(a + i * 8, fa);
+    Row8<T>::load(b + i * 8, fb);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) fy[j] = OP::apply(fa[j], fb[j]);
+    Row8<T>::store(y + i * 8, fy);
+  }
+  if (blockIdx.x == 0) {
+    for (int64_t i = nvec * 8 + threadIdx.x; i < n; i += kBlock)
+      stf(y + i, OP::apply(ldf(a + i), ldf(b + i)));
+  }
+}
+
+template <typename OP>
+int launch_binary(const void *a, const void *b, void *y, int dtype, int64_t n, hipStream_t st) {
+  if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (n < 0) return AXHIP_INVALID_ARGUMENT;
+  if (n == 0) return AXHIP_OK;
+  if (!a || !b || !y) return AXHIP_INVALID_PTR;
+  if (!aligned16(a) || !aligned16(b) || !aligned16(y)) return AXHIP_INVALID_ARGUMENT;
+  const int64_t nvec = n / 8;
+  unsigned grid = blocks_for(nvec > 0 ? nvec : 1, kBlock);
+  if (grid > 256u * 16u) grid = 256u * 16u;
+  if (dtype == AXHIP_FLOAT16)
+    hipLaunchKernelGGL((binary_kernel<__half, OP>), dim3(grid), dim3(kBlock), 0, st,
+                       static_cast<const __half *>(a), static_cast<const __half *>(b),
+                       static_cast<__half *>(y), n);
+  else
+    hipLaunchKernelGGL((binary_kernel<float, OP>), dim3(grid), dim3(kBlock), 0, st,
+                       static_cast<const float *>(a), static_cast<const float *>(b),
+                       static_cast<float *>(y), n);
+  return launch_status();
+}
+
+template <typename S, typename Dt>
+__global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ src,
+                                                      Dt *__restrict__ dst, int64_t n) {
+  const int64_t nvec = n / 8;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
+    float f[8];
+    Row8<S>::load(src + i * 8, f);
+    Row8<Dt>::store(dst + i * 8, f);
+  }
+  if (blockIdx.x == 0) {
+    for (int64_t i = nvec * 8 + threadIdx.x; i < n; i += kBlock) stf(dst + i, ldf(src + i));
+  }
+}
+
+// Plain 16-byte copy / fill (graph-capturable replacements for memcpy / memset nodes).
+__global__ __launch_bounds__(kBlock) void copy_bytes_kernel(const uint8_t *__restrict__ src,
+                                                            uint8_t *__restrict__ dst, int64_t n,
+                                                            int vec_ok) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (vec_ok) {
+    const int64_t nvec = n / 16;
+    for (int64_t i = t; i < nvec; i += stride) st16(dst + i * 16, ld16(src + i * 16));
+    for (int64_t i = nvec * 16 + t; i < n; i += stride) dst[i] = src[i];
+  } else {
+    for (int64_t i = t; i < n; i += stride) dst[i] = src[i];
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_kernel(uint8_t *__restrict__ dst, int64_t n,
+                                                           int64_t head) {
+  // `head` unaligned leading bytes, then 16-byte stores, then the tail
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (t < head) dst[t] = 0;
+  uint8_t *body = dst + head;
+  const int64_t nb = n - head, nvec = nb / 16;
+  Vec16 z;
+  z.w[0] = z.w[1] = z.w[2] = z.w[3] = 0u;
+  for (int64_t i = t; i < nvec; i += stride) st16(body + i * 16, z);
+  for (int64_t i = nvec * 16 + t; i < nb; i += stride) body[i] = 0;
+}
+
+int launch_copy(const void *src, void *dst, int64_t n, hipStream_t st) {
+  if (n <= 0) return AXHIP_OK;
+  const int vec_ok = aligned16(src) && aligned16(dst);
+  unsigned grid = blocks_for((n + 15) / 16, kBlock);
+  if (grid > 256u * 16u) grid = 256u * 16u;
+  hipLaunchKernelGGL(copy_bytes_kernel, dim3(grid), dim3(kBlock), 0, st,
+                     static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), n, vec_ok);
+  return launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// Rotary embeddings.  One thread rotates 8 pairs (i, i + dim/2) of one (row, head).
+// ------------------------------------------------------------------------------------------------
+constexpr int kMaxHalf = 256;
+struct FreqTable {
+  float f[kMaxHalf];
+};
+
+enum RopeMode { kRopeTheta = 0, kRopeThd = 1, kRopeTable = 2 };
+
+struct RopeArgs {
+  const void *x;
+  void *out;
+  const int64_t *pos;     // [rows] (theta) or [3, rows] (thd)
+  const float *inv_freq;  // device [half] (thd)
+  const float *cos_t;     // device [rows, dim] (table)
+  const float *sin_t;
+  int64_t rows;
+  int heads, dim, h_lim, w_lim;
+};
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kBlock) void rope_kernel(RopeArgs a, FreqTable ft) {
+  const int half = a.dim / 2;
+  const int chunks = (half + 7) / 8;  // 8-pair chunks per (row, head)
+  const int64_t total = a.rows * a.heads * chunks;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (t >= total) return;
+  const int ch = static_cast<int>(t % chunks);
+  const int64_t rh = t / chunks;
+  const int64_t row = rh / a.heads;
+  const T *src = static_cast<const T *>(a.x) + rh * a.dim;
+  T *dst = static_cast<T *>(a.out) + rh * a.dim;
+  float pt = 0.f, ph = 0.f, pw = 0.f;
+  if (MODE == kRopeTheta) pt = static_cast<float>(a.pos[row]);
+  if (MODE == kRopeThd) {
+    pt = static_cast<float>(a.pos[row]);
+    ph = static_cast<float>(a.pos[a.rows + row]);
+    pw = static_cast<float>(a.pos[2 * a.rows + row]);
+  }
+  const int i0 = ch * 8;
+  const bool full = (i0 + 8 <= half) && (half % 8 == 0) && (sizeof(T) * a.dim % 16 == 0);
+  float lo[8], hi[8];
+  if (full) {
+    Row8<T>::load(src + i0, lo);
+    Row8<T>::load(src + i0 + half, hi);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      lo[j] = (i0 + j < half) ? ldf(src + i0 + j) : 0.f;
+      hi[j] = (i0 + j < half) ? ldf(src + i0 + j + half) : 0.f;
+    }
+  }
+  float olo[8], ohi[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int i = i0 + j;
+    float c_lo, s_lo, c_hi, s_hi;
+    if (MODE == kRopeTable) {
+      const bool in = i < half;
+      const float *cr = a.cos_t + row * a.dim, *sr = a.sin_t + row * a.dim;
+      c_lo = in ? cr[i] : 1.f;
+      s_lo = in ? sr[i] : 0.f;
+      c_hi = in ? cr[i + half] : 1.f;
+      s_hi = in ? sr[i + half] : 0.f;
+    } else {
+      float f, ang;
+      if (MODE == kRopeTheta) {
+        f = ft.f[i < kMaxHalf ? i : 0];
+        ang = pt * f;
+      } else {
+        f = i < half ? a.inv_freq[i] : 0.f;
+        ang = pt * f;
+        if (i % 3 == 1 && i < a.h_lim)
+          ang = ph * f;
+        else if (i % 3 == 2 && i < a.w_lim)
+          ang = pw * f;
+      }
+      sincosf(ang, &s_lo, &c_lo);
+      c_hi = c_lo;
+      s_hi = s_lo;
+    }
+    olo[j] = lo[j] * c_lo - hi[j] * s_lo;
+    ohi[j] = hi[j] * c_hi + lo[j] * s_hi;
+  }
+  if (full) {
+    Row8<T>::store(dst + i0, olo);
+    Row8<T>::store(dst + i0 + half, ohi);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (i0 + j < half) {
+        stf(dst + i0 + j, olo[j]);
+        stf(dst + i0 + j + half, ohi[j]);
+      }
+    }
+  }
+}
+
+template <int MODE>
+int launch_rope(const RopeArgs &a, const FreqTable &ft, int dtype, hipStream_t st) {
+  if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (a.dim % 2 != 0 || a.dim <= 0 || a.heads <= 0 || a.rows < 0) return AXHIP_INVALID_ARGUMENT;
+  if (a.rows == 0) return AXHIP_OK;
+  if (!a.x || !a.out) return AXHIP_INVALID_PTR;
+  if (!aligned16(a.x) || !aligned16(a.out)) return AXHIP_INVALID_ARGUMENT;
+  const int chunks = (a.dim / 2 + 7) / 8;
+  const unsigned grid = blocks_for(a.rows * a.heads * chunks, kBlock);
+  if (dtype == AXHIP_FLOAT16)
+    hipLaunchKernelGGL((rope_kernel<__half, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft);
+  else
+    hipLaunchKernelGGL((rope_kernel<float, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft);
+  return launch_status();
+}
+
+__global__ __launch_bounds__(kBlock) void mrope_cos_sin_kernel(const int64_t *__restrict__ pos,
+                                                               const float *__restrict__ inv_freq,
+                                                               int h_lim, int w_lim,
+                                                               float *__restrict__ cos_out,
+                                                               float *__restrict__ sin_out,
+                                                               int64_t rows, int half) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (t >= rows * half) return;
+  const int i = static_cast<int>(t % half);
+  const int64_t r = t / half;
+  const float f = inv_freq[i];
+  float ang = static_cast<float>(pos[r]) * f;
+  if (i % 3 == 1 && i < h_lim)
+    ang = static_cast<float>(pos[rows + r]) * f;
+  else if (i % 3 == 2 && i < w_lim)
+    ang = static_cast<float>(pos[2 * rows + r]) * f;
+  float s, c;
+  sincosf(ang, &s, &c);
+  float *cr = cos_out + r * 2 * half, *sr = sin_out + r * 2 * half;
+  cr[i] = c;
+  cr[i + half] = c;
+  sr[i] = s;
+  sr[i + half] = s;
+}
+
+// ------------------------------------------------------------------------------------------------
+// KV-cache append: cache[b, hk, pos[b], :] = new[b, hk, :] for K and V, 16 bytes per thread.
+// ------------------------------------------------------------------------------------------------
+template <typename P>
+__global__ __launch_bounds__(kBlock) void kv_append_kernel(const uint8_t *__restrict__ k_new,
+                                                           const uint8_t *__restrict__ v_new,
+                                                           uint8_t *__restrict__ k_cache,
+                                                           uint8_t *__restrict__ v_cache,
+                                                           const P *__restrict__ pos, int B, int Hkv,
+                                                           int Lmax, int row_bytes) {
+  const int vec_per_row = row_bytes / 16;
+  const int64_t total = static_cast<int64_t>(B) * Hkv * vec_per_row;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (t >= total) return;
+  const int vi = static_cast<int>(t % vec_per_row);
+  const int64_t bh = t / vec_per_row;
+  const int b = static_cast<int>(bh / Hkv);
+  const int64_t p = static_cast<int64_t>(pos[b]);
+  if (p < 0 || p >= Lmax) return;
+  const int64_t src = bh * row_bytes + vi * 16;
+  const int64_t dst = (bh * Lmax + p) * row_bytes + vi * 16;
+  st16(k_cache + dst, ld16(k_new + src));
+  st16(v_cache + dst, ld16(v_new + src));
+}
+
+// ------------------------------------------------------------------------------------------------
+// Embedding gather and argmax.
+// ------------------------------------------------------------------------------------------------
+template <typename I>
+__global__ __launch_bounds__(kBlock) void embedding_kernel(const I *__restrict__ ids,
+                                                           const uint8_t *__restrict__ table,
+                                                           uint8_t *__restrict__ out, int64_t vocab,
+                                                           int64_t row_bytes, int vec_ok) {
+  const int64_t i = blockIdx.x;
+  int64_t id = static_cast<int64_t>(ids[i]);
+  const bool valid = id >= 0 && id < vocab;  // out-of-range ids give a zero row instead of a fault
+  const uint8_t *src = table + (valid ? id : 0) * row_bytes;
+  uint8_t *dst = out + i * row_bytes;
+  if (vec_ok) {
+    Vec16 z;
+    z.w[0] = z.w[1] = z.w[2] = z.w[3] = 0u;
+    for (int64_t o = threadIdx.x * 16; o < row_bytes; o += kBlock * 16)
+      st16(dst + o, valid ? ld16(src + o) : z);
+  } else {
+    for (int64_t o = threadIdx.x; o < row_bytes; o += kBlock) dst[o] = valid ? src[o] : 0;
+  }
+}
+
+constexpr int kArgmaxBlock = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(kArgmaxBlock) void argmax_kernel(const T *__restrict__ x,
+                                                              int64_t *__restrict__ out,
+                                                              int64_t cols) {
+  __shared__ float s_val[kArgmaxBlock / 64];
+  __shared__ int64_t s_idx[kArgmaxBlock / 64];
+  const T *row = x + static_cast<int64_t>(blockIdx.x) * cols;
+  float best = -INFINITY;
+  int64_t bi = INT64_MAX;
+  // strided scan keeps indices increasing per thread, so `>` keeps the first maximum
+  for (int64_t c = threadIdx.x; c < cols; c += kArgmaxBlock) {
+    const float v = ldf(row + c);
+    if (v > best || bi == INT64_MAX) {
+      best = v;
+      bi = c;
+    }
+  }
+  // wavefront then block reduction; ties go to the smaller index
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int64_t oi = __shfl_xor(bi, off, 64);
+    if (oi != INT64_MAX && (bi == INT64_MAX || ov > best || (ov == best && oi < bi))) {
+      best = ov;
+      bi = oi;
+    }
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    s_val[wave] = best;
+    s_idx[wave] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kArgmaxBlock / 64; ++w) {
+      const float ov = s_val[w];
+      const int64_t oi = s_idx[w];
+      if (oi != INT64_MAX && (bi == INT64_MAX || ov > best || (ov == best && oi < bi))) {
+        best = ov;
+        bi = oi;
+      }
+    }
+    out[blockIdx.x] = bi == INT64_MAX ? 0 : bi;
+  }
+}
+
+}  // namespace
+}  // namespace axhip
+
+using namespace axhip;
+
+extern "C" {
+
+AXHIP_API int axhip_add_rms_norm(const void *x, const void *residual, const void *weight, float eps,
+                                 void *y, void *out, int dtype, int w_dtype, int64_t rows,
+                                 int64_t hidden, axhip_stream stream) {
+  if (!weight) return AXHIP_INVALID_PTR;
+  return dispatch_rms<true>(x, residual, weight, eps, y, out, dtype, w_dtype, rows, hidden,
+                            as_stream(stream));
+}
+
+AXHIP_API int axhip_rms_norm(const void *x, const void *weight, float eps, void *out, int dtype,
+                             int w_dtype, int64_t rows, int64_t cols, axhip_stream stream) {
+  return dispatch_rms<false>(x, nullptr, weight, eps, nullptr, out, dtype, w_dtype, rows, cols,
+                             as_stream(stream));
+}
+
+AXHIP_API int axhip_silu_mul(const void *gate, const void *up, void *y, int dtype, int64_t n,
+                             axhip_stream stream) {
+  return launch_binary<SiluMulOp>(gate, up, y, dtype, n, as_stream(stream));
+}
+
+AXHIP_API int axhip_add(const void *a, const void *b, void *out, int dtype, int64_t n,
+                        axhip_stream stream) {
+  return launch_binary<AddOp>(a, b, out, dtype, n, as_stream(stream));
+}
+
+AXHIP_API int axhip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n,
+                         axhip_stream stream) {
+  if (!is_float_dtype(src_dtype) || !is_float_dtype(dst_dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (n < 0) return AXHIP_INVALID_ARGUMENT;
+  if (n == 0) return AXHIP_OK;
+  if (!src || !dst) return AXHIP_INVALID_PTR;
+  if (!aligned16(src) || !aligned16(dst)) return AXHIP_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  if (src_dtype == dst_dtype)
+    return launch_copy(src, dst, n * (src_dtype == AXHIP_FLOAT16 ? 2 : 4), st);
+  unsigned grid = blocks_for(n / 8 > 0 ? n / 8 : 1, kBlock);
+  if (grid > 256u * 16u) grid = 256u * 16u;
+  if (src_dtype == AXHIP_FLOAT32)
+    hipLaunchKernelGGL((cast_kernel<float, __half>), dim3(grid), dim3(kBlock), 0, st,
+                       static_cast<const float *>(src), static_cast<__half *>(dst), n);
+  else
+    hipLaunchKernelGGL((cast_kernel<__half, float>), dim3(grid), dim3(kBlock), 0, st,
+                       static_cast<const __half *>(src), static_cast<float *>(dst), n);
+  return launch_status();
+}
+
+AXHIP_API int axhip_rope(const void *x, const int64_t *pos, float theta, void *out, int dtype,
+                         int64_t rows, int64_t heads, int64_t dim, axhip_stream stream) {
+  if (dim <= 0 || dim % 2 != 0 || dim / 2 > kMaxHalf) return AXHIP_INVALID_ARGUMENT;
+  if (!pos && rows > 0) return AXHIP_INVALID_PTR;
+  FreqTable ft;
+  // same expression, in fp32 on the host, as the CPU operator evaluates per element
+  for (int64_t i = 0; i < dim / 2; ++i)
+    ft.f[i] = std::pow(theta, -2.0f * static_cast<float>(i) / static_cast<float>(dim));
+  RopeArgs a{x, out, pos, nullptr, nullptr, nullptr, rows, static_cast<int>(heads),
+             static_cast<int>(dim), 0, 0};
+  return launch_rope<kRopeTheta>(a, ft, dtype, as_stream(stream));
+}
+
+AXHIP_API int axhip_rope_thd(const void *x, const int64_t *pos, const float *inv_freq, int t_sec,
+                             int h_sec, int w_sec, void *out, int dtype, int64_t rows,
+                             int64_t heads, int64_t dim, axhip_stream stream) {
+  (void)t_sec;
+  if ((!pos || !inv_freq) && rows > 0) return AXHIP_INVALID_PTR;
+  RopeArgs a{x, out, pos, inv_freq, nullptr, nullptr, rows, static_cast<int>(heads),
+             static_cast<int>(dim), h_sec * 3, w_sec * 3};
+  FreqTable ft{};
+  return launch_rope<kRopeThd>(a, ft, dtype, as_stream(stream));
+}
+
+AXHIP_API int axhip_rope_with_cos_sin(const void *x, const float *cos_t, const float *sin_t,
+                                      void *out, int dtype, int64_t rows, int64_t heads,
+                                      int64_t dim, axhip_stream stream) {
+  if ((!cos_t || !sin_t) && rows > 0) return AXHIP_INVALID_PTR;
+  RopeArgs a{x, out, nullptr, nullptr, cos_t, sin_t, rows, static_cast<int>(heads),
+             static_cast<int>(dim), 0, 0};
+  FreqTable ft{};
+  return launch_rope<kRopeTable>(a, ft, dtype, as_stream(stream));
+}
+
+AXHIP_API int axhip_mrope_cos_sin(const int64_t *pos, const float *inv_freq, int h_sec, int w_sec,
+                                  float *cos_out, float *sin_out, int64_t rows, int64_t half,
+                                  axhip_stream stream) {
+  if (half <= 0 || rows < 0) return AXHIP_INVALID_ARGUMENT;
+  if (rows == 0) return AXHIP_OK;
+  if (!pos || !inv_freq || !cos_out || !sin_out) return AXHIP_INVALID_PTR;
+  hipLaunchKernelGGL(mrope_cos_sin_kernel, dim3(blocks_for(rows * half, kBlock)), dim3(kBlock), 0,
+                     as_stream(stream), pos, inv_freq, h_sec * 3, w_sec * 3, cos_out, sin_out, rows,
+                     static_cast<int>(half));
+  return launch_status();
+}
+
+AXHIP_API int axhip_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache,
+                              const void *pos, int pos_dtype, int elem_bytes, int B, int Hkv,
+                              int Lmax, int D, axhip_stream stream) {
+  if (pos_dtype != AXHIP_INT32 && pos_dtype != AXHIP_INT64) return AXHIP_UNSUPPORTED_TYPE;
+  if (elem_bytes != 2 && elem_bytes != 4) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || Hkv <= 0 || Lmax <= 0 || D <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (B == 0) return AXHIP_OK;
+  if (!k_new || !v_new || !k_cache || !v_cache || !pos) return AXHIP_INVALID_PTR;
+  const int row_bytes = D * elem_bytes;
+  if (row_bytes % 16 != 0 || !aligned16(k_new) || !aligned16(v_new) || !aligned16(k_cache) ||
+      !aligned16(v_cache))
+    return AXHIP_INVALID_ARGUMENT;
+  const int64_t total = static_cast<int64_t>(B) * Hkv * (row_bytes / 16);
+  const dim3 grid(blocks_for(total, kBlock));
+  hipStream_t st = as_stream(stream);
+  const uint8_t *kn = static_cast<const uint8_t *>(k_new), *vn = static_cast<const uint8_t *>(v_new);
+  uint8_t *kc = static_cast<uint8_t *>(k_cache), *vc = static_cast<uint8_t *>(v_cache);
+  if (pos_dtype == AXHIP_INT32)
+    hipLaunchKernelGGL((kv_append_kernel<int32_t>), grid, dim3(kBlock), 0, st, kn, vn, kc, vc,
+                       static_cast<const int32_t *>(pos), B, Hkv, Lmax, row_bytes);
+  else
+    hipLaunchKernelGGL((kv_append_kernel<int64_t>), grid, dim3(kBlock), 0, st, kn, vn, kc, vc,
+                       static_cast<const int64_t *>(pos), B, Hkv, Lmax, row_bytes);
+  return launch_status();
+}
+
+AXHIP_API int axhip_concat(const void *a, const void *b, void *out, int64_t outer, int64_t a_bytes,
+                           int64_t b_bytes, axhip_stream stream) {
+  if (outer < 0 || a_bytes < 0 || b_bytes < 0) return AXHIP_INVALID_ARGUMENT;
+  if (outer == 0 || a_bytes + b_bytes == 0) return AXHIP_OK;
+  if ((a_bytes && !a) || (b_bytes && !b) || !out) return AXHIP_INVALID_PTR;
+  hipStream_t st = as_stream(stream);
+  uint8_t *dst = static_cast<uint8_t *>(out);
+  for (int64_t o = 0; o < outer; ++o) {
+    int rc = launch_copy(static_cast<const uint8_t *>(a) + o * a_bytes, dst, a_bytes, st);
+    if (rc != AXHIP_OK) return rc;
+    dst += a_bytes;
+    rc = launch_copy(static_cast<const uint8_t *>(b) + o * b_bytes, dst, b_bytes, st);
+    if (rc != AXHIP_OK) return rc;
+    dst += b_bytes;
+  }
+  return AXHIP_OK;
+}
+
+AXHIP_API int axhip_embedding(const void *ids, int ids_dtype, const void *table, void *out,
+                              int dtype, int64_t n_ids, int64_t vocab, int64_t hidden,
+                              axhip_stream stream) {
+  if (ids_dtype != AXHIP_INT32 && ids_dtype != AXHIP_INT64) return AXHIP_UNSUPPORTED_TYPE;
+  if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (n_ids < 0 || vocab <= 0 || hidden <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (n_ids == 0) return AXHIP_OK;
+  if (!ids || !table || !out) return AXHIP_INVALID_PTR;
+  const int64_t row_bytes = hidden * (dtype == AXHIP_FLOAT16 ? 2 : 4);
+  const int vec_ok = aligned16(table) && aligned16(out) && row_bytes % 16 == 0;
+  const dim3 grid(static_cast<unsigned>(n_ids));
+  hipStream_t st = as_stream(stream);
+  if (ids_dtype == AXHIP_INT64)
+    hipLaunchKernelGGL((embedding_kernel<int64_t>), grid, dim3(kBlock), 0, st,
+                       static_cast<const int64_t *>(ids), static_cast<const uint8_t *>(table),
+                       static_cast<uint8_t *>(out), vocab, row_bytes, vec_ok);
+  else
+    hipLaunchKernelGGL((embedding_kernel<int32_t>), grid, dim3(kBlock), 0, st,
+                       static_cast<const int32_t *>(ids), static_cast<const uint8_t *>(table),
+                       static_cast<uint8_t *>(out), vocab, row_bytes, vec_ok);
+  return launch_status();
+}
+
+AXHIP_API int axhip_argmax(const void *x, int64_t *out, int dtype, int64_t rows, int64_t cols,
+                           axhip_stream stream) {
+  if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (rows < 0 || cols <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (rows == 0) return AXHIP_OK;
+  if (!x || !out) return AXHIP_INVALID_PTR;
+  hipStream_t st = as_stream(stream);
+  const dim3 grid(static_cast<unsigned>(rows));
+  if (dtype == AXHIP_FLOAT16)
+    hipLaunchKernelGGL((argmax_kernel<__half>), grid, dim3(kArgmaxBlock), 0, st,
+                       static_cast<const __half *>(x), out, cols);
+  else
+    hipLaunchKernelGGL((argmax_kernel<float>), grid, dim3(kArgmaxBlock), 0, st,
+                       static_cast<const float *>(x), out, cols);
+  return launch_status();
+}
+
+// Device-to-device copy and zero fill as kernels (used by the runtime; capturable).
+int axhip_internal_copy(const void *src, void *dst, int64_t n, hipStream_t st) {
+  return launch_copy(src, dst, n, st);
+}
+int axhip_internal_fill_zero(void *dst, int64_t n, hipStream_t st) {
+  if (n <= 0) return AXHIP_OK;
+  const int64_t mis = reinterpret_cast<uintptr_t>(dst) & 15;
+  int64_t head = mis ? 16 - mis : 0;
+  if (head > n) head = n;
+  unsigned grid = blocks_for((n + 15) / 16, kBlock);
+  if (grid > 256u * 16u) grid = 256u * 16u;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(kBlock), 0, st, static_cast<uint8_t *>(dst),
+                     n, head);
+  return launch_status();
+}
+
+}  // extern "C"

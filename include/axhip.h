@@ -1,0 +1,301 @@
+/*
+ * axhip.h — C ABI of libaxhip.so: the LLM decode path of Axono as hand-written gfx950 kernels,
+ * plus the small device runtime (caching allocator, current stream, hipGraph capture) that path
+ * needs.  Plain pointers and sizes only; every operator takes the HIP stream it must run on.
+ *
+ * Conventions (they mirror the reference's operator layer, whose functions have the form
+ * `Status Op(const Context&, const Tensor&..., Tensor& result)`, include/axono/ops/cuda/ headers):
+ *   - every function returns an `axhip_status`; its values are the reference's `core::Status`
+ *     (include/axono/core/types.h:54-64), so a binding can forward the int unchanged;
+ *   - `dtype` arguments use the reference's `core::DataType` numbering (types.h:18-27);
+ *   - buffers are caller-owned device memory, contiguous row-major unless strides are passed;
+ *   - nothing synchronises: work is enqueued on `stream` (NULL = the legacy default stream) and
+ *     is safe to record into a hipGraph (no allocation, no host<->device copy, no memset node).
+ */
+#ifndef AXHIP_H_
+#define AXHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AXHIP_API __attribute__((visibility("default")))
+
+/* core::Status, include/axono/core/types.h:54-64 */
+typedef enum {
+  AXHIP_OK = 0,
+  AXHIP_INVALID_ARGUMENT = 1,
+  AXHIP_OUT_OF_MEMORY = 2,
+  AXHIP_UNSUPPORTED_TYPE = 3,
+  AXHIP_SHAPE_MISMATCH = 4,
+  AXHIP_INTERNAL_ERROR = 5,
+  AXHIP_DEVICE_ERROR = 6,
+  AXHIP_INVALID_PTR = 7,
+  AXHIP_DEVICE_MISMATCH = 8
+} axhip_status;
+
+/* core::DataType, include/axono/core/types.h:18-27 */
+typedef enum {
+  AXHIP_INT8 = 0,
+  AXHIP_INT16 = 1,
+  AXHIP_INT32 = 2,
+  AXHIP_INT64 = 3,
+  AXHIP_FLOAT16 = 4,
+  AXHIP_FLOAT32 = 5,
+  AXHIP_FLOAT64 = 6,
+  AXHIP_BOOLEAN = 7
+} axhip_dtype;
+
+typedef void *axhip_stream; /* a hipStream_t */
+
+/* ============================================================================================
+ * Device runtime
+ * ========================================================================================== */
+
+/* Library version string, "0.2.0-hip" (the reference module reports "0.2.0",
+ * axono/python/src/nanobind_module.cpp:1327). */
+AXHIP_API const char *axhip_version(void);
+
+/* Number of HIP devices; the `hip:<id>` device of the Python surface maps to these ids.
+ * Replaces cuda_available(), nanobind_module.cpp:1211-1217. */
+AXHIP_API int axhip_device_count(int *count);
+AXHIP_API int axhip_set_device(int device_id);
+/* Device name and whether it is the gfx950 target the kernels are built for. */
+AXHIP_API int axhip_device_info(int device_id, char *name, size_t name_len, int *is_gfx950,
+                                size_t *total_bytes, int *compute_units);
+
+/* Caching allocator.  Replaces cuda::detail::CudaAllocateStorage / ReturnToCache,
+ * src/core/cuda/detail.cu:93-289.  Exact-size free lists; released blocks stay cached up to the
+ * budget (default: half of the device's memory, where the reference used 2 GiB) and are evicted
+ * oldest first.  `zero` != 0 zero-fills the block on the current stream, as the reference does
+ * for every tensor it creates (detail.cu:221-222,246); kernels that overwrite their whole output
+ * pass 0 and skip that write.  While a capture-pool recording or a graph capture is active the
+ * call follows the capture pool instead (see axhip_capture_pool_*). */
+AXHIP_API int axhip_alloc(size_t bytes, int zero, void **out);
+AXHIP_API int axhip_free(void *ptr);
+/* cached_bytes() / set_cache_budget(bytes), nanobind_module.cpp:398-400 */
+AXHIP_API size_t axhip_cached_bytes(void);
+AXHIP_API int axhip_set_cache_budget(size_t bytes);
+AXHIP_API size_t axhip_cache_budget(void);
+/* Frees every cached block (ClearDeviceCache, detail.cu:106-122). */
+AXHIP_API int axhip_empty_cache(void);
+/* Bytes currently handed out (diagnostic; no reference counterpart). */
+AXHIP_API size_t axhip_allocated_bytes(void);
+
+/* Copies.  Host<->device copies are synchronous with respect to the current stream, like the
+ * reference's blocking cudaMemcpy (src/core/cuda/detail.cu:314-350, tensor.cpp:186-215), and are
+ * refused with AXHIP_INVALID_ARGUMENT while the calling thread is capturing a graph.
+ * Device-to-device copies and fills are kernels on the current stream (capturable). */
+AXHIP_API int axhip_memcpy_h2d(void *dst, const void *src, size_t bytes);
+AXHIP_API int axhip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+AXHIP_API int axhip_memcpy_d2d(void *dst, const void *src, size_t bytes);
+AXHIP_API int axhip_fill_zero(void *dst, size_t bytes);
+
+/* The stream operators should be given: the calling thread's capture stream while it captures,
+ * else the legacy default stream.  Replaces cuda::AxonoCurrentStream, src/core/cuda/graph.cu:58-60. */
+AXHIP_API axhip_stream axhip_current_stream(void);
+/* 1 while the calling thread is between axhip_graph_begin_capture and end/abort
+ * (cuda::IsCapturing, include/axono/core/cuda/capture.h:19-33). */
+AXHIP_API int axhip_is_capturing(void);
+/* Waits for the current stream (no-op error while capturing). */
+AXHIP_API int axhip_synchronize(void);
+
+/* hipGraph capture.  Replaces BeginGraphCapture / EndGraphCapture / AbortGraphCapture and
+ * CudaGraphExec::{Finalize,Replay,Sync,Reset}, src/core/cuda/graph.cu:79-215, and the binding's
+ * CUDAGraph class, nanobind_module.cpp:1226-1324.
+ *   begin    creates a non-blocking capture stream, starts a thread-local capture on it and
+ *            makes it the thread's current stream;
+ *   end      ends the capture, rejects an empty graph (AXHIP_INVALID_ARGUMENT), instantiates it
+ *            and returns the executable graph and its node count;
+ *   abort    ends and discards a capture after a failure inside the captured body;
+ *   launch   enqueues one replay on the graph's stream (no wait); `sync` waits for it.
+ *            The reference's replay() is launch + sync. */
+typedef void *axhip_graph; /* opaque executable graph */
+AXHIP_API int axhip_graph_begin_capture(axhip_stream *stream_out);
+AXHIP_API int axhip_graph_end_capture(axhip_stream stream, axhip_graph *graph_out,
+                                      size_t *num_nodes_out);
+AXHIP_API int axhip_graph_abort_capture(axhip_stream stream);
+AXHIP_API int axhip_graph_launch(axhip_graph graph);
+AXHIP_API int axhip_graph_sync(axhip_graph graph);
+AXHIP_API int axhip_graph_destroy(axhip_graph graph);
+
+/* Capture pool: address stability between the warm-up run and the captured run of the same
+ * body.  Replaces ResetCapturePool / SetCapturePoolRecording / the size->ptr FIFO,
+ * src/core/cuda/capture_pool.cu:21-51 and detail.cu:193-199,259-264.  While recording, every
+ * axhip_alloc is remembered (size -> pointer, in order); while capturing, an axhip_alloc of the
+ * same size pops the remembered pointer instead of allocating, so the graph sees the warm-up's
+ * addresses.  Blocks remembered by the pool are owned by it until axhip_capture_pool_reset. */
+AXHIP_API int axhip_capture_pool_reset(void);
+AXHIP_API int axhip_capture_pool_set_recording(int on);
+
+/* Events on the current stream, for timing kernels (no reference counterpart; the reference
+ * times with the host clock). */
+typedef void *axhip_event;
+AXHIP_API int axhip_event_create(axhip_event *out);
+AXHIP_API int axhip_event_record(axhip_event ev, axhip_stream stream);
+AXHIP_API int axhip_event_elapsed_ms(axhip_event start, axhip_event stop, float *ms_out);
+AXHIP_API int axhip_event_destroy(axhip_event ev);
+
+/* ============================================================================================
+ * Decode attention
+ * ========================================================================================== */
+
+/* Split-K flash-decoding for one query token per sequence, grouped-query heads.
+ * Replaces ops::cuda::GqaDecodeAttention (include/axono/ops/cuda/gqa.h:16-20,
+ * src/ops/cuda/gqa.cu:139-182: GqaDecodeSplitKernel :31-92, GqaDecodeMergeKernel :95-129) and its
+ * short-context fallback to ScaledDotProductAttention(is_causal=false) (gqa.cu:150-151).
+ * Result per sequence b and head h:  softmax(q[b,h] . K[b, h/group, 0:len_b]^T / sqrt(D)) V[...].
+ *
+ *   q, out      [B, Hq, D], dtype `dtype` (FLOAT16 or FLOAT32), contiguous
+ *   k, v        element (b, hk, s, :) at  base + b*stride_b + hk*stride_h + s*stride_s  (strides in
+ *               elements, rows of D contiguous elements).  The batched cache [B,Hkv,Lmax,D] has
+ *               stride_b = Hkv*Lmax*D, stride_h = Lmax*D, stride_s = D; the reference's per-call
+ *               layout (L,Hkv,D) is B = 1, stride_h = D, stride_s = Hkv*D.
+ *   seq_lens    device int32[B] with each sequence's current length, or NULL: every sequence has
+ *               `max_len` keys.  Read by the kernels, so a captured graph follows lengths that
+ *               change between replays.  A length of 0 yields zeros.
+ *   max_len     upper bound of every length (sizes the split grid; lengths above it are clamped)
+ *   workspace   device scratch of at least axhip_gqa_decode_workspace_bytes(...) bytes
+ *   D in {64, 128, 256}; Hq % Hkv == 0.  fp32 accumulation throughout; fp16 data is widened
+ *   exactly and only the final store rounds. */
+AXHIP_API size_t axhip_gqa_decode_workspace_bytes(int B, int Hq, int Hkv, int D, int max_len);
+AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
+                               const int32_t *seq_lens, void *out, void *workspace,
+                               size_t workspace_bytes, int dtype, int B, int Hq, int Hkv, int D,
+                               int max_len, int64_t stride_b, int64_t stride_h, int64_t stride_s,
+                               axhip_stream stream);
+
+/* The split plan the launcher uses for these sizes (it depends on host-side sizes only), and a
+ * measurement hook that overrides the heuristics: target_workgroups = resident workgroups to aim
+ * for, force_splits > 0 fixes the split count; 0 restores a default.  No reference counterpart
+ * (the reference hard-codes min(256, ceil(L/64)), gqa.cu:158-160). */
+AXHIP_API void axhip_gqa_decode_plan(int B, int Hq, int Hkv, int max_len, int *n_splits, int *chunk);
+AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
+
+/* General attention for prefill and short contexts: q [Sq,Hq,D], k/v [Skv,Hkv,D] contiguous,
+ * optional causal mask with the reference's rule (keys 0..t visible when Skv >= t+1).
+ * Replaces ops::cuda::ScaledDotProductAttention, src/ops/cuda/sequence.cu:105-163,451-472.
+ * Any D up to 256; not tuned (it fills the cache before the timed decode loop). */
+AXHIP_API int axhip_sdpa(const void *q, const void *k, const void *v, void *out, int dtype,
+                         int Sq, int Hq, int Hkv, int D, int Skv, int is_causal,
+                         axhip_stream stream);
+
+/* ============================================================================================
+ * KV-cache append
+ * ========================================================================================== */
+
+/* cache[b, hk, pos[b], :] = new[b, hk, :] for K and V in one launch; a byte copy (bit exact).
+ * Replaces DynamicKVCache.update's concat-append (axono/python/axono/nn/kv_cache.py:96-102 ->
+ * ops::cuda::Concat axis 0, src/ops/cuda/sequence.cu:474-521), which re-copies the whole cache
+ * every step.  k_new, v_new [B,Hkv,D]; caches [B,Hkv,Lmax,D]; pos device int32[B] or int64[B]
+ * (`pos_dtype`); a position outside [0,Lmax) is skipped.  `elem_bytes` is 2 or 4. */
+AXHIP_API int axhip_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache,
+                              const void *pos, int pos_dtype, int elem_bytes, int B, int Hkv,
+                              int Lmax, int D, axhip_stream stream);
+
+/* out = [a ; b] along an axis: `outer` blocks of a_bytes then b_bytes each (axis 0: outer = 1).
+ * Replaces ops::cuda::Concat, src/ops/cuda/sequence.cu:474-521. */
+AXHIP_API int axhip_concat(const void *a, const void *b, void *out, int64_t outer, int64_t a_bytes,
+                           int64_t b_bytes, axhip_stream stream);
+
+/* ============================================================================================
+ * Fused and row-wise operators (dtype FLOAT16 or FLOAT32; arithmetic in fp32)
+ * ========================================================================================== */
+
+/* y = x + residual ; out = y * rsqrt(mean(y^2) + eps) * weight.  Two results, like the reference.
+ * Replaces ops::cuda::AddRmsNorm, src/ops/cuda/fused.cu:38-72,91-110.  weight dtype may differ
+ * from the activation dtype (`w_dtype`). */
+AXHIP_API int axhip_add_rms_norm(const void *x, const void *residual, const void *weight, float eps,
+                                 void *y, void *out, int dtype, int w_dtype, int64_t rows,
+                                 int64_t hidden, axhip_stream stream);
+
+/* y = gate / (1 + exp(-gate)) * up.  Replaces ops::cuda::SiluMul, src/ops/cuda/fused.cu:28-34,76-89. */
+AXHIP_API int axhip_silu_mul(const void *gate, const void *up, void *y, int dtype, int64_t n,
+                             axhip_stream stream);
+
+/* out = x * rsqrt(mean(x^2) + eps) [* weight] over the last dim; weight may be NULL.
+ * Replaces ops::cuda::RmsNorm, src/ops/cuda/llm.cu:140-158. */
+AXHIP_API int axhip_rms_norm(const void *x, const void *weight, float eps, void *out, int dtype,
+                             int w_dtype, int64_t rows, int64_t cols, axhip_stream stream);
+
+/* out = a + b.  Replaces ops::cuda::Add for equal shapes, src/ops/cuda/add.cu:17-24. */
+AXHIP_API int axhip_add(const void *a, const void *b, void *out, int dtype, int64_t n,
+                        axhip_stream stream);
+
+/* fp16 <-> fp32 conversion, IEEE round-to-nearest-even.  Replaces Half2FloatKernel /
+ * Float2HalfKernel, src/core/cuda/tensor/kernel.cu:175-223 (Tensor::CastTo on device). */
+AXHIP_API int axhip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n,
+                         axhip_stream stream);
+
+/* ============================================================================================
+ * Rotary position embeddings.  x, out [rows, heads, dim]; rotate-half pairing (i, i + dim/2).
+ * ========================================================================================== */
+
+/* freq_i = powf(theta, -2 i / dim) evaluated on the host in fp32 exactly as the reference's CPU
+ * operator does, angle = float(pos) * freq_i in fp32, accurate sinf/cosf.  pos device int64[rows].
+ * Replaces ops::cuda::Rope, src/ops/cuda/sequence.cu:84-101,318-342 (CPU: sequence.cpp:54-93).
+ * dim <= 512. */
+AXHIP_API int axhip_rope(const void *x, const int64_t *pos, float theta, void *out, int dtype,
+                         int64_t rows, int64_t heads, int64_t dim, axhip_stream stream);
+
+/* M-RoPE with interleaved T/H/W channels: pos device int64[3, rows], inv_freq device fp32[dim/2];
+ * channel i uses H if i%3==1 && i<3*h_sec, W if i%3==2 && i<3*w_sec, else T (t_sec is unused, as
+ * in the reference).  Replaces ops::cuda::RopeThd, src/ops/cuda/sequence.cu:186-212,421-449. */
+AXHIP_API int axhip_rope_thd(const void *x, const int64_t *pos, const float *inv_freq, int t_sec,
+                             int h_sec, int w_sec, void *out, int dtype, int64_t rows,
+                             int64_t heads, int64_t dim, axhip_stream stream);
+
+/* cos/sin tables [rows, 2*half] fp32 (both halves equal) for M-RoPE.
+ * Replaces ops::cuda::MropeCosSin, src/ops/cuda/sequence.cu:372-419. */
+AXHIP_API int axhip_mrope_cos_sin(const int64_t *pos, const float *inv_freq, int h_sec, int w_sec,
+                                  float *cos_out, float *sin_out, int64_t rows, int64_t half,
+                                  axhip_stream stream);
+
+/* Rotation by given fp32 tables cos, sin [rows, dim]; the second element of a pair uses the
+ * second half of the table.  Replaces ops::cuda::RopeWithCosSin, src/ops/cuda/sequence.cu:166-183,344-369. */
+AXHIP_API int axhip_rope_with_cos_sin(const void *x, const float *cos_t, const float *sin_t,
+                                      void *out, int dtype, int64_t rows, int64_t heads,
+                                      int64_t dim, axhip_stream stream);
+
+/* ============================================================================================
+ * fp16 Linear (cast_linear_fp16)
+ * ========================================================================================== */
+
+/* out[M,N] = x[M,K] . W[N,K]^T (+ bias[N]); W and bias FLOAT16, fp32 accumulation on MFMA.
+ * x is FLOAT32 (converted to fp16 round-to-nearest-even first, as the reference does,
+ * src/ops/cuda/linear.cu:105-110) or FLOAT16; out is FLOAT32 (the reference's contract,
+ * nanobind_module.cpp:760-762) or FLOAT16.  bias may be NULL.
+ * Replaces the fp16 branch of ops::cuda::Linear, src/ops/cuda/linear.cu:105-176 (cast kernel +
+ * bias/zero fill + cublasGemmEx).  K % 8 == 0.  `workspace` holds split-K partial sums for skinny
+ * M: at least axhip_linear_f16_workspace_bytes(M,K,N) bytes (may be 0, then pass NULL). */
+AXHIP_API size_t axhip_linear_f16_workspace_bytes(int64_t M, int64_t K, int64_t N);
+/* Measurement hook for the skinny-M kernel's plan (0 restores a default): wavefronts to aim for,
+ * 16-row groups of W per wavefront (1, 2 or 4), K splits across workgroups.  No reference
+ * counterpart (the reference leaves the choice to cuBLAS). */
+AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_ks_outer);
+AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const void *bias,
+                               void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
+                               void *workspace, size_t workspace_bytes, axhip_stream stream);
+
+/* ============================================================================================
+ * Index operators of the decode step
+ * ========================================================================================== */
+
+/* out[i, :] = table[ids[i], :]; ids device int64 (or int32 via `ids_dtype`); table/out `dtype`.
+ * Replaces ops::cuda::Embedding, src/ops/cuda/sequence.cu:75-81,296-316. */
+AXHIP_API int axhip_embedding(const void *ids, int ids_dtype, const void *table, void *out,
+                              int dtype, int64_t n_ids, int64_t vocab, int64_t hidden,
+                              axhip_stream stream);
+
+/* out[r] = index of the first maximum of x[r, :]; out device int64[rows].
+ * Replaces ops::cuda::ArgmaxLastDim, src/ops/cuda/sequence.cu:262-292. */
+AXHIP_API int axhip_argmax(const void *x, int64_t *out, int dtype, int64_t rows, int64_t cols,
+                           axhip_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXHIP_H_ */

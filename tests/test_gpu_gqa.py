@@ -1,0 +1,142 @@
+"""GQA decode attention on the GPU against the CPU oracle (through the C ABI).
+
+fp32: max abs error <= 1e-5.  fp16: inputs are fp16-rounded, the oracle does fp32 arithmetic on
+them, the kernel rounds once at the store: max abs error <= 2e-3.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import port
+
+from gpu_util import gqa_decode, lib
+
+pytestmark = pytest.mark.gpu
+
+TOL32, TOL16 = 1e-5, 2e-3
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "decode_path_golden.npz"))
+
+
+def _qkv_ref(rng, L, hq=16, hkv=8, d=128, dtype=np.float32):
+    q = rng.standard_normal((1, hq, d)).astype(np.float32).astype(dtype)
+    k = rng.standard_normal((L, hkv, d)).astype(np.float32).astype(dtype)
+    v = rng.standard_normal((L, hkv, d)).astype(np.float32).astype(dtype)
+    return q, k, v
+
+
+def test_reference_shape_fp32_config1():
+    """B=1, Hq16/Hkv8, D=128, L=1024, fp32 (the reference's own call shape)."""
+    rng = np.random.default_rng(1)
+    q, k, v = _qkv_ref(rng, 1024)
+    out = gqa_decode(q, k, v, layout="ref")
+    np.testing.assert_allclose(out, port.gqa_decode(q, k, v), rtol=0, atol=TOL32)
+
+
+@pytest.mark.parametrize("L", [1, 7, 256, 512, 1024])
+def test_reference_seeds_fp32(L):
+    rs = np.random.RandomState(3)
+    for n in (1, 7, 256, 512, 1024):
+        q = rs.randn(1, 16, 128).astype(np.float32)
+        k = rs.randn(n, 8, 128).astype(np.float32)
+        v = rs.randn(n, 8, 128).astype(np.float32)
+        if n == L:
+            np.testing.assert_allclose(gqa_decode(q, k, v, layout="ref"), port.gqa_decode(q, k, v), rtol=0, atol=TOL32)
+
+
+def test_golden_fixtures():
+    for L in (1, 7, 40):
+        out = gqa_decode(G[f"gqa_L{L}_q"], G[f"gqa_L{L}_k"], G[f"gqa_L{L}_v"], layout="ref")
+        np.testing.assert_allclose(out, G[f"gqa_L{L}_out"], rtol=0, atol=TOL32)
+    out = gqa_decode(G["gqa16_q"], G["gqa16_k"], G["gqa16_v"], layout="ref")
+    np.testing.assert_allclose(out.astype(np.float32), G["gqa16_out"], rtol=0, atol=TOL16)
+
+
+@pytest.mark.parametrize("L", [2048, 4097, 16385])
+def test_long_context_splits_fp32(L):
+    """Lengths the reference would send to its split-K kernels (L >= 2048), incl. a ragged tail."""
+    rng = np.random.default_rng(L)
+    q, k, v = _qkv_ref(rng, L)
+    np.testing.assert_allclose(gqa_decode(q, k, v, layout="ref"), port.gqa_decode(q, k, v), rtol=0, atol=TOL32)
+
+
+@pytest.mark.parametrize("B,L", [(1, 1024), (8, 1024), (32, 1024), (4, 8192), (2, 32768)])
+def test_cache_layout_fp16(B, L):
+    rng = np.random.default_rng(B * 100003 + L)
+    q = rng.standard_normal((B, 16, 128)).astype(np.float32).astype(np.float16)
+    k = rng.standard_normal((B, 8, L, 128)).astype(np.float32).astype(np.float16)
+    v = rng.standard_normal((B, 8, L, 128)).astype(np.float32).astype(np.float16)
+    out = gqa_decode(q, k, v).astype(np.float32)
+    want = port.gqa_decode_cache_native(q, k, v)
+    err = np.abs(out - want).max()
+    assert err <= TOL16, (err, np.abs(want).max())
+
+
+def test_ragged_batch_fp16():
+    rng = np.random.default_rng(77)
+    B, Lmax = 8, 4096
+    lens = rng.integers(1, Lmax + 1, B).astype(np.int32)
+    lens[0], lens[1], lens[2] = Lmax, 1, 0  # full, single key, empty (zeros by convention)
+    q = rng.standard_normal((B, 16, 128)).astype(np.float32).astype(np.float16)
+    k = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
+    v = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
+    out = gqa_decode(q, k, v, lens).astype(np.float32)
+    want = port.gqa_decode_cache_native(q, k, v, lens)
+    assert np.abs(out - want).max() <= TOL16
+    assert np.all(out[2] == 0)
+    np.testing.assert_array_equal(out[1, 0], v[1, 0, 0].astype(np.float32))  # one key: out = v
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 8, 64), (8, 2, 128), (16, 2, 64), (4, 1, 256), (6, 2, 128)])
+def test_head_shapes(hq, hkv, d):
+    """group sizes 1, 4, 8, 4 (D=256) and 3 (not a power of two)."""
+    rng = np.random.default_rng(hq * 31 + d)
+    B, L = 3, 777
+    lens = np.array([777, 300, 1], np.int32)
+    for dtype, tol in ((np.float32, TOL32), (np.float16, TOL16)):
+        q = rng.standard_normal((B, hq, d)).astype(np.float32).astype(dtype)
+        k = rng.standard_normal((B, hkv, L, d)).astype(np.float32).astype(dtype)
+        v = rng.standard_normal((B, hkv, L, d)).astype(np.float32).astype(dtype)
+        out = gqa_decode(q, k, v, lens).astype(np.float32)
+        want = port.gqa_decode_cache_native(q, k, v, lens)
+        assert np.abs(out - want).max() <= tol
+
+
+def test_result_independent_of_split_count():
+    rng = np.random.default_rng(5)
+    q, k, v = _qkv_ref(rng, 5000)
+    outs = []
+    for splits in (1, 3, 16):
+        lib().axhip_gqa_decode_tune(0, splits)
+        outs.append(gqa_decode(q, k, v, layout="ref"))
+    lib().axhip_gqa_decode_tune(0, 0)
+    want = port.gqa_decode(q, k, v)
+    for o in outs:
+        np.testing.assert_allclose(o, want, rtol=0, atol=TOL32)
+
+
+def test_invariants_full_size_headline():
+    """B=32, L=8192 fp16 (1 GiB of cache): properties that need no oracle pass over the data.
+    Identical keys give the mean of V; the first sequence is also checked against the oracle."""
+    B, L = 32, 8192
+    rng = np.random.default_rng(9)
+    q = rng.standard_normal((B, 16, 128)).astype(np.float32).astype(np.float16)
+    v = rng.standard_normal((B, 8, L, 128)).astype(np.float32).astype(np.float16)
+    k = np.empty((B, 8, L, 128), np.float16)
+    k[:] = rng.standard_normal((B, 8, 1, 128)).astype(np.float16)  # every key of a head identical
+    k[0] = rng.standard_normal((8, L, 128)).astype(np.float16)      # sequence 0: ordinary keys
+    out = gqa_decode(q, k, v).astype(np.float32)
+    mean_v = v.astype(np.float32).mean(axis=2)  # [B,8,128]
+    for h in range(16):
+        assert np.abs(out[1:, h] - mean_v[1:, h // 2]).max() <= TOL16
+    want0 = port.gqa_decode_cache_native(q[:1], k[:1], v[:1])
+    assert np.abs(out[:1] - want0).max() <= TOL16
+
+
+def test_error_codes():
+    l = lib()
+    assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 8, 128, 16, 0, 0, 0, None) == 7
+    assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 5, 128, 16, 0, 0, 0, None) == 4
+    assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 3, 1, 16, 8, 128, 16, 0, 0, 0, None) == 3
+    assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 8, 96, 16, 0, 0, 0, None) == 1

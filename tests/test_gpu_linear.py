@@ -1,0 +1,98 @@
+"""fp16 Linear (x @ W^T + b, fp16 operands, fp32 accumulate on MFMA) against the CPU oracle.
+
+Products of two fp16 values are exact in fp32, so the only difference from the oracle's sequential
+fp32 sum is accumulation order; the bound used is 1e-5 + 4 * sqrt(K) * 2^-24 * sum|terms| per
+output (fp32 output), and 2e-3 for the fp16-output variant at |out| < 2.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import port
+
+import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "decode_path_golden.npz"))
+
+
+def h16(a):
+    return np.asarray(a, np.float32).astype(np.float16)
+
+
+def check_linear(x, w, b=None):
+    out = gu.linear_f16(x, w, b)
+    x32 = x.astype(np.float16).astype(np.float32)  # fp32 activations are rounded to fp16 first (RNE)
+    w32 = w.astype(np.float32)
+    want = port.linear(x32, w32, None if b is None else b.astype(np.float32))
+    K = x.shape[1]
+    mag = np.abs(x32) @ np.abs(w32).T
+    bound = 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag
+    err = np.abs(out - want)
+    assert np.all(err <= bound), (err.max(), bound.min(), x.shape, w.shape)
+    return out
+
+
+def test_golden_fixture():
+    np.testing.assert_allclose(gu.linear_f16(G["lin_x"], G["lin_w"]), G["lin_out"], rtol=0, atol=2e-5)
+    np.testing.assert_allclose(gu.linear_f16(G["lin_x"], G["lin_w"], G["lin_b"]), G["lin_out_bias"], rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("M", [1, 16, 32, 512])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 12288), (6144, 2048)])
+def test_config4_shapes(M, K, N):
+    rng = np.random.default_rng(M * 7 + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    check_linear(x, w)
+
+
+def test_lm_head_slice_and_full_M16():
+    rng = np.random.default_rng(99)
+    K, N = 2048, 151936
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    x = h16(rng.standard_normal((16, K)))
+    out = gu.linear_f16(x, w)
+    # the oracle on every 37th output column (the full 16x151936x2048 CPU product takes minutes)
+    cols = np.arange(0, N, 37)
+    want = port.linear(x.astype(np.float32), w[cols].astype(np.float32))
+    assert np.abs(out[:, cols] - want).max() <= 1e-4
+    # linearity in x: f(2x) = 2 f(x) exactly (scaling by 2 is exact in fp16 and fp32)
+    np.testing.assert_array_equal(gu.linear_f16(h16(2 * x.astype(np.float32)), w), 2 * out)
+
+
+def test_fp32_activations_bias_odd_shapes():
+    rng = np.random.default_rng(5)
+    for (M, K, N) in [(8, 64, 32), (3, 72, 50), (17, 136, 33), (33, 520, 130), (130, 264, 190)]:
+        x = rng.standard_normal((M, K)).astype(np.float32)  # fp32 in, as the reference's Linear.forward passes
+        w = h16(0.05 * rng.standard_normal((N, K)))
+        b = h16(0.05 * rng.standard_normal(N))
+        check_linear(x, w, b)
+        check_linear(x, w)
+
+
+def test_fp16_output_variant():
+    rng = np.random.default_rng(6)
+    x = h16(rng.standard_normal((16, 2048)))
+    w = h16(0.02 * rng.standard_normal((2048, 2048)))
+    out16 = gu.linear_f16(x, w, out_dtype=np.float16)
+    want = port.linear(x.astype(np.float32), w.astype(np.float32))
+    assert np.abs(out16.astype(np.float32) - want).max() <= 2e-3 * max(1.0, np.abs(want).max() / 2)
+
+
+def test_matches_fp32_linear_loosely_like_reference_test():
+    """tests/core/test_fp16.py:28-46 of the reference: fp16 Linear vs fp32 Linear at 5e-2."""
+    rng = np.random.default_rng(1)
+    x = rng.normal(size=(8, 64)).astype(np.float32)
+    w = (rng.normal(size=(32, 64)) * 0.05).astype(np.float32)
+    b = (rng.normal(size=(32,)) * 0.05).astype(np.float32)
+    out = gu.linear_f16(x, h16(w), h16(b))
+    np.testing.assert_allclose(out, x @ w.T + b, rtol=5e-2, atol=5e-2)
+
+
+def test_error_codes():
+    l = gu.lib()
+    assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 60, 8, None, 0, None) == 1  # K % 8
+    assert l.axhip_linear_f16(None, 2, None, None, None, 5, 4, 64, 8, None, 0, None) == 3  # x dtype
+    assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 64, 8, None, 0, None) == 7  # null pointers

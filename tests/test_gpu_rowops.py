@@ -1,0 +1,221 @@
+"""Fused / row-wise / rotary / cache-append kernels on the GPU against the CPU oracle.
+
+Tolerances: fp32 max abs error <= 1e-5; fp16 <= 2e-3 against the fp32 oracle on fp16-rounded
+inputs (the kernel rounds once at the store; where |value| >= 4 half an fp16 ulp alone is 1.95e-3,
+so those few elements are compared at one ulp of their magnitude).  Byte movers are bit exact.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import port
+
+import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+TOL32, TOL16 = 1e-5, 2e-3
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "decode_path_golden.npz"))
+
+
+def h16(a):
+    return np.asarray(a, np.float32).astype(np.float16)
+
+
+def assert_fp16_close(got, want):
+    """<= 2e-3 absolute, or for large magnitudes half an fp16 ulp of the value plus 2e-3 relative slack."""
+    got = got.astype(np.float32)
+    err = np.abs(got - want)
+    ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
+    bound = np.maximum(TOL16, 0.5 * ulp + 1e-3 * np.abs(want))
+    assert np.all(err <= bound), (err.max(), np.abs(want).max())
+
+
+# ---- config 1 (fp32 op check) and golden fixtures ---------------------------------------------
+def test_add_rms_norm_fp32_config1():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((1, 2048)).astype(np.float32)
+    r = rng.standard_normal((1, 2048)).astype(np.float32)
+    w = (1 + 0.02 * rng.standard_normal(2048)).astype(np.float32)
+    y, out = gu.add_rms_norm(x, r, w, 1e-6)
+    wy, wout = port.add_rms_norm(x, r, w, 1e-6)
+    np.testing.assert_array_equal(y, wy)  # a single fp32 add
+    np.testing.assert_allclose(out, wout, rtol=0, atol=TOL32)
+
+
+def test_golden_fused_and_rotary_fp32():
+    y, out = gu.add_rms_norm(G["arn_x"], G["arn_res"], G["arn_w"], 1e-6)
+    np.testing.assert_array_equal(y, G["arn_y"])
+    np.testing.assert_allclose(out, G["arn_out"], rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.rms_norm(G["arn_x"], G["arn_w"], 1e-6), G["rms_out"], rtol=0, atol=TOL32)
+    s = gu.silu_mul(G["silu_gate"], G["silu_up"])
+    np.testing.assert_allclose(s, G["silu_out"], rtol=2e-6, atol=TOL32)
+    x, pos = G["rope_x"], G["rope_pos"]
+    np.testing.assert_allclose(gu.rope(x, pos, 1e6), G["rope_out_theta1e6"], rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.rope(x, pos, 1e4), G["rope_out_theta1e4"], rtol=0, atol=TOL32)
+    inv, pos3 = G["mrope_inv_freq"], G["mrope_pos3"]
+    np.testing.assert_allclose(gu.rope_thd(x, pos3, inv, [24, 20, 20]), G["rope_thd_out"], rtol=0, atol=TOL32)
+    c, s_ = gu.mrope_cos_sin(pos3, inv, 20, 20)
+    np.testing.assert_allclose(c, G["mrope_cos"], rtol=0, atol=TOL32)
+    np.testing.assert_allclose(s_, G["mrope_sin"], rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.rope_with_cos_sin(x, G["mrope_cos"], G["mrope_sin"]), G["rope_cos_sin_out"], rtol=0, atol=TOL32)
+
+
+def test_reference_test_shapes_fp32():
+    """Shapes of the reference's own fused tests: 37x53 silu_mul (odd size), 4x128 and 2x64 norms."""
+    rs = np.random.RandomState(0)
+    g = rs.randn(37, 53).astype(np.float32)
+    u = rs.randn(37, 53).astype(np.float32)
+    np.testing.assert_allclose(gu.silu_mul(g, u), port.silu_mul(g, u), rtol=2e-6, atol=1e-6)
+    rs = np.random.RandomState(1)
+    x = rs.randn(4, 128).astype(np.float32)
+    r = rs.randn(4, 128).astype(np.float32)
+    w = rs.randn(128).astype(np.float32)
+    y, out = gu.add_rms_norm(x, r, w, 1e-6)
+    wy, wout = port.add_rms_norm(x, r, w, 1e-6)
+    np.testing.assert_array_equal(y, wy)
+    np.testing.assert_allclose(out, wout, rtol=0, atol=TOL32)
+    # rows that are not a multiple of 16 bytes take the element-wise path
+    x = rs.randn(5, 53).astype(np.float32)
+    w = rs.randn(53).astype(np.float32)
+    np.testing.assert_allclose(gu.rms_norm(x, w, 1e-5), port.rms_norm(x, w, 1e-5), rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.rms_norm(x, None, 1e-5), port.rms_norm(x, None, 1e-5), rtol=0, atol=TOL32)
+
+
+# ---- config 2 (fp16, B = 32) -------------------------------------------------------------------
+def test_add_rms_norm_fp16_config2():
+    rng = np.random.default_rng(20)
+    x, r = h16(rng.standard_normal((32, 2048))), h16(rng.standard_normal((32, 2048)))
+    w32 = (1 + 0.02 * rng.standard_normal(2048)).astype(np.float32)
+    wy, wout = port.add_rms_norm(x, r, h16(w32), 1e-6)
+    for w in (h16(w32),):
+        y, out = gu.add_rms_norm(x, r, w, 1e-6)
+        np.testing.assert_array_equal(y.view(np.uint16), wy.astype(np.float16).view(np.uint16))  # one rounding of an exact-in-fp32 sum
+        assert_fp16_close(out, wout)
+    # fp32 weights with fp16 activations
+    wy, wout = port.add_rms_norm(x, r, w32, 1e-6)
+    y, out = gu.add_rms_norm(x, r, w32, 1e-6)
+    assert_fp16_close(out, wout)
+
+
+def test_silu_mul_fp16_config2():
+    rng = np.random.default_rng(21)
+    g, u = h16(rng.standard_normal((32, 6144))), h16(rng.standard_normal((32, 6144)))
+    assert_fp16_close(gu.silu_mul(g, u), port.silu_mul(g, u))
+
+
+def test_rope_fp16_config2():
+    rng = np.random.default_rng(22)
+    pos = rng.integers(0, 8192, 32).astype(np.int64)
+    for heads in (16, 8):
+        x = h16(rng.standard_normal((32, heads, 128)))
+        assert_fp16_close(gu.rope(x, pos, 1e6), port.rope(x, pos, 1e6))
+    # fp32 at the same positions: the fp32 angle products are formed exactly as on the CPU
+    x = rng.standard_normal((32, 16, 128)).astype(np.float32)
+    np.testing.assert_allclose(gu.rope(x, pos, 1e6), port.rope(x, pos, 1e6), rtol=0, atol=TOL32)
+
+
+def test_mrope_family():
+    rng = np.random.default_rng(23)
+    rows = 33
+    inv = port.rope_inv_freq(1e6, 128)
+    pos3 = rng.integers(0, 8192, (3, rows)).astype(np.int64)
+    x = rng.standard_normal((rows, 4, 128)).astype(np.float32)
+    np.testing.assert_allclose(gu.rope_thd(x, pos3, inv, [24, 20, 20]), port.rope_thd(x, pos3, inv, [24, 20, 20]), rtol=0, atol=TOL32)
+    assert_fp16_close(gu.rope_thd(h16(x), pos3, inv, [24, 20, 20]), port.rope_thd(h16(x), pos3, inv, [24, 20, 20]))
+    c, s = gu.mrope_cos_sin(pos3, inv, 20, 20)
+    wc, ws = port.mrope_cos_sin(pos3, inv, 20, 20)
+    np.testing.assert_allclose(c, wc, rtol=0, atol=TOL32)
+    np.testing.assert_allclose(s, ws, rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.rope_with_cos_sin(x, wc, ws), port.rope_with_cos_sin(x, wc, ws), rtol=0, atol=TOL32)
+    # decode case T = H = W: rope_thd equals rope
+    p = pos3[0]
+    np.testing.assert_allclose(gu.rope_thd(x, np.stack([p, p, p]), inv, [24, 20, 20]), port.rope(x, p, 1e6), rtol=0, atol=TOL32)
+    # small head (the reference's rope test shape 4x2x8, theta 1e4)
+    xs = rng.standard_normal((4, 2, 8)).astype(np.float32)
+    np.testing.assert_allclose(gu.rope(xs, np.arange(4), 1e4), port.rope(xs, np.arange(4), 1e4), rtol=0, atol=TOL32)
+
+
+def test_kv_append_bit_exact_config2():
+    rng = np.random.default_rng(24)
+    B, Hkv, Lmax, D = 32, 8, 8192, 128
+    kc = rng.integers(0, 65536, (B, Hkv, Lmax, D), dtype=np.uint16).view(np.float16)
+    vc = rng.integers(0, 65536, (B, Hkv, Lmax, D), dtype=np.uint16).view(np.float16)
+    kn = rng.integers(0, 65536, (B, Hkv, D), dtype=np.uint16).view(np.float16)  # all bit patterns incl. NaNs
+    vn = rng.integers(0, 65536, (B, Hkv, D), dtype=np.uint16).view(np.float16)
+    pos = rng.integers(0, Lmax, B).astype(np.int64)
+    pos[0], pos[1] = 0, Lmax - 1
+    gk, gv = gu.kv_append(kn, vn, kc, vc, pos)
+    port.kv_append(kn, vn, kc, vc, pos)  # in place on the host copies
+    np.testing.assert_array_equal(gk.view(np.uint16), kc.view(np.uint16))  # incl. every untouched byte
+    np.testing.assert_array_equal(gv.view(np.uint16), vc.view(np.uint16))
+
+
+def test_kv_append_int32_pos_fp32_and_out_of_range():
+    rng = np.random.default_rng(25)
+    B, Hkv, Lmax, D = 3, 2, 16, 64
+    kc = rng.standard_normal((B, Hkv, Lmax, D)).astype(np.float32)
+    vc = rng.standard_normal((B, Hkv, Lmax, D)).astype(np.float32)
+    kn = rng.standard_normal((B, Hkv, D)).astype(np.float32)
+    vn = rng.standard_normal((B, Hkv, D)).astype(np.float32)
+    pos = np.array([5, 16, -1], np.int32)  # the last two are outside [0,Lmax): skipped
+    gk, gv = gu.kv_append(kn, vn, kc, vc, pos)
+    wk, wv = kc.copy(), vc.copy()
+    wk[0, :, 5], wv[0, :, 5] = kn[0], vn[0]
+    np.testing.assert_array_equal(gk, wk)
+    np.testing.assert_array_equal(gv, wv)
+
+
+def test_concat_append_matches_reference_semantics():
+    rng = np.random.default_rng(26)
+    a = h16(rng.standard_normal((300, 8, 128)))
+    b = h16(rng.standard_normal((1, 8, 128)))
+    np.testing.assert_array_equal(gu.concat_axis0(a, b).view(np.uint16), port.concat_axis0(a, b).view(np.uint16))
+    a8 = rng.integers(0, 255, (7, 3), dtype=np.uint8).view(np.int8)  # unaligned sizes
+    b8 = rng.integers(0, 255, (2, 3), dtype=np.uint8).view(np.int8)
+    da, db = gu.dev(a8), gu.dev(b8)
+    do = gu.DeviceBuffer(27)
+    gu._run("axhip_concat", da.ptr, db.ptr, do.ptr, 1, 21, 6, None)
+    gu.synchronize()
+    np.testing.assert_array_equal(do.download(np.int8, (9, 3)), np.concatenate([a8, b8]))
+
+
+def test_cast_add_embedding_argmax():
+    rng = np.random.default_rng(27)
+    x = rng.standard_normal(100003).astype(np.float32) * 10
+    np.testing.assert_array_equal(gu.cast(x, np.float16).view(np.uint16), x.astype(np.float16).view(np.uint16))  # IEEE RNE
+    np.testing.assert_array_equal(gu.cast(np.array([1.0, -0.5, 65504.0, 0.0, 1e-7, 70000.0], np.float32), np.float16).view(np.uint16),
+                                  np.array([1.0, -0.5, 65504.0, 0.0, 1e-7, 70000.0], np.float32).astype(np.float16).view(np.uint16))
+    hb = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16)  # every finite non-negative half, subnormals too
+    np.testing.assert_array_equal(gu.cast(hb, np.float32), hb.astype(np.float32))
+    a, b = rng.standard_normal((16, 2048)).astype(np.float32), rng.standard_normal((16, 2048)).astype(np.float32)
+    np.testing.assert_array_equal(gu.add(a, b), a + b)
+    np.testing.assert_array_equal(gu.add(h16(a), h16(b)).view(np.uint16), (h16(a).astype(np.float32) + h16(b).astype(np.float32)).astype(np.float16).view(np.uint16))
+    table = h16(rng.standard_normal((1000, 2048)))
+    ids = rng.integers(0, 1000, (16, 1)).astype(np.int64)
+    np.testing.assert_array_equal(gu.embedding(ids, table).view(np.uint16), table[ids].view(np.uint16))
+    t32 = rng.standard_normal((10, 4)).astype(np.float32)
+    ids2 = np.array([[1, 3], [5, 2]], np.int64)
+    np.testing.assert_array_equal(gu.embedding(ids2, t32), port.embedding(ids2, t32))
+    lg = rng.standard_normal((16, 151936)).astype(np.float32)
+    lg[3, 777] = lg[3, 150000] = 50.0  # tie: first index wins
+    np.testing.assert_array_equal(gu.argmax(lg), port.argmax(lg))
+    assert gu.argmax(lg)[3] == 777
+    np.testing.assert_array_equal(gu.argmax(h16(lg)), port.argmax(h16(lg).astype(np.float32)))
+
+
+def test_sdpa_prefill_and_small_heads():
+    rng = np.random.default_rng(28)
+    q = rng.standard_normal((50, 4, 64)).astype(np.float32)
+    k = rng.standard_normal((50, 2, 64)).astype(np.float32)
+    v = rng.standard_normal((50, 2, 64)).astype(np.float32)
+    for causal in (True, False):
+        np.testing.assert_allclose(gu.sdpa(q, k, v, causal), port.sdpa(q, k, v, causal), rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.sdpa(G["sdpa_q"], G["sdpa_k"], G["sdpa_v"], True), G["sdpa_causal_out"], rtol=0, atol=TOL32)
+    np.testing.assert_allclose(gu.sdpa(G["sdpa_q"], G["sdpa_k"], G["sdpa_v"], False), G["sdpa_full_out"], rtol=0, atol=TOL32)
+    # decode-with-cache equals causal full forward (tests/nn/test_kv_cache.py:120-148 of the reference)
+    full = gu.sdpa(q, k, v, True)
+    for t in (0, 17, 49):
+        step = gu.sdpa(q[t:t + 1], k[:t + 1], v[:t + 1], False)
+        np.testing.assert_allclose(step[0], full[t], rtol=0, atol=TOL32)

@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  The metric is BASELINE.json's: "GQA decode HBM GB/s (% of peak) B=32 L=8k
+fp16; decode tok/s 2B-shape B=16".  `value` is the first half: achieved algorithmic GB/s of the
+split-K GQA decode attention at B=32, Hq=16, Hkv=8, D=128, L=8192, fp16 KV cache resident in HBM.
+A "step" is one pass of that operator over one batch (split kernel + merge kernel).  The second half
+(tokens/s of the Qwen3-VL-2B-shaped text decode step, B=16, 128 hipGraph replays) is reported in
+`decode_step` on the same line.
+
+Algorithmic bytes per step: 4096 * sum_b L_b (K and V: 2 * Hkv * D * 2 bytes per token) + 8192 * B
+(q and out) = 1 074 003 968 B.  Split-K workspace traffic is not credited.  Several KV buffers are
+rotated so that no step can find its cache lines in the 256 MB Infinity Cache.
+
+The CPU baseline runs Axono's own CPU operator (oracle/_ref, compiled from the reference's sources)
+or, where that is absent, the C restatement, on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+F16 = 4
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gqa_bytes(B, L_sum, Hq=16, Hkv=8, D=128, esz=2):
+    return 2 * Hkv * D * esz * L_sum + 2 * Hq * D * esz * B
+
+
+class GqaBench:
+    """Headline workload: fp16 cache [B,Hkv,L,D], one query token per sequence."""
+
+    def __init__(self, B=32, L=8192, Hq=16, Hkv=8, D=128, n_rot=4, seed=0, lens=None):
+        from axono_amd import _lib
+        from axono_amd.device import DeviceBuffer, check
+
+        self.lib = _lib.load()
+        self.check = check
+        self.B, self.L, self.Hq, self.Hkv, self.D = B, L, Hq, Hkv, D
+        rng = np.random.default_rng(seed)
+        cache_elems = B * Hkv * L * D
+        # one 64 MiB block of N(0,1) fp16 values tiled over every buffer at shifting offsets: the
+        # values do not affect the timing and the parity check below uses its own small case
+        block = rng.standard_normal(32 * 1024 * 1024).astype(np.float32).astype(np.float16)
+        self.kv = []
+        for r in range(n_rot):
+            kb, vb = DeviceBuffer(cache_elems * 2), DeviceBuffer(cache_elems * 2)
+            for buf, shift in ((kb, 2 * r), (vb, 2 * r + 1)):
+                off = 0
+                rolled = np.roll(block, 4099 * (shift + 1))
+                while off < cache_elems * 2:
+                    n = min(rolled.nbytes, cache_elems * 2 - off)
+                    buf.upload(rolled[: n // 2], off)
+                    off += n
+            self.kv.append((kb, vb))
+        q = rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16)
+        self.q = DeviceBuffer.from_numpy(q)
+        self.out = DeviceBuffer(q.nbytes)
+        self.lens_host = None if lens is None else np.asarray(lens, np.int32)
+        self.lens = DeviceBuffer.from_numpy(self.lens_host) if lens is not None else None
+        self.ws_bytes = self.lib.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
+        self.ws = DeviceBuffer(max(self.ws_bytes, 256))
+        self.step_i = 0
+        L_sum = int(self.lens_host.sum()) if lens is not None else B * L
+        self.bytes_per_step = gqa_bytes(B, L_sum, Hq, Hkv, D)
+
+    def step(self):
+        kb, vb = self.kv[self.step_i % len(self.kv)]
+        self.step_i += 1
+        B, Hq, Hkv, D, L = self.B, self.Hq, self.Hkv, self.D, self.L
+        self.check(self.lib.axhip_gqa_decode(self.q.ptr, kb.ptr, vb.ptr, self.lens.ptr if self.lens else None,
+                                             self.out.ptr, self.ws.ptr, self.ws_bytes, F16, B, Hq, Hkv, D, L,
+                                             Hkv * L * D, L * D, D, None), "gqa_decode")
+
+    def plan(self):
+        s, c = C.c_int(0), C.c_int(0)
+        self.lib.axhip_gqa_decode_plan(self.B, self.Hq, self.Hkv, self.L, C.byref(s), C.byref(c))
+        return {"n_splits": s.value, "chunk": c.value}
+
+
+def time_steps(lib, step, steps, warmup):
+    """Returns (wall ms per step, HIP-event ms per step) over exactly `steps` steps."""
+    from axono_amd.device import check
+
+    for _ in range(warmup):
+        step()
+    check(lib.axhip_synchronize(), "sync")
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.axhip_event_create(C.byref(e0)), "event")
+    check(lib.axhip_event_create(C.byref(e1)), "event")
+    t0 = time.perf_counter()
+    check(lib.axhip_event_record(e0, None), "event_record")  # same stream as the kernels (default)
+    for _ in range(steps):
+        step()
+    check(lib.axhip_event_record(e1, None), "event_record")
+    check(lib.axhip_synchronize(), "sync")
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = C.c_float(0)
+    check(lib.axhip_event_elapsed_ms(e0, e1, C.byref(ms)), "event_elapsed")
+    lib.axhip_event_destroy(e0)
+    lib.axhip_event_destroy(e1)
+    return wall_ms, ms.value / steps
+
+
+def cpu_baseline_gqa(budget_s=12.0):
+    """Axono's CPU attention on B_s sequences of the headline shape (fp32 math on fp16-rounded
+    data), threads = host cores.  Returns the cpu_baseline object."""
+    import oracle
+
+    cores = oracle.port.num_threads()
+    kind = "reference" if oracle.ref is not None else "port"
+    ops = oracle.ref if oracle.ref is not None else oracle.port
+    rng = np.random.default_rng(1)
+    L, Hq, Hkv, D = 8192, 16, 8, 128
+    q = rng.standard_normal((1, Hq, D)).astype(np.float16).astype(np.float32)
+    k = rng.standard_normal((L, Hkv, D)).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((L, Hkv, D)).astype(np.float16).astype(np.float32)
+    ops.sdpa(q, k, v, False)  # warm
+    n, t_total, best = 0, 0.0, float("inf")
+    while t_total < budget_s and n < 4096:
+        t0 = time.perf_counter()
+        ops.sdpa(q, k, v, False)
+        dt = time.perf_counter() - t0
+        best = min(best, dt)
+        t_total += dt
+        n += 1
+    gbs = gqa_bytes(1, L) / best / 1e9
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": cores, "kind": kind,
+            "sample": f"one sequence of the headline shape (B=1 of 32, L=8192, Hq16/Hkv8/D128), "
+                      f"min of {n} runs, fp32 arithmetic on fp16-rounded data; bytes counted as fp16"}
+
+
+def smoke_parity(lib):
+    """Small invocation checked against the oracle; raises on mismatch."""
+    import oracle
+    from axono_amd.device import DeviceBuffer, check
+
+    rng = np.random.default_rng(3)
+    B, Hq, Hkv, D, L = 2, 16, 8, 128, 600
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16)
+    k = rng.standard_normal((B, Hkv, L, D)).astype(np.float32).astype(np.float16)
+    v = rng.standard_normal((B, Hkv, L, D)).astype(np.float32).astype(np.float16)
+    lens = np.array([600, 123], np.int32)
+    dq, dk, dv, dl = (DeviceBuffer.from_numpy(a) for a in (q, k, v, lens))
+    do = DeviceBuffer(q.nbytes)
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
+    ws = DeviceBuffer(max(wsb, 256))
+    check(lib.axhip_gqa_decode(dq.ptr, dk.ptr, dv.ptr, dl.ptr, do.ptr, ws.ptr, wsb, F16, B, Hq, Hkv, D, L,
+                               Hkv * L * D, L * D, D, None), "gqa_decode")
+    check(lib.axhip_synchronize(), "sync")
+    got = do.download(np.float16, q.shape).astype(np.float32)
+    want = oracle.port.gqa_decode_cache_native(q, k, v, lens)
+    err = float(np.abs(got - want).max())
+    if not err <= 2e-3:
+        raise RuntimeError(f"GQA decode parity check failed: max abs err {err}")
+    return err
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode-step", action="store_true")
+    ap.add_argument("--decode-steps", type=int, default=128)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported "
+              "(the decode path shards by batch or kv-head with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    from axono_amd import _lib
+
+    lib = _lib.load()
+    if _lib.device_count() < 1:
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        sys.exit(3)
+    name = C.create_string_buffer(256)
+    gfx, tot, cus = C.c_int(0), C.c_size_t(0), C.c_int(0)
+    lib.axhip_device_info(0, name, 256, C.byref(gfx), C.byref(tot), C.byref(cus))
+    log(f"device: {name.value.decode()} CUs={cus.value} mem={tot.value / 2**30:.0f} GiB")
+
+    err = smoke_parity(lib)
+    log(f"parity (small case vs oracle): max abs err {err:.2e}")
+
+    wl = GqaBench()
+    log(f"GQA decode plan: {wl.plan()}  bytes/step={wl.bytes_per_step}")
+    wall_ms, ev_ms = time_steps(lib, wl.step, args.steps, args.warmup)
+    gbs = wl.bytes_per_step / (ev_ms * 1e-3) / 1e9
+    gbs_wall = wl.bytes_per_step / (wall_ms * 1e-3) / 1e9
+    log(f"GQA decode: {ev_ms * 1e3:.1f} us/step (events), {wall_ms * 1e3:.1f} us/step (wall): "
+        f"{gbs:.0f} GB/s = {100 * gbs / HBM_PEAK_GBS:.1f}% of {HBM_PEAK_GBS:.0f}")
+
+    result = {
+        "metric": "GQA decode HBM GB/s (% of peak) B=32 L=8k fp16; decode tok/s 2B-shape B=16",
+        "value": round(gbs_wall, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "split-K GQA flash-decoding, fp16 KV cache [B,Hkv,L,D], fp32 accumulate",
+                   "B": 32, "Hq": 16, "Hkv": 8, "D": 128, "L": 8192, "plan": wl.plan(),
+                   "kv_buffers_rotated": len(wl.kv)},
+        "pct_of_hbm_peak": round(100 * gbs_wall / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gqa_decode_split_kernel<half,128,2> (+ merge)",
+                     "avg_launch_us": round(ev_ms * 1e3, 2), "algorithmic_bytes": wl.bytes_per_step},
+    }
+    del wl
+
+    if not args.no_decode_step:
+        try:
+            from axono_amd.examples import qwen3vl_text_bench
+        except ImportError:
+            qwen3vl_text_bench = None
+        if qwen3vl_text_bench is not None:
+            result["decode_step"] = qwen3vl_text_bench.run(decode_steps=args.decode_steps, log=log)
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_gqa()
+        log(f"cpu baseline: {result['cpu_baseline']}")
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

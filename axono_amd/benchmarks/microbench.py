@@ -1,0 +1,222 @@
+"""Per-operator micro-benchmarks of the decode path (HIP-event timing, through the C ABI).
+
+    python -m axono_amd.benchmarks.microbench gqa   [--B 32 --L 8192 --steps 100 --ragged]
+    python -m axono_amd.benchmarks.microbench gqa-sweep
+    python -m axono_amd.benchmarks.microbench copy  [--mib 1024 --steps 20]
+    python -m axono_amd.benchmarks.microbench rowops
+    python -m axono_amd.benchmarks.microbench linear
+
+Each line reports algorithmic bytes (or flops) over the average launch time and the fraction of
+the MI355X peak (HBM 8 TB/s; fp16 dense MFMA 2.5 PFLOP/s).  `copy` is the plain device-to-device
+copy kernel of known size that counter readings (FETCH_SIZE / WRITE_SIZE) are scaled against.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import sys
+
+import numpy as np
+
+from axono_amd import _lib
+from axono_amd.device import DeviceBuffer, check
+
+HBM_PEAK = 8000.0      # GB/s
+MFMA_F16_PEAK = 2500.0  # TFLOP/s dense
+F16, F32, I64 = 4, 5, 3
+
+
+def _time(lib, fn, steps, warmup=5):
+    for _ in range(warmup):
+        fn()
+    check(lib.axhip_synchronize(), "sync")
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.axhip_event_create(C.byref(e0))
+    lib.axhip_event_create(C.byref(e1))
+    lib.axhip_event_record(e0, None)
+    for _ in range(steps):
+        fn()
+    lib.axhip_event_record(e1, None)
+    ms = C.c_float(0)
+    check(lib.axhip_event_elapsed_ms(e0, e1, C.byref(ms)), "elapsed")
+    lib.axhip_event_destroy(e0)
+    lib.axhip_event_destroy(e1)
+    return ms.value / steps * 1e3  # us
+
+
+def _rand_fill(buf, nbytes, seed):
+    rng = np.random.default_rng(seed)
+    block = rng.standard_normal(8 * 1024 * 1024).astype(np.float32).astype(np.float16)
+    off = 0
+    while off < nbytes:
+        n = min(block.nbytes, nbytes - off)
+        buf.upload(block[: n // 2], off)
+        off += n
+
+
+def _emit(rec):
+    print(json.dumps(rec), flush=True)
+
+
+def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag="gqa"):
+    elems = B * Hkv * L * D
+    if n_rot is None:  # enough distinct buffers to exceed the 256 MB Infinity Cache several times
+        n_rot = max(2, min(8, int(2**30 // (elems * 4)) + 1))
+    kv = []
+    for r in range(n_rot):
+        kb, vb = DeviceBuffer(elems * 2), DeviceBuffer(elems * 2)
+        _rand_fill(kb, elems * 2, 2 * r)
+        _rand_fill(vb, elems * 2, 2 * r + 1)
+        kv.append((kb, vb))
+    q = DeviceBuffer.from_numpy(np.random.default_rng(9).standard_normal((B, Hq, D)).astype(np.float16))
+    out = DeviceBuffer(B * Hq * D * 2)
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
+    ws = DeviceBuffer(max(wsb, 256))
+    dl = DeviceBuffer.from_numpy(np.asarray(lens, np.int32)) if lens is not None else None
+    state = {"i": 0}
+
+    def step():
+        kb, vb = kv[state["i"] % n_rot]
+        state["i"] += 1
+        check(lib.axhip_gqa_decode(q.ptr, kb.ptr, vb.ptr, dl.ptr if dl else None, out.ptr, ws.ptr, wsb, F16, B,
+                                   Hq, Hkv, D, L, Hkv * L * D, L * D, D, None), "gqa_decode")
+
+    us = _time(lib, step, steps)
+    L_sum = int(np.sum(lens)) if lens is not None else B * L
+    nbytes = 2 * Hkv * D * 2 * L_sum + 2 * Hq * D * 2 * B
+    s, c = C.c_int(0), C.c_int(0)
+    lib.axhip_gqa_decode_plan(B, Hq, Hkv, L, C.byref(s), C.byref(c))
+    gbs = nbytes / us / 1e3
+    _emit({"op": tag, "B": B, "L": L, "ragged": lens is not None, "us": round(us, 2), "bytes": nbytes,
+           "GBps": round(gbs, 1), "pct_hbm_peak": round(100 * gbs / HBM_PEAK, 1), "splits": s.value,
+           "chunk": c.value, "kv_buffers": n_rot})
+    return us
+
+
+def bench_copy(lib, mib, steps):
+    n = mib * 2**20
+    a, b = DeviceBuffer(n), DeviceBuffer(n)
+    _rand_fill(a, n, 1)
+    us = _time(lib, lambda: check(lib.axhip_memcpy_d2d(b.ptr, a.ptr, n), "copy"), steps)
+    gbs = 2 * n / us / 1e3
+    _emit({"op": "copy_bytes_kernel", "bytes_read": n, "bytes_written": n, "us": round(us, 2),
+           "GBps_read_plus_write": round(gbs, 1), "pct_hbm_peak": round(100 * gbs / HBM_PEAK, 1)})
+
+
+def bench_rowops(lib, steps=200):
+    rng = np.random.default_rng(0)
+
+    def h(shape, scale=1.0):
+        return DeviceBuffer.from_numpy((scale * rng.standard_normal(shape)).astype(np.float32).astype(np.float16))
+
+    for rows in (32, 4096, 65536):
+        x, r, w = h((rows, 2048)), h((rows, 2048)), h((2048,))
+        y, o = DeviceBuffer(rows * 4096), DeviceBuffer(rows * 4096)
+        us = _time(lib, lambda: check(lib.axhip_add_rms_norm(x.ptr, r.ptr, w.ptr, 1e-6, y.ptr, o.ptr, F16, F16,
+                                                              rows, 2048, None), "arn"), steps)
+        nb = 4 * rows * 4096 + 4096
+        _emit({"op": "add_rms_norm", "rows": rows, "hidden": 2048, "us": round(us, 2), "bytes": nb,
+               "GBps": round(nb / us / 1e3, 1), "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 2)})
+        g, u = h((rows, 6144)), h((rows, 6144))
+        so = DeviceBuffer(rows * 6144 * 2)
+        us = _time(lib, lambda: check(lib.axhip_silu_mul(g.ptr, u.ptr, so.ptr, F16, rows * 6144, None), "silu"), steps)
+        nb = 3 * rows * 6144 * 2
+        _emit({"op": "silu_mul", "rows": rows, "cols": 6144, "us": round(us, 2), "bytes": nb,
+               "GBps": round(nb / us / 1e3, 1), "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 2)})
+        qx, kx = h((rows, 16, 128)), h((rows, 8, 128))
+        qo, ko = DeviceBuffer(rows * 16 * 256), DeviceBuffer(rows * 8 * 256)
+        pos = DeviceBuffer.from_numpy(rng.integers(0, 8192, rows).astype(np.int64))
+
+        def rope2():
+            check(lib.axhip_rope(qx.ptr, pos.ptr, 1e6, qo.ptr, F16, rows, 16, 128, None), "rope")
+            check(lib.axhip_rope(kx.ptr, pos.ptr, 1e6, ko.ptr, F16, rows, 8, 128, None), "rope")
+
+        us = _time(lib, rope2, steps)
+        nb = 2 * rows * 24 * 128 * 2
+        _emit({"op": "rope q+k (2 launches)", "rows": rows, "us": round(us, 2), "bytes": nb,
+               "GBps": round(nb / us / 1e3, 1), "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 2)})
+    B, Hkv, Lmax, D = 32, 8, 8192, 128
+    kc, vc = DeviceBuffer(B * Hkv * Lmax * D * 2), DeviceBuffer(B * Hkv * Lmax * D * 2)
+    kn, vn = h((B, Hkv, D)), h((B, Hkv, D))
+    pos = DeviceBuffer.from_numpy(rng.integers(0, Lmax, B).astype(np.int64))
+    us = _time(lib, lambda: check(lib.axhip_kv_append(kn.ptr, vn.ptr, kc.ptr, vc.ptr, pos.ptr, I64, 2, B, Hkv, Lmax,
+                                                       D, None), "append"), steps)
+    nb = 4 * B * Hkv * D * 2
+    _emit({"op": "kv_append", "B": B, "us": round(us, 2), "bytes": nb, "GBps": round(nb / us / 1e3, 2),
+           "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 3)})
+
+
+def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512)):
+    rng = np.random.default_rng(0)
+    shapes = shapes or [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 151936)]
+    for K, N in shapes:
+        w_host = (0.02 * rng.standard_normal((min(N, 4096), K))).astype(np.float32).astype(np.float16)
+        # several weight copies are rotated when one is smaller than the Infinity Cache
+        n_rot = max(1, min(8, int(600e6 // (2 * K * N)) + 1))
+        ws_ = []
+        for r in range(n_rot):
+            wb = DeviceBuffer(N * K * 2)
+            off = 0
+            while off < N * K * 2:
+                n = min(w_host.nbytes, N * K * 2 - off)
+                wb.upload(w_host.reshape(-1)[: n // 2], off)
+                off += n
+            ws_.append(wb)
+        for M in Ms:
+            x = DeviceBuffer.from_numpy(rng.standard_normal((M, K)).astype(np.float32).astype(np.float16))
+            out = DeviceBuffer(M * N * 4)
+            wsb = lib.axhip_linear_f16_workspace_bytes(M, K, N)
+            ws = DeviceBuffer(max(wsb, 256))
+            st = {"i": 0}
+
+            def step():
+                wb = ws_[st["i"] % n_rot]
+                st["i"] += 1
+                check(lib.axhip_linear_f16(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, ws.ptr, wsb, None), "linear")
+
+            us = _time(lib, step, steps)
+            nb = 2 * K * N + 2 * M * K + 4 * M * N
+            fl = 2.0 * M * K * N
+            _emit({"op": "linear_f16", "M": M, "K": K, "N": N, "us": round(us, 2), "bytes": nb,
+                   "GBps": round(nb / us / 1e3, 1), "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 1),
+                   "TFLOPs": round(fl / us / 1e6, 1), "pct_mfma_f16_peak": round(100 * fl / us / 1e6 / MFMA_F16_PEAK, 2),
+                   "weight_copies": n_rot})
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "copy", "rowops", "linear"])
+    ap.add_argument("--B", type=int, default=32)
+    ap.add_argument("--L", type=int, default=8192)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--mib", type=int, default=1024)
+    ap.add_argument("--ragged", action="store_true")
+    ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--target-wgs", type=int, default=0)
+    args = ap.parse_args(argv)
+    lib = _lib.load()
+    if _lib.device_count() < 1:
+        sys.exit("no HIP device")
+    if args.what == "gqa":
+        lib.axhip_gqa_decode_tune(args.target_wgs, args.splits)
+        lens = None
+        if args.ragged:
+            lens = np.random.default_rng(0).integers(512, args.L + 1, args.B)
+        bench_gqa(lib, args.B, args.L, args.steps, lens)
+    elif args.what == "gqa-sweep":
+        for B in (1, 8, 32, 64):
+            for L in (1024, 8192, 32768):
+                bench_gqa(lib, B, L, max(10, min(args.steps, int(2e9 // (B * L * 4096)) + 10)))
+        lens = np.random.default_rng(0).integers(512, 32769, 32)
+        bench_gqa(lib, 32, 32768, 20, lens, tag="gqa_ragged_512_32768")
+    elif args.what == "copy":
+        bench_copy(lib, args.mib, args.steps)
+    elif args.what == "rowops":
+        bench_rowops(lib)
+    elif args.what == "linear":
+        bench_linear(lib)
+
+
+if __name__ == "__main__":
+    main()

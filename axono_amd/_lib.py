@@ -27,6 +27,7 @@ PROTOTYPES = {
     "axhip_device_info": (c_i, [c_i, C.c_char_p, c_sz, C.POINTER(c_i), C.POINTER(c_sz), C.POINTER(c_i)]),
     "axhip_alloc": (c_i, [c_sz, c_i, C.POINTER(c_vp)]),
     "axhip_free": (c_i, [c_vp]),
+    "axhip_block_is_capture_owned": (c_i, [c_vp, C.POINTER(c_i)]),
     "axhip_cached_bytes": (c_sz, []),
     "axhip_set_cache_budget": (c_i, [c_sz]),
     "axhip_cache_budget": (c_sz, []),
@@ -73,6 +74,10 @@ PROTOTYPES = {
     "axhip_linear_f16": (c_i, [c_vp, c_i, c_vp, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_vp, c_sz, c_vp]),
     "axhip_embedding": (c_i, [c_vp, c_i, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_vp]),
     "axhip_argmax": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
+    "axhip_qkv_norm_rope_append": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp,
+                                         c_i, c_i, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "axhip_silu_mul_fused": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
+    "axhip_index_add": (c_i, [c_vp, c_i, c_i64, c_i64, c_vp]),
 }
 
 _lib = None

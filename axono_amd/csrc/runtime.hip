@@ -230,6 +230,15 @@ AXHIP_API int axhip_free(void *ptr) {
   return AXHIP_OK;
 }
 
+AXHIP_API int axhip_block_is_capture_owned(const void *ptr, int *owned) {
+  if (!owned) return AXHIP_INVALID_PTR;
+  std::lock_guard<std::mutex> lk(g_mu);
+  auto it = g_live.find(const_cast<void *>(ptr));
+  if (it == g_live.end()) return AXHIP_INVALID_PTR;
+  *owned = it->second.pool_owned ? 1 : 0;
+  return AXHIP_OK;
+}
+
 AXHIP_API size_t axhip_cached_bytes(void) {
   std::lock_guard<std::mutex> lk(g_mu);
   return g_cached_bytes;

@@ -27,7 +27,7 @@ def check(code: int, op: str) -> None:
 class DeviceBuffer:
     """A block of device memory owned by this object (returned to the allocator on release)."""
 
-    __slots__ = ("ptr", "nbytes", "_lib")
+    __slots__ = ("ptr", "nbytes", "_lib", "_owned")
 
     def __init__(self, nbytes: int, zero: bool = False):
         self._lib = _lib.load()
@@ -35,6 +35,12 @@ class DeviceBuffer:
         p = C.c_void_p()
         check(self._lib.axhip_alloc(self.nbytes, 1 if zero else 0, C.byref(p)), "alloc")
         self.ptr = p.value or 0
+        # blocks handed out while a capture pool records or a graph captures belong to the pool /
+        # the graph: this object must never free them (the address may be reused after a reset)
+        owned = C.c_int(0)
+        self._owned = True
+        if self.ptr and self._lib.axhip_block_is_capture_owned(self.ptr, C.byref(owned)) == 0 and owned.value:
+            self._owned = False
 
     @classmethod
     def from_numpy(cls, arr: np.ndarray) -> "DeviceBuffer":
@@ -60,7 +66,8 @@ class DeviceBuffer:
 
     def release(self) -> None:
         if self.ptr:
-            self._lib.axhip_free(self.ptr)
+            if self._owned:
+                self._lib.axhip_free(self.ptr)
             self.ptr = 0
 
     def __del__(self):

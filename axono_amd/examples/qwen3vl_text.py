@@ -1,0 +1,252 @@
+"""Text tower of a Qwen3-VL-shaped decoder on the hip device: batched prefill into a static KV cache
+and a decode step that is captured once into a hipGraph and replayed.
+
+Follows the op sequence of the reference's example model
+(axono/python/examples/vlm/qwen3vl/model.py:308-501 for the layers, :729-761 for decode_step):
+input RMSNorm -> q/k/v projections -> per-head q/k RMSNorm (over head_dim) -> M-RoPE -> KV append ->
+grouped-query attention -> o_proj -> fused add + RMSNorm -> gate/up projections -> SiLU-mul ->
+down_proj -> residual add; final RMSNorm and the tied lm_head; greedy argmax.
+
+What differs from the reference, by design of the captured step: the cache is pre-allocated
+[B, n_kv, max_len, d_head] per layer with lengths on the device; q/k/v and gate/up are fused
+projections (their weights are the row-wise concatenation of the separate matrices); the residual
+add at the end of a layer is folded into the next layer's fused add + RMSNorm; next-token argmax,
+the embedding lookup of that token and the position increment all run on the device, so a step has
+no host <-> device traffic.  Linear weights and the embedding table are FLOAT16; the residual
+stream and every Linear output are FLOAT32, as in the reference's fp16-Linear mode.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+
+import numpy as np
+
+from .. import _lib
+from .. import libaxono as L
+from .. import nn
+from ..core.hip_graph import HIPGraph
+from ..core.tensor import Tensor
+from ..core.types import DataType
+from ..device import check, current_stream
+
+
+@dataclass
+class TextConfig:
+    """Qwen3-VL-2B text tower by default."""
+    num_hidden_layers: int = 28
+    hidden_size: int = 2048
+    num_attention_heads: int = 16
+    num_key_value_heads: int = 8
+    head_dim: int = 128
+    intermediate_size: int = 6144
+    vocab_size: int = 151936
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1e6
+    mrope_section: list = field(default_factory=lambda: [24, 20, 20])
+
+
+def inv_freq_table(theta: float, d_head: int) -> np.ndarray:
+    """1 / theta^(2i/d) in fp32, as the reference builds it (model.py:474-481)."""
+    return (1.0 / (theta ** (np.arange(0, d_head, 2, dtype=np.float32) / d_head))).astype(np.float32)
+
+
+def random_weights(cfg: TextConfig, seed: int = 0) -> dict:
+    """Random-init weights of the architecture: Linear / embedding ~ N(0, 0.02) rounded to fp16, norm
+    weights 1.  Names follow the reference's module tree; q/k/v and gate/up are stored fused."""
+    rng = np.random.default_rng(seed)
+    H, D = cfg.hidden_size, cfg.head_dim
+    nq, nkv, I = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.intermediate_size
+
+    def lin(n, k):
+        return (0.02 * rng.standard_normal((n, k), dtype=np.float32)).astype(np.float16)
+
+    w = {"embed_tokens.weight": lin(cfg.vocab_size, H), "norm.weight": np.ones(H, np.float32)}
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        w[p + "self_attn.qkv_proj.weight"] = lin((nq + 2 * nkv) * D, H)
+        w[p + "self_attn.o_proj.weight"] = lin(H, nq * D)
+        w[p + "self_attn.q_norm.weight"] = np.ones(D, np.float32)
+        w[p + "self_attn.k_norm.weight"] = np.ones(D, np.float32)
+        w[p + "mlp.gate_up_proj.weight"] = lin(2 * I, H)
+        w[p + "mlp.down_proj.weight"] = lin(H, I)
+        w[p + "input_layernorm.weight"] = np.ones(H, np.float32)
+        w[p + "post_attention_layernorm.weight"] = np.ones(H, np.float32)
+    return w
+
+
+def _dev(arr, device):
+    return Tensor.from_numpy_ref(np.ascontiguousarray(arr)).to(device)
+
+
+class Qwen3VLTextDecoder(nn.Module):
+    def __init__(self, cfg: TextConfig, weights: dict, batch: int, max_len: int, device: str = "hip"):
+        super().__init__()
+        self._cfg = cfg
+        self._device = device
+        self._batch = batch
+        self._lib = _lib.load()
+        for name, arr in weights.items():
+            self._parameters[name] = _dev(arr, device)
+        self._inv_freq = _dev(inv_freq_table(cfg.rope_theta, cfg.head_dim), device)
+        self._cache = nn.StaticKVCache(cfg.num_hidden_layers, batch, cfg.num_key_value_heads, max_len, cfg.head_dim,
+                                       DataType.FLOAT16, device)
+        # static state of the captured step
+        self._ids = Tensor(DataType.INT64, [batch], device)
+        self._pos = Tensor(DataType.INT64, [3, batch], device)
+        wsb = self._lib.axhip_gqa_decode_workspace_bytes(batch, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                                         cfg.head_dim, max_len)
+        self._attn_ws = Tensor(DataType.INT8, [max(wsb, 256)], device)
+        self._graph = None
+        self._graph_out = None
+
+    # ---- pieces ----------------------------------------------------------------------------
+    def _w(self, name):
+        return self._parameters[name]
+
+    @property
+    def cache(self) -> nn.StaticKVCache:
+        return self._cache
+
+    def _mlp(self, xn, p):
+        gu = L.linear_nobias(xn, self._w(p + "mlp.gate_up_proj.weight"))
+        return L.linear_nobias(L.silu_mul_fused(gu), self._w(p + "mlp.down_proj.weight"))
+
+    def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None):
+        """One token per sequence.  ids INT64 [B]; pos INT64 [3,B]; appends to the cache at
+        cache.seq_lens and attends over seq_lens + 1 keys.  Returns (logits FLOAT32 [B,V], next ids
+        INT64 [B]).  Does not advance the lengths."""
+        cfg = self._cfg
+        B = self._batch
+        cache = self._cache
+        max_len = attn_max_len or cache.max_len
+        h = L.embedding(ids, self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)  # [B,H]
+        xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps)
+        # lengths that include the token being appended (the kernel reads them on the device)
+        lens_now = self._lens_plus_one
+        for i in range(cfg.num_hidden_layers):
+            p = f"layers.{i}."
+            qkv = L.linear_nobias(xn, self._w(p + "self_attn.qkv_proj.weight"))
+            kc, vc = cache.get(i)
+            q = L.qkv_norm_rope_append(qkv, self._w(p + "self_attn.q_norm.weight"), self._w(p + "self_attn.k_norm.weight"),
+                                       cfg.rms_norm_eps, pos, self._inv_freq, cfg.mrope_section, cache.seq_lens, kc, vc,
+                                       cfg.num_attention_heads)
+            attn = L.gqa_decode_attention_cache(q, kc, vc, lens_now, max_len, workspace=self._attn_ws)
+            attn_out = L.linear_nobias(attn.reshape([B, cfg.num_attention_heads * cfg.head_dim]),
+                                       self._w(p + "self_attn.o_proj.weight"))
+            h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps)
+            mlp_out = self._mlp(xn2, p)
+            nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
+            # h = h + mlp_out folded into the following RMSNorm (next layer's input norm / final norm)
+            h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps)
+        logits = L.linear_nobias(xn, self._w("embed_tokens.weight"))  # tied lm_head
+        return logits, L.argmax(logits)
+
+    # ---- prefill -----------------------------------------------------------------------------
+    def prefill(self, ids: np.ndarray, positions: np.ndarray | None = None):
+        """ids int64 [B, S] (host).  Fills the cache for every sequence (one sequence at a time, all
+        S tokens at once) and returns (last-position logits FLOAT32 [B,V] as a Tensor, next ids [B]).
+        Text-only positions by default: T = H = W = token index."""
+        cfg = self._cfg
+        B, S = ids.shape
+        assert B == self._batch and S <= self._cache.max_len
+        lib, dev = self._lib, self._device
+        H, D, nq, nkv = cfg.hidden_size, cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
+        width = (nq + 2 * nkv) * D
+        lmax = self._cache.max_len
+        if positions is None:
+            positions = np.broadcast_to(np.arange(S, dtype=np.int64), (3, S))
+        pos_t = _dev(np.ascontiguousarray(positions, dtype=np.int64), dev)
+        vis = _dev(np.arange(1, S + 1, dtype=np.int32), dev)  # causal: row t sees t+1 keys
+        wsb = lib.axhip_gqa_decode_workspace_bytes(S, nq, nkv, D, S)
+        ws = Tensor(DataType.INT8, [max(wsb, 256)], dev, _zero=False)
+        last_h = Tensor(DataType.FLOAT32, [B, H], dev)
+        esz = 2
+        for b in range(B):
+            h = L.embedding(_dev(ids[b].astype(np.int64), dev), self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)
+            xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps)
+            for i in range(cfg.num_hidden_layers):
+                p = f"layers.{i}."
+                qkv = L.linear_nobias(xn, self._w(p + "self_attn.qkv_proj.weight"))  # [S, width] fp32
+                kc, vc = self._cache.get(i)
+                seq_off = b * nkv * lmax * D * esz
+                q = Tensor(DataType.FLOAT16, [S, nq, D], dev, _zero=False)
+                base = qkv.data_ptr
+                check(lib.axhip_qkv_norm_rope_append(
+                    base, width, base + nq * D * 4, width, base + (nq + nkv) * D * 4, width,
+                    self._w(p + "self_attn.q_norm.weight").data_ptr, self._w(p + "self_attn.k_norm.weight").data_ptr,
+                    int(DataType.FLOAT32), cfg.rms_norm_eps, pos_t.data_ptr, self._inv_freq.data_ptr,
+                    cfg.mrope_section[1], cfg.mrope_section[2], None, q.data_ptr, kc.data_ptr + seq_off,
+                    vc.data_ptr + seq_off, int(DataType.FLOAT16), 1, S, nq, nkv, D, lmax, current_stream()),
+                    "qkv_norm_rope_append")
+                attn = Tensor(DataType.FLOAT16, [S, nq * D], dev, _zero=False)
+                # every query row is a "sequence" of the decode kernel over this sequence's cache rows
+                check(lib.axhip_gqa_decode(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, vis.data_ptr,
+                                           attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq, nkv,
+                                           D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
+                attn_out = L.linear_nobias(attn, self._w(p + "self_attn.o_proj.weight"))
+                h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps)
+                mlp_out = self._mlp(xn2, p)
+                nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
+                h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps)
+            # keep the normalised hidden state of the last position for the lm_head
+            check(lib.axhip_memcpy_d2d(last_h.data_ptr + b * H * 4, xn.data_ptr + (S - 1) * H * 4, H * 4), "copy")
+        self._cache.set_lengths(np.full(B, S, np.int32))
+        logits = L.linear_nobias(last_h, self._w("embed_tokens.weight"))
+        return logits, L.argmax(logits)
+
+    # ---- captured decode loop ------------------------------------------------------------------
+    def start_decode(self, first_ids: np.ndarray, first_pos: np.ndarray, max_new_tokens: int):
+        """Sets the static step inputs (ids [B], positions [3,B]) and captures the step.  The
+        attention split plan is sized for the lengths the loop will reach."""
+        B = self._batch
+        self._ids.copy_from_numpy(np.ascontiguousarray(first_ids, dtype=np.int64).reshape(B))
+        self._pos.copy_from_numpy(np.ascontiguousarray(first_pos, dtype=np.int64).reshape(3, B))
+        bound = min(self._cache.max_len, len(self._cache) + max_new_tokens + 1)
+        self._lens_plus_one = Tensor(DataType.INT32, [B], self._device)
+
+        def step():
+            # lens_plus_one = seq_lens + 1 (keys visible to this step's query, incl. the new token)
+            check(self._lib.axhip_memcpy_d2d(self._lens_plus_one.data_ptr, self._cache.seq_lens.data_ptr, 4 * B), "copy")
+            L.index_add(self._lens_plus_one, 1)
+            logits, nxt = self.decode_forward(self._ids, self._pos, bound)
+            # feed the device-side state of the next step
+            check(self._lib.axhip_memcpy_d2d(self._ids.data_ptr, nxt.data_ptr, 8 * B), "copy")
+            L.index_add(self._pos, 1)
+            L.index_add(self._cache.seq_lens, 1)
+            return logits, nxt
+
+        self._step_fn = step
+        return step
+
+    def capture(self):
+        """Captures one decode step (after a warm-up run) and rewinds the state both runs advanced."""
+        B = self._batch
+        ids0 = self._ids.numpy().copy()
+        pos0 = self._pos.numpy().copy()
+        lens0 = self._cache.seq_lens.numpy().copy()
+        g = HIPGraph()
+        g.capture(self._step_fn)  # runs the step twice (warm-up + recorded run): cache rows get the same values
+        self._ids.copy_from_numpy(ids0)
+        self._pos.copy_from_numpy(pos0)
+        self._cache.seq_lens.copy_from_numpy(lens0)
+        self._graph = g
+        self._graph_out = g.outputs
+        return g
+
+    def generate(self, max_new_tokens: int, use_graph: bool = True):
+        """Greedy decode loop.  Returns int64 [steps, B] of generated ids.  The tokens of every step
+        are gathered on the device and read back once at the end."""
+        B = self._batch
+        tokens = Tensor(DataType.INT64, [max_new_tokens, B], self._device)
+        lib = self._lib
+        for s in range(max_new_tokens):
+            if use_graph:
+                self._graph.launch()
+                nxt = self._graph_out[1]
+            else:
+                _, nxt = self._step_fn()
+            check(lib.axhip_memcpy_d2d(tokens.data_ptr + s * 8 * B, nxt.data_ptr, 8 * B), "copy")
+        L.synchronize()
+        self._cache._host_len += max_new_tokens
+        return tokens.numpy()

@@ -1,0 +1,5 @@
+from .kv_cache import DynamicKVCache, KVCache, StaticKVCache
+from .layers import Embedding, Linear, RMSNorm
+from .module import Module
+
+__all__ = ["Module", "Linear", "RMSNorm", "Embedding", "KVCache", "DynamicKVCache", "StaticKVCache"]

@@ -76,6 +76,11 @@ AXHIP_API int axhip_device_info(int device_id, char *name, size_t name_len, int 
  * call follows the capture pool instead (see axhip_capture_pool_*). */
 AXHIP_API int axhip_alloc(size_t bytes, int zero, void **out);
 AXHIP_API int axhip_free(void *ptr);
+/* Whether a live block belongs to the capture pool or to a captured graph (then axhip_free on it
+ * is a no-op and the block is released by axhip_capture_pool_reset / axhip_graph_destroy; a holder
+ * must not free it after that).  The reference expresses the same with a no-op deleter,
+ * detail.cu:196-199,262-264. */
+AXHIP_API int axhip_block_is_capture_owned(const void *ptr, int *owned);
 /* cached_bytes() / set_cache_budget(bytes), nanobind_module.cpp:398-400 */
 AXHIP_API size_t axhip_cached_bytes(void);
 AXHIP_API int axhip_set_cache_budget(size_t bytes);
@@ -294,6 +299,38 @@ AXHIP_API int axhip_embedding(const void *ids, int ids_dtype, const void *table,
  * Replaces ops::cuda::ArgmaxLastDim, src/ops/cuda/sequence.cu:262-292. */
 AXHIP_API int axhip_argmax(const void *x, int64_t *out, int dtype, int64_t rows, int64_t cols,
                            axhip_stream stream);
+
+/* ============================================================================================
+ * Glue kernels of the captured decode step (fusions of the operators above)
+ * ========================================================================================== */
+
+/* For every token r (B sequences of S consecutive tokens each, r = b*S + t; S = 1 in a decode
+ * step, S = prompt length in prefill) and head: q heads -> rms_norm over D (weight q_weight) ->
+ * M-RoPE -> stored as `cache_dtype` into q_out [B*S,Hq,D]; k heads -> rms_norm (k_weight) -> M-RoPE
+ * -> written to k_cache[b, hk, seq_lens[b] + t, :]; v heads -> converted and written to
+ * v_cache[b, hk, seq_lens[b] + t, :].  seq_lens may be NULL (append from position 0).
+ * Equals rms_norm + rope_thd + cast + kv_append applied in that order (the reference's sequence,
+ * examples/vlm/qwen3vl/model.py:353-364), with one rounding at the store.  q, k, v are fp32 rows of
+ * the projection output with the given row strides (elements), so a fused QKV projection can be
+ * passed as three offsets into one buffer.  pos int64 [3,B*S]; inv_freq fp32 [D/2]; seq_lens int32 [B]
+ * (an append position outside [0,Lmax) is skipped).  Norm weights may be NULL. */
+AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const float *k,
+                                         int64_t k_stride, const float *v, int64_t v_stride,
+                                         const void *q_weight, const void *k_weight, int w_dtype,
+                                         float eps, const int64_t *pos, const float *inv_freq,
+                                         int h_sec, int w_sec, const int32_t *seq_lens, void *q_out,
+                                         void *k_cache, void *v_cache, int cache_dtype, int B, int S,
+                                         int Hq, int Hkv, int D, int Lmax, axhip_stream stream);
+
+/* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
+ * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0. */
+AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int64_t rows, int64_t cols,
+                                   axhip_stream stream);
+
+/* x[i] += delta in place for INT32 / INT64 device arrays (sequence lengths and positions that a
+ * captured decode step advances on the device; the reference rebuilds them on the host each step,
+ * examples/vlm/qwen3vl/model.py:739-748). */
+AXHIP_API int axhip_index_add(void *x, int dtype, int64_t n, int64_t delta, axhip_stream stream);
 
 #ifdef __cplusplus
 }

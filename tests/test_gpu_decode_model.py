@@ -1,0 +1,93 @@
+"""The decode-step module (prefill + captured decode step) on a small text-tower configuration
+against the CPU restatement of the same op sequence (oracle/decode_step.py).
+
+Logits are FLOAT32; tolerance 2e-3 absolute (fp16 data formats inside the step: weights, the
+activation entering each Linear, q and the KV cache)."""
+import numpy as np
+import pytest
+
+from axono_amd.examples.qwen3vl_text import Qwen3VLTextDecoder, TextConfig, random_weights
+from oracle.decode_step import OracleDecoder
+
+pytestmark = pytest.mark.gpu
+
+CFG = TextConfig(num_hidden_layers=3, hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+                 intermediate_size=512, vocab_size=1000)
+
+
+def _setup(B=3, S=21, max_len=64, seed=0):
+    w = random_weights(CFG, seed)
+    # non-trivial norm weights so a dropped weight would show
+    rng = np.random.default_rng(seed + 1)
+    for k in w:
+        if k.endswith("norm.weight") or k.endswith("layernorm.weight"):
+            w[k] = (1 + 0.1 * rng.standard_normal(w[k].shape)).astype(np.float32)
+    gpu = Qwen3VLTextDecoder(CFG, w, B, max_len, "hip:0")
+    cpu = OracleDecoder(CFG, w, B, max_len)
+    ids = rng.integers(0, CFG.vocab_size, (B, S)).astype(np.int64)
+    return gpu, cpu, ids
+
+
+def test_prefill_logits_and_cache():
+    gpu, cpu, ids = _setup()
+    g_logits, g_next = gpu.prefill(ids)
+    c_logits, c_next = cpu.prefill(ids)
+    err = np.abs(g_logits.to_numpy() - c_logits).max()
+    assert err <= 2e-3, err
+    S = ids.shape[1]
+    for i in range(CFG.num_hidden_layers):
+        kc, vc = gpu.cache.get(i)
+        assert np.abs(kc.numpy()[:, :, :S].astype(np.float32) - cpu.k[i][:, :, :S].astype(np.float32)).max() <= 4e-3
+        assert np.abs(vc.numpy()[:, :, :S].astype(np.float32) - cpu.v[i][:, :, :S].astype(np.float32)).max() <= 4e-3
+        assert np.all(kc.numpy()[:, :, S:] == 0)
+    np.testing.assert_array_equal(gpu.cache.seq_lens.to_numpy(), [S] * ids.shape[0])
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_decode_steps_match_oracle(use_graph):
+    gpu, cpu, ids = _setup(seed=3)
+    B, S = ids.shape
+    _, g_next = gpu.prefill(ids)
+    _, c_next = cpu.prefill(ids)
+    first = g_next.to_numpy()
+    pos = np.full((3, B), S, np.int64)  # text-only: position = index of the token being decoded
+    n_steps = 6
+    gpu.start_decode(first, pos, n_steps)
+    if use_graph:
+        g = gpu.capture()
+        assert g.num_nodes > 10
+    toks = gpu.generate(n_steps, use_graph=use_graph)
+    # the oracle follows the GPU's token choices so that one near-tie cannot derail the comparison
+    cur = first
+    for s in range(n_steps):
+        logits, nxt = cpu.decode_step(cur, pos + s)
+        # the GPU token must be (within tolerance) a maximiser of the oracle's logits
+        chosen = logits[np.arange(B), toks[s]]
+        assert np.all(chosen >= logits.max(-1) - 4e-3), (s, chosen, logits.max(-1))
+        cur = toks[s]
+    np.testing.assert_array_equal(gpu.cache.seq_lens.to_numpy(), [S + n_steps] * B)
+    # cache rows written by the decode steps
+    for i in range(CFG.num_hidden_layers):
+        kc = gpu.cache.get(i)[0].numpy()[:, :, S:S + n_steps].astype(np.float32)
+        assert np.abs(kc - cpu.k[i][:, :, S:S + n_steps].astype(np.float32)).max() <= 4e-3
+
+
+def test_eager_and_graph_logits_agree_every_replay():
+    """Each replay is checked against an eager run of the same step from the same state."""
+    gpu, _, ids = _setup(seed=7)
+    B, S = ids.shape
+    _, nxt = gpu.prefill(ids)
+    first = nxt.to_numpy()
+    pos = np.full((3, B), S, np.int64)
+    gpu.start_decode(first, pos, 8)
+    gpu.capture()
+    for s in range(4):
+        state = (gpu._ids.numpy().copy(), gpu._pos.numpy().copy(), gpu.cache.seq_lens.numpy().copy())
+        e_logits, e_next = gpu._step_fn()
+        e_logits, e_next = e_logits.to_numpy().copy(), e_next.to_numpy().copy()
+        gpu._ids.copy_from_numpy(state[0])
+        gpu._pos.copy_from_numpy(state[1])
+        gpu.cache.seq_lens.copy_from_numpy(state[2])
+        gpu._graph.replay()
+        np.testing.assert_array_equal(gpu._graph_out[0].to_numpy(), e_logits)
+        np.testing.assert_array_equal(gpu._graph_out[1].to_numpy(), e_next)

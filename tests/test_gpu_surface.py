@@ -1,0 +1,319 @@
+"""The Python surface on the hip device: the reference's own test cases for the decode path,
+re-stated (tests/core/test_fused.py, test_gqa.py, test_sequence_ops.py, test_fp16.py,
+test_cuda_graph.py, tests/nn/test_kv_cache.py of the reference), plus compile() and the allocator.
+Expected values come from the CPU oracle / NumPy closed forms."""
+import math
+
+import numpy as np
+import pytest
+
+import axono_amd as axono
+from axono_amd import DataType, Tensor, nn
+from axono_amd import libaxono as L
+from oracle import port
+
+pytestmark = pytest.mark.gpu
+
+DEV = "hip:0"
+
+
+def t(arr, device=DEV):
+    return Tensor.from_numpy(np.ascontiguousarray(arr)).to(device)
+
+
+def ids_t(arr, device=DEV):
+    x = Tensor.zeros(tuple(np.asarray(arr).shape), dtype=DataType.INT64, device=device)
+    x.copy_from_numpy(np.asarray(arr, dtype=np.int64))
+    return x
+
+
+@pytest.fixture
+def hip_env():
+    axono.set_backend("hip")
+    yield
+    axono.set_backend("cpu")
+
+
+def test_tensor_device_round_trip_and_zero_init(hip_env):
+    assert axono.hip_available()
+    z = Tensor(DataType.FLOAT32, [3, 5], "hip:0")
+    assert np.all(z.to_numpy() == 0) and z.is_hip and not z.is_cuda
+    x = np.random.default_rng(0).standard_normal((4, 7)).astype(np.float32)
+    d = Tensor.from_numpy(x)  # default device is hip inside hip_env
+    assert d.device == "hip"
+    np.testing.assert_array_equal(d.to_numpy(), x)
+    assert d.to("hip") is d and d.to("hip:0") is d
+    back = d.to("cpu")
+    assert back is not d and back.device == "cpu"
+    np.testing.assert_array_equal(back.to_numpy(), x)
+    h = d.cast_to(DataType.FLOAT16)
+    np.testing.assert_array_equal(h.numpy(), x.astype(np.float16))
+    np.testing.assert_array_equal(h.cast_to(DataType.FLOAT32).to_numpy(), x.astype(np.float16).astype(np.float32))
+    d.copy_from_numpy(2 * x)
+    np.testing.assert_array_equal(d.to_numpy(), 2 * x)
+    d.fill_zero()
+    assert np.all(d.to_numpy() == 0)
+    with pytest.raises(IndexError):
+        Tensor(DataType.FLOAT32, [1], "hip:7")
+
+
+def test_fused_ops_reference_cases():
+    rs = np.random.RandomState(0)
+    g, u = rs.randn(37, 53).astype(np.float32), rs.randn(37, 53).astype(np.float32)
+    y = axono.fused.silu_mul(t(g), t(u)).to_numpy()
+    np.testing.assert_allclose(y, g / (1.0 + np.exp(-g)) * u, rtol=1e-5, atol=1e-6)
+    e = np.array([-10.0, -1.0, 0.0, 1.0, 10.0, 0, 0, 0], np.float32)
+    np.testing.assert_allclose(axono.silu_mul(t(e), t(np.ones(8, np.float32))).to_numpy(), e / (1.0 + np.exp(-e)), rtol=1e-5, atol=1e-6)
+    rs = np.random.RandomState(1)
+    x, r, w = rs.randn(4, 128).astype(np.float32), rs.randn(4, 128).astype(np.float32), rs.randn(128).astype(np.float32)
+    yt, out = axono.fused.add_rms_norm(t(x), t(r), t(w), 1e-6)
+    s = x + r
+    np.testing.assert_allclose(yt.to_numpy(), s, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(out.to_numpy(), s / np.sqrt((s ** 2).mean(-1, keepdims=True) + 1e-6) * w, rtol=1e-4, atol=1e-5)
+    # y feeds the next layer's residual
+    rs = np.random.RandomState(2)
+    h, a1, a2 = (rs.randn(2, 64).astype(np.float32) for _ in range(3))
+    w1 = np.ones(64, np.float32)
+    h1, _ = axono.add_rms_norm(t(a1), t(h), t(w1), 1e-6)
+    h2, _ = axono.add_rms_norm(t(a2), h1, t(w1), 1e-6)
+    np.testing.assert_allclose(h2.to_numpy(), a2 + a1 + h, rtol=1e-5, atol=1e-6)
+    with pytest.raises(RuntimeError) as ei:
+        axono.silu_mul(t(g), t(u[:5]))
+    assert "silu_mul 失败, 错误代码: 4" in str(ei.value)
+
+
+def test_gqa_matches_numpy_and_sdpa_op():
+    rs = np.random.RandomState(3)
+    for skv in (1, 7, 256, 512, 1024, 3000):
+        q = rs.randn(1, 16, 128).astype(np.float32)
+        k = rs.randn(skv, 8, 128).astype(np.float32)
+        v = rs.randn(skv, 8, 128).astype(np.float32)
+        out = axono.gqa_decode_attention(t(q), t(k), t(v))
+        assert out.shape == [1, 16, 128]
+        np.testing.assert_allclose(out.to_numpy(), port.gqa_decode(q, k, v), rtol=1e-4, atol=1e-4)
+    rs = np.random.RandomState(4)
+    q, k, v = rs.randn(1, 16, 128).astype(np.float32), rs.randn(300, 8, 128).astype(np.float32), rs.randn(300, 8, 128).astype(np.float32)
+    a1 = axono.gqa_decode_attention(t(q), t(k), t(v)).to_numpy()
+    a2 = axono.scaled_dot_product_attention(t(q), t(k), t(v), False).to_numpy()
+    np.testing.assert_allclose(a1, a2, rtol=1e-4, atol=1e-4)
+    with pytest.raises(RuntimeError) as ei:
+        axono.gqa_decode_attention(t(np.zeros((2, 16, 128), np.float32)), t(k), t(v))
+    assert "错误代码: 1" in str(ei.value)  # decode takes exactly one query token
+
+
+def test_sequence_ops_reference_cases():
+    rs = np.random.RandomState(2027)
+    x = rs.randn(4, 2, 8).astype(np.float32)
+    out = axono.rope(t(x), ids_t(np.arange(4)), 10000.0).to_numpy()
+    np.testing.assert_allclose(out, port.rope(x, np.arange(4), 10000.0), rtol=1e-4, atol=1e-5)
+    rng = np.random.default_rng(8)
+    pos3 = rng.integers(0, 50, size=(3, 17)).astype(np.int64)
+    inv = (1.0 / (5e6 ** (np.arange(0, 128, 2, dtype=np.float32) / 128))).astype(np.float32)
+    c, s = axono.mrope_cos_sin(ids_t(pos3), t(inv), 20, 20)
+    wc, ws = port.mrope_cos_sin(pos3, inv, 20, 20)
+    np.testing.assert_allclose(c.to_numpy(), wc, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(s.to_numpy(), ws, rtol=1e-5, atol=1e-6)
+    xr = rng.standard_normal((17, 4, 128)).astype(np.float32)
+    np.testing.assert_allclose(axono.rope_thd(t(xr), ids_t(pos3), t(inv), [24, 20, 20]).to_numpy(),
+                               port.rope_thd(xr, pos3, inv, [24, 20, 20]), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(axono.rope_with_cos_sin(t(xr), c, s).to_numpy(), port.rope_with_cos_sin(xr, wc, ws), rtol=1e-5, atol=1e-5)
+    a, b = rng.standard_normal((2, 3, 4)).astype(np.float32), rng.standard_normal((2, 3, 5)).astype(np.float32)
+    np.testing.assert_array_equal(axono.concat(t(a), t(b), -1).to_numpy(), np.concatenate([a, b], -1))
+    np.testing.assert_array_equal(axono.concat(t(a), t(a), 0).to_numpy(), np.concatenate([a, a], 0))
+    np.testing.assert_array_equal(axono.slice_(t(b), -1, 1, 3).to_numpy(), b[..., 1:4])
+    np.testing.assert_array_equal(axono.slice_(t(b), 0, 1, 1).to_numpy(), b[1:2])
+    table = rng.standard_normal((10, 4)).astype(np.float32)
+    ids = np.array([[1, 3], [5, 2]], np.int64)
+    np.testing.assert_array_equal(axono.embedding(ids_t(ids), t(table)).to_numpy(), table[ids])
+    lg = rng.standard_normal((3, 100)).astype(np.float32)
+    am = axono.argmax(t(lg))
+    assert am.dtype == DataType.INT64
+    np.testing.assert_array_equal(am.to_numpy(), np.argmax(lg, -1))
+    np.testing.assert_array_equal(axono.add(t(a), t(a)).to_numpy(), a + a)
+    w = rng.standard_normal(5).astype(np.float32)
+    np.testing.assert_allclose(axono.rms_norm(t(b), t(w), 1e-6).to_numpy(), port.rms_norm(b, w, 1e-6), rtol=1e-5, atol=1e-5)
+
+
+def test_linear_fp16_module_path(hip_env):
+    """tests/core/test_fp16.py:28-46 of the reference: nn.Linear after cast_linear_fp16()."""
+    rng = np.random.default_rng(1)
+    x_np = rng.normal(size=(8, 64)).astype(np.float32)
+    w_np = (rng.normal(size=(32, 64)) * 0.05).astype(np.float32)
+    b_np = (rng.normal(size=(32,)) * 0.05).astype(np.float32)
+    lin = nn.Linear(64, 32, device="hip")
+    lin.load_state_dict({"weight": w_np, "bias": b_np})
+    lin.cast_linear_fp16()
+    assert lin.weight.dtype == DataType.FLOAT16 and lin.weight.is_hip
+    out = lin(Tensor.from_numpy(x_np))
+    assert out.dtype == DataType.FLOAT32 and out.shape == [8, 32]
+    np.testing.assert_allclose(out.to_numpy(), x_np @ w_np.T + b_np, rtol=5e-2, atol=5e-2)
+    want = port.linear(x_np.astype(np.float16).astype(np.float32), w_np.astype(np.float16).astype(np.float32),
+                       b_np.astype(np.float16).astype(np.float32))
+    np.testing.assert_allclose(out.to_numpy(), want, rtol=0, atol=2e-5)
+    nb = nn.Linear(64, 32, bias=False, device="hip")
+    nb.load_state_dict({"weight": w_np})
+    nb.cast_linear_fp16()
+    np.testing.assert_allclose(nb(Tensor.from_numpy(x_np)).to_numpy(), want - b_np.astype(np.float16).astype(np.float32), rtol=0, atol=2e-5)
+
+
+def _np_attention(q, k, v, causal):
+    sq, hq, d = q.shape
+    skv, hkv = k.shape[:2]
+    out = np.zeros((sq, hq, d), np.float32)
+    for i in range(sq):
+        for h in range(hq):
+            end = min(i + 1, skv) if causal else skv
+            s = q[i, h] @ k[:end, h // (hq // hkv)].T / math.sqrt(d)
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            out[i, h] = p @ v[:end, h // (hq // hkv)]
+    return out
+
+
+def test_dynamic_kv_cache_with_attention():
+    """tests/nn/test_kv_cache.py of the reference: append / len / reset, and decode with the cache
+    equals the causal full forward."""
+    rng = np.random.default_rng(0)
+    cache = nn.DynamicKVCache(2, device=DEV)
+    k1 = rng.standard_normal((5, 2, 8)).astype(np.float32)
+    k2 = rng.standard_normal((1, 2, 8)).astype(np.float32)
+    cache.update(0, t(k1), t(k1))
+    assert len(cache) == 5
+    cache.update(0, t(k2), t(k2))
+    assert len(cache) == 6
+    np.testing.assert_allclose(cache.get(0)[0].to_numpy(), np.concatenate([k1, k2], 0), rtol=1e-6)
+    cache.reset()
+    assert len(cache) == 0
+    sq, hq, hkv, d = 6, 4, 2, 64
+    q, k, v = (rng.standard_normal(s).astype(np.float32) for s in ((sq, hq, d), (sq, hkv, d), (sq, hkv, d)))
+    full = axono.scaled_dot_product_attention(t(q), t(k), t(v), True).to_numpy()
+    np.testing.assert_allclose(full, _np_attention(q, k, v, True), rtol=1e-4, atol=1e-5)
+    cache = nn.DynamicKVCache(1, device=DEV)
+    for i in range(sq):
+        cache.update(0, t(k[i:i + 1]), t(v[i:i + 1]))
+        kk, vv = cache.get(0)
+        step = axono.gqa_decode_attention(t(q[i:i + 1]), kk, vv) if i > 0 else axono.scaled_dot_product_attention(t(q[i:i + 1]), kk, vv, False)
+        np.testing.assert_allclose(step.to_numpy()[0], full[i], rtol=1e-4, atol=1e-5)
+
+
+def test_static_kv_cache_matches_dynamic():
+    rng = np.random.default_rng(5)
+    B, hkv, d, lmax = 3, 2, 64, 16
+    st = nn.StaticKVCache(1, B, hkv, lmax, d, DataType.FLOAT16, DEV)
+    dyn = [nn.DynamicKVCache(1, device=DEV) for _ in range(B)]
+    for step in range(5):
+        kn = rng.standard_normal((B, hkv, d)).astype(np.float16)
+        vn = rng.standard_normal((B, hkv, d)).astype(np.float16)
+        st.update(0, t(kn), t(vn))
+        st.advance()
+        for b in range(B):
+            dyn[b].update(0, t(kn[b:b + 1]), t(vn[b:b + 1]))
+    assert len(st) == 5
+    np.testing.assert_array_equal(st.seq_lens.to_numpy(), [5, 5, 5])
+    kc = st.get(0)[0].numpy()
+    for b in range(B):
+        np.testing.assert_array_equal(np.transpose(kc[b, :, :5], (1, 0, 2)).view(np.uint16), dyn[b].get(0)[0].numpy().view(np.uint16))
+    assert np.all(kc[:, :, 5:] == 0)
+
+
+def test_graph_capture_replay_semantics():
+    """tests/core/test_cuda_graph.py of the reference: replay is idempotent, an in-place input update
+    is visible after replay, temporaries inside the body are fine, replay before capture raises, an
+    empty capture raises, reset allows a new capture."""
+    rng = np.random.default_rng(0)
+    a = t(rng.standard_normal((8, 256)).astype(np.float32))
+    b = t(rng.standard_normal((8, 256)).astype(np.float32))
+    w = t(np.ones(256, np.float32))
+
+    def body():
+        s = axono.add(a, b)                      # a temporary
+        y, o = axono.add_rms_norm(s, a, w, 1e-6)
+        return axono.silu_mul(o, y), y
+
+    eager = [x.to_numpy().copy() for x in body()]
+    g = axono.HIPGraph()
+    with pytest.raises(RuntimeError):
+        g.replay()
+    g.capture(body)
+    assert g.is_captured and g.num_nodes >= 3
+    for _ in range(3):  # several replays, each checked against the eager result
+        g.replay()
+        L.synchronize()
+        for got, want in zip(g.outputs, eager):
+            np.testing.assert_allclose(got.to_numpy(), want, rtol=1e-6, atol=1e-6)
+    a_new = rng.standard_normal((8, 256)).astype(np.float32)
+    a.copy_from_numpy(a_new)  # refresh the static input in place
+    g.replay()
+    eager2 = [x.to_numpy().copy() for x in body()]
+    for got, want in zip(g.outputs, eager2):
+        np.testing.assert_allclose(got.to_numpy(), want, rtol=1e-6, atol=1e-6)
+    assert g.output is g.outputs[0]
+    g.reset()
+    assert not g.is_captured
+    g.capture(lambda: axono.add(a, b))
+    g.replay()
+    np.testing.assert_allclose(g.output.to_numpy(), a_new + b.to_numpy(), rtol=1e-6)
+    g.reset()
+    with pytest.raises(RuntimeError):
+        axono.HIPGraph().capture(lambda: None)  # nothing captured
+    # context-manager form: the block is captured as it runs
+    with axono.hip_graph() as g2:
+        y = axono.add(a, b)
+        g2.output = y
+    a.copy_from_numpy(np.zeros((8, 256), np.float32))
+    g2.replay()
+    np.testing.assert_allclose(g2.output.to_numpy(), b.to_numpy(), rtol=1e-6)
+    # a failing body aborts the capture and leaves the library usable
+    with pytest.raises(ZeroDivisionError):
+        axono.HIPGraph().capture(lambda: 1 / 0)
+    assert L._lib_().axhip_is_capturing() == 0
+    np.testing.assert_allclose(axono.add(a, b).to_numpy(), b.to_numpy(), rtol=1e-6)
+
+
+def test_compile_caches_by_signature_and_refreshes_inputs():
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w = t(np.linspace(0.5, 1.5, 128).astype(np.float32))
+
+        def forward(self, x, res):
+            y, o = axono.add_rms_norm(x, res, self.w, 1e-6)
+            return axono.silu_mul(o, y)
+
+    m = Block()
+    cm = axono.compile(m)
+    rng = np.random.default_rng(2)
+    for trial in range(3):
+        x, r = rng.standard_normal((4, 128)).astype(np.float32), rng.standard_normal((4, 128)).astype(np.float32)
+        got = cm(t(x), t(r)).to_numpy().copy()
+        want = m(t(x), t(r)).to_numpy()
+        np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+    assert len(cm._graphs) == 1
+    x8 = rng.standard_normal((8, 128)).astype(np.float32)
+    np.testing.assert_allclose(cm(t(x8), t(x8)).to_numpy(), m(t(x8), t(x8)).to_numpy(), rtol=1e-6, atol=1e-6)
+    assert len(cm._graphs) == 2 and "graphs=2" in repr(cm)
+    assert cm.w is m.w  # attribute access passes through to the model
+
+
+def test_allocator_cache_and_budget():
+    L.synchronize()
+    L.empty_cache()
+    base = L.cached_bytes()
+    assert base == 0
+    x = Tensor(DataType.FLOAT32, [1 << 20], DEV)  # 4 MiB
+    p = x.data_ptr
+    assert np.all(x.to_numpy() == 0)
+    x.copy_from_numpy(np.ones(1 << 20, np.float32))
+    del x
+    assert L.cached_bytes() == 4 << 20            # released blocks stay cached
+    y = Tensor(DataType.FLOAT32, [1 << 20], DEV)
+    assert y.data_ptr == p                         # same-size request reuses the cached block
+    assert np.all(y.to_numpy() == 0)               # and a new tensor still reads as zeros
+    assert L.cached_bytes() == 0
+    del y
+    L.set_cache_budget(1 << 20)                    # smaller than the block: evicted on release
+    assert L.cached_bytes() == 0
+    z = Tensor(DataType.FLOAT32, [1 << 20], DEV)
+    del z
+    assert L.cached_bytes() <= 1 << 20
+    L.set_cache_budget(64 << 30)

@@ -147,6 +147,45 @@ def cpu_baseline_gqa(budget_s=12.0):
                       f"min of {n} runs, fp32 arithmetic on fp16-rounded data; bytes counted as fp16"}
 
 
+def cpu_decode_step_hook(cfg, weights, model, first, pos, batch, max_len, log):
+    """One decode step of the CPU restatement from the post-prefill cache, timed, and compared with
+    the device's eager step from the same state."""
+    from oracle.decode_step import OracleDecoder
+    import oracle
+
+    cpu = OracleDecoder(cfg, weights, batch, max_len)
+    ctx = int(model.cache.seq_lens.to_numpy()[0])
+    for i in range(cfg.num_hidden_layers):
+        kc, vc = model.cache.get(i)
+        cpu.k[i][:] = kc.numpy()
+        cpu.v[i][:] = vc.numpy()
+    cpu.lens[:] = ctx
+    # device: one eager step, then rewind
+    state = (model._ids.numpy().copy(), model._pos.numpy().copy(), model.cache.seq_lens.numpy().copy())
+    g_logits, g_next = model._step_fn()
+    g_logits, g_next = g_logits.to_numpy().copy(), g_next.to_numpy().copy()
+    model._ids.copy_from_numpy(state[0])
+    model._pos.copy_from_numpy(state[1])
+    model.cache.seq_lens.copy_from_numpy(state[2])
+    for name in list(weights):  # widen the weights outside the timed region
+        if weights[name].dtype == np.float16:
+            cpu.W(name)
+    t0 = time.perf_counter()
+    c_logits, c_next = cpu.decode_step(first, pos)
+    cpu_s = time.perf_counter() - t0
+    err = float(np.abs(g_logits - c_logits).max())
+    chosen = c_logits[np.arange(batch), g_next]
+    agree = bool(np.all(chosen >= c_logits.max(-1) - 4e-3))
+    log(f"[decode] CPU restatement: one step in {cpu_s:.1f} s ({batch / cpu_s:.2f} tok/s, {oracle.port.num_threads()} threads); "
+        f"logits max abs err {err:.2e}, |logits| max {np.abs(c_logits).max():.2f}, greedy tokens agree: {agree}")
+    cpu.drop_cache()
+    base = {"value": round(batch / cpu_s, 3), "unit": "tok/s", "cores": oracle.port.num_threads(), "kind": "port",
+            "sample": f"1 decode step (batch {batch}, context {ctx}) of the C restatement from the post-prefill cache"}
+    par = {"logits_max_abs_err": err, "logits_abs_max": float(np.abs(c_logits).max()), "greedy_tokens_agree": agree}
+    return {"cpu_baseline": base, "parity": par}
+
+
+
 def smoke_parity(lib):
     """Small invocation checked against the oracle; raises on mismatch."""
     import oracle
@@ -239,7 +278,8 @@ def main():
         except ImportError:
             qwen3vl_text_bench = None
         if qwen3vl_text_bench is not None:
-            result["decode_step"] = qwen3vl_text_bench.run(decode_steps=args.decode_steps, log=log)
+            hook = None if args.no_cpu_baseline else cpu_decode_step_hook
+            result["decode_step"] = qwen3vl_text_bench.run(decode_steps=args.decode_steps, log=log, cpu_step_hook=hook)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_gqa()

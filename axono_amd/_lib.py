@@ -61,6 +61,8 @@ PROTOTYPES = {
     "axhip_kv_append": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_concat": (c_i, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "axhip_add_rms_norm": (c_i, [c_vp, c_vp, c_vp, c_f, c_vp, c_vp, c_i, c_i, c_i64, c_i64, c_vp]),
+    "axhip_add_rms_norm_ex": (c_i, [c_vp, c_vp, c_vp, c_f, c_vp, c_vp, c_i, c_i, c_i, c_i64, c_i64, c_vp]),
+    "axhip_rms_norm_ex": (c_i, [c_vp, c_vp, c_f, c_vp, c_i, c_i, c_i, c_i64, c_i64, c_vp]),
     "axhip_silu_mul": (c_i, [c_vp, c_vp, c_vp, c_i, c_i64, c_vp]),
     "axhip_rms_norm": (c_i, [c_vp, c_vp, c_f, c_vp, c_i, c_i, c_i64, c_i64, c_vp]),
     "axhip_add": (c_i, [c_vp, c_vp, c_vp, c_i, c_i64, c_vp]),
@@ -76,7 +78,7 @@ PROTOTYPES = {
     "axhip_argmax": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
     "axhip_qkv_norm_rope_append": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp,
                                          c_i, c_i, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
-    "axhip_silu_mul_fused": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
+    "axhip_silu_mul_fused": (c_i, [c_vp, c_vp, c_i, c_i, c_i64, c_i64, c_vp]),
     "axhip_index_add": (c_i, [c_vp, c_i, c_i64, c_i64, c_vp]),
 }
 

@@ -104,9 +104,9 @@ __global__ __launch_bounds__(kBlock) void qkv_norm_rope_append_kernel(QkvArgs a)
   }
 }
 
-template <typename T>
+template <typename T, typename OT>
 __global__ __launch_bounds__(kBlock) void silu_mul_fused_kernel(const T *__restrict__ gu,
-                                                                T *__restrict__ y, int64_t rows,
+                                                                OT *__restrict__ y, int64_t rows,
                                                                 int cols) {
   // gu [rows, 2*cols] = [gate | up]; 8 elements per thread (cols % 8 == 0)
   const int vec_per_row = cols / 8;
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void silu_mul_fused_kernel(const T *__restr
     Row8<T>::load(gu + r * 2 * cols + cols + c, u);
 #pragma unroll
     for (int j = 0; j < 8; ++j) o[j] = g[j] / (1.0f + expf(-g[j])) * u[j];
-    Row8<T>::store(y + r * cols + c, o);
+    Row8<OT>::store(y + r * cols + c, o);
   }
 }
 
@@ -174,9 +174,10 @@ AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const
   return launch_status();
 }
 
-AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int64_t rows, int64_t cols,
-                                   axhip_stream stream) {
+AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int out_dtype, int64_t rows,
+                                   int64_t cols, axhip_stream stream) {
   if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (out_dtype != dtype && !(dtype == AXHIP_FLOAT32 && out_dtype == AXHIP_FLOAT16)) return AXHIP_UNSUPPORTED_TYPE;
   if (rows < 0 || cols <= 0 || cols % 8 != 0) return AXHIP_INVALID_ARGUMENT;
   if (rows == 0) return AXHIP_OK;
   if (!gate_up || !y) return AXHIP_INVALID_PTR;
@@ -186,11 +187,15 @@ AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int6
   if (grid > 256u * 16u) grid = 256u * 16u;
   hipStream_t st = as_stream(stream);
   if (dtype == AXHIP_FLOAT16)
-    hipLaunchKernelGGL((silu_mul_fused_kernel<__half>), dim3(grid), dim3(kBlock), 0, st,
+    hipLaunchKernelGGL((silu_mul_fused_kernel<__half, __half>), dim3(grid), dim3(kBlock), 0, st,
                        static_cast<const __half *>(gate_up), static_cast<__half *>(y), rows,
                        static_cast<int>(cols));
+  else if (out_dtype == AXHIP_FLOAT16)
+    hipLaunchKernelGGL((silu_mul_fused_kernel<float, __half>), dim3(grid), dim3(kBlock), 0, st,
+                       static_cast<const float *>(gate_up), static_cast<__half *>(y), rows,
+                       static_cast<int>(cols));
   else
-    hipLaunchKernelGGL((silu_mul_fused_kernel<float>), dim3(grid), dim3(kBlock), 0, st,
+    hipLaunchKernelGGL((silu_mul_fused_kernel<float, float>), dim3(grid), dim3(kBlock), 0, st,
                        static_cast<const float *>(gate_up), static_cast<float *>(y), rows,
                        static_cast<int>(cols));
   return launch_status();

@@ -15,8 +15,9 @@
 //
 // Scores are kept in the log2 domain (q.k * scale * log2 e) so that the exponentials are single
 // v_exp_f32 instructions.  Per-split results (unnormalised output, running max, running sum) go to
-// a workspace and a second small kernel merges them; with one split the first kernel normalises
-// and writes the result itself.
+// a workspace; the workgroup that finishes last for a (sequence, head group) - decided by a ticket
+// counter - merges them and writes the result, so one launch does the whole operator.  With one
+// split the workgroup normalises and writes the result itself.
 #include "common.hpp"
 
 namespace axhip {
@@ -31,8 +32,16 @@ constexpr int kMinChunk = 256;
 struct Tuning {
   int target_workgroups = 1024;  // 256 CUs x 4 resident workgroups
   int force_splits = 0;          // > 0: fixed split count (measurement sweeps)
+  int separate_merge = 0;        // 1: merge in a second kernel instead of the last workgroup
 };
 Tuning g_tuning;
+
+// Ticket counters of the in-kernel merge, one per (sequence, head group).  They start at zero and
+// the merging workgroup puts its counter back to zero, so no launch ever has to clear them.
+// Launches that overlap in time on one device must not share (sequence, head group) slots; calls on
+// one stream, and replays of a captured graph, never overlap.
+constexpr int kTicketSlots = 1 << 16;
+__device__ unsigned int g_tickets[kTicketSlots];
 
 struct SplitPlan {
   int n_splits;
@@ -120,7 +129,14 @@ struct DecodeArgs {
   int Hq, group, max_len, chunk, n_splits;
   int64_t stride_b, stride_h, stride_s;
   float scale_log2e;
+  int fused_merge;  // the last workgroup of a (sequence, head group) merges the splits
 };
+
+// Loads that must observe other workgroups' stores of this launch: served by L2, never by a stale
+// line of this CU's vector cache.
+__device__ __forceinline__ float ld_agent(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int max_len) {
   int len = seq_lens ? seq_lens[b] : max_len;
@@ -186,12 +202,20 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_split_kernel(DecodeArgs a
   const int split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
   const int len = clamped_len(a.seq_lens, b, a.max_len);
   const int s0 = split * a.chunk;
-  if (s0 >= len) return;  // the merge kernel never reads an empty split
+  const int tid = threadIdx.x;
+  const int h0 = hg * G;            // first query head of this workgroup
+  if (s0 >= len) {
+    // An empty split is never read by the merge.  A sequence without keys gets zeros, written by
+    // its split-0 workgroup when no separate merge kernel will do it.
+    if (len == 0 && split == 0 && (a.n_splits == 1 || a.fused_merge)) {
+      for (int o = tid; o < G * D; o += kThreads)
+        stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + h0) * D + o, 0.0f);
+    }
+    return;
+  }
   const int s1 = min(s0 + a.chunk, len);
 
-  const int tid = threadIdx.x;
   const int rg = tid / LPR, dl = tid % LPR;
-  const int h0 = hg * G;            // first query head of this workgroup
   const int hk = h0 / a.group;      // the kv head those G query heads share
 
   const T *q = static_cast<const T *>(a.q);
@@ -254,6 +278,37 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_split_kernel(DecodeArgs a
       }
     }
   }
+  if (a.n_splits == 1 || !a.fused_merge) return;
+
+  // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
+  const int n_valid = (len + a.chunk - 1) / a.chunk;  // splits that run for this sequence
+  __shared__ int s_last;
+  __threadfence();   // this workgroup's partials are visible device-wide before its ticket is
+  __syncthreads();
+  if (tid == 0) {
+    unsigned int *ticket = &g_tickets[b * gridDim.y + hg];
+    const unsigned int t = atomicAdd(ticket, 1u);
+    s_last = (t == static_cast<unsigned int>(n_valid - 1));
+    if (s_last) atomicExch(ticket, 0u);  // ready for the next launch
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  for (int o = tid; o < G * D; o += kThreads) {
+    const int g = o / D, d = o % D;
+    const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
+    const float *ml = a.part_ml + bh * a.n_splits * 2;
+    const float *pa = a.part_acc + bh * a.n_splits * D + d;
+    float mx = kNegBig;
+    for (int s = 0; s < n_valid; ++s) mx = fmaxf(mx, ld_agent(ml + 2 * s));
+    float lsum = 0.0f, asum = 0.0f;
+    for (int s = 0; s < n_valid; ++s) {
+      const float w = __builtin_amdgcn_exp2f(ld_agent(ml + 2 * s) - mx);
+      lsum = __builtin_fmaf(ld_agent(ml + 2 * s + 1), w, lsum);
+      asum = __builtin_fmaf(ld_agent(pa + static_cast<int64_t>(s) * D), w, asum);
+    }
+    stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
+  }
 }
 
 // Cross-split merge: one workgroup of D threads per (sequence, query head).
@@ -286,7 +341,7 @@ int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   constexpr int U = (sizeof(T) == 2 ? 8 : 4) / (G >= 4 ? 2 : 1);
   const dim3 grid(a.n_splits, a.Hq / G, B);
   hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U>), grid, dim3(kThreads), 0, st, a);
-  if (a.n_splits > 1)
+  if (a.n_splits > 1 && !a.fused_merge)
     hipLaunchKernelGGL((gqa_decode_merge_kernel<T, D>), dim3(a.Hq, B), dim3(D), 0, st, a);
   return launch_status();
 }
@@ -322,6 +377,8 @@ extern "C" {
 
 // Measurement hook: overrides the split heuristics (0 restores the default).
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits) {
+  // a negative target selects the two-kernel form (split kernel + merge kernel)
+  g_tuning.separate_merge = target_workgroups < 0 ? 1 : 0;
   g_tuning.target_workgroups = target_workgroups > 0 ? target_workgroups : Tuning().target_workgroups;
   g_tuning.force_splits = force_splits > 0 ? force_splits : 0;
 }
@@ -378,6 +435,7 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v, cons
   a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
   a.part_acc = nullptr;
   a.part_ml = nullptr;
+  a.fused_merge = (!g_tuning.separate_merge && static_cast<long>(B) * (Hq / G) <= kTicketSlots) ? 1 : 0;
   if (plan.n_splits > 1) {
     const size_t acc_elems = static_cast<size_t>(B) * Hq * plan.n_splits * D;
     const size_t need = (acc_elems + static_cast<size_t>(B) * Hq * plan.n_splits * 2) * sizeof(float);

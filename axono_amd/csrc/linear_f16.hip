@@ -10,9 +10,9 @@
 // HBM-bound.  A wavefront owns NT*16 rows of W and a K slice, with the W rows as the MFMA "A"
 // operand and the (few) x rows as "B", so the output fragment holds out^T.  Nothing is staged
 // through LDS: x is small and stays in L2.  The four wavefronts of a workgroup take four K slices
-// of the same rows and add their fragments through LDS; further K splitting across workgroups
-// (needed to fill 256 CUs when N is small) goes through fp32 partial sums in a workspace and a
-// small reduction kernel.
+// of the same rows and add their fragments through LDS, so one launch finishes the product; small
+// N gets up to 16 wavefronts (K slices) per workgroup so that the launch still fills 256 CUs.
+//
 //
 // Larger M runs a tiled GEMM (128x128 output tile per workgroup, 32x32x16 MFMA, operands staged
 // through LDS with register double buffering); it is MFMA-bound once M reaches a few hundred rows.
@@ -21,22 +21,24 @@
 namespace axhip {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
-constexpr int kMaxOuterSplits = 8;
+constexpr int kThreads = 256;   // tiled GEMM workgroup
 constexpr int kSkinnyMaxM = 32;
+constexpr int kMaxWaves = 16;   // wavefronts per workgroup of the skinny kernel (K slices)
 
 struct LinearTuning {
   int target_waves = 2048;  // wavefronts to aim for in the skinny kernel (256 CUs x 8)
   int force_nt = 0;         // > 0: rows-of-16 per wavefront (1, 2 or 4)
-  int force_ks_outer = 0;   // > 0: K splits across workgroups
+  int force_waves = 0;      // > 0: wavefronts (K slices) per workgroup (4, 8 or 16)
 };
 LinearTuning g_lin;
 
 struct SkinnyPlan {
-  int nt, mt, ks_outer, k_per_wave;
+  int nt, mt, waves, k_per_wave;
 };
 
+// A workgroup owns NT*16 rows of W and all of K; its wavefronts split K and add their fragments
+// through LDS, so one launch finishes the product.  Small N gets more wavefronts per workgroup
+// (down to 128 of K each) so that the launch still fills the chip.
 SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
   SkinnyPlan p;
   p.mt = M <= 16 ? 1 : 2;
@@ -48,17 +50,15 @@ SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
     p.nt = N >= 32768 ? 4 : (N >= 8192 ? 2 : 1);
   if (p.mt == 2 && p.nt > 2) p.nt = 2;
   const int64_t ntiles = (N + p.nt * 16 - 1) / (p.nt * 16);
-  int64_t ks = g_lin.force_ks_outer > 0
-                   ? g_lin.force_ks_outer
-                   : (g_lin.target_waves + ntiles * kWaves - 1) / (ntiles * kWaves);
-  const int64_t cap = K / (kWaves * 256);  // at least 256 of K per wavefront
-  if (ks > cap) ks = cap;
-  if (ks > kMaxOuterSplits) ks = kMaxOuterSplits;
-  if (ks < 1) ks = 1;
-  int64_t kpw = (K + kWaves * ks - 1) / (kWaves * ks);
-  kpw = (kpw + 127) / 128 * 128;
-  p.ks_outer = static_cast<int>((K + kWaves * kpw - 1) / (kWaves * kpw));
-  p.k_per_wave = static_cast<int>(kpw);
+  int64_t want = g_lin.force_waves > 0 ? g_lin.force_waves : (g_lin.target_waves + ntiles - 1) / ntiles;
+  int waves = 4;
+  while (waves < want && waves < kMaxWaves) waves *= 2;
+  while (waves > 4 && K / waves < 128) waves /= 2;
+  if (p.nt == 4 && waves > 4) waves = 4;   // LDS: the reduction buffer grows with NT * waves
+  if (p.nt * p.mt >= 2 && waves > 8) waves = 8;
+  p.waves = waves;
+  int64_t kpw = (K + waves - 1) / waves;
+  p.k_per_wave = static_cast<int>((kpw + 127) / 128 * 128);
   return p;
 }
 
@@ -91,36 +91,47 @@ struct LinearArgs {
   const __half *w;
   const __half *bias;
   void *out;
-  float *partial;  // [ks_outer, M, N] when ks_outer > 1
   int M, K, N;
-  int k_per_wave, ks_outer, out_f16;
+  int k_per_wave, out_f16;
 };
 
-// Final store of 4 consecutive n for one m (bias added here when this is the last reduction).
-__device__ __forceinline__ void store_out4(const LinearArgs &a, int m, int n, const float (&v)[4],
-                                           bool add_bias) {
+// Final store of 4 consecutive n for one m, bias added.
+__device__ __forceinline__ void store_out4(const LinearArgs &a, int m, int n, const float (&v)[4]) {
   if (m >= a.M) return;
+  const int64_t o = static_cast<int64_t>(m) * a.N + n;
+  if (n + 3 < a.N && (a.N & 3) == 0) {
+    float y[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) y[r] = v[r] + (a.bias ? __half2float(a.bias[n + r]) : 0.f);
+    if (a.out_f16) {
+      half4_t h;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) h[r] = static_cast<_Float16>(y[r]);
+      *reinterpret_cast<half4_t *>(static_cast<__half *>(a.out) + o) = h;
+    } else {
+      *reinterpret_cast<float4_t *>(static_cast<float *>(a.out) + o) = float4_t{y[0], y[1], y[2], y[3]};
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     if (n + r >= a.N) continue;
     float y = v[r];
-    if (add_bias && a.bias) y += __half2float(a.bias[n + r]);
-    const int64_t o = static_cast<int64_t>(m) * a.N + n + r;
+    if (a.bias) y += __half2float(a.bias[n + r]);
     if (a.out_f16)
-      static_cast<__half *>(a.out)[o] = __float2half_rn(y);
+      static_cast<__half *>(a.out)[o + r] = __float2half_rn(y);
     else
-      static_cast<float *>(a.out)[o] = y;
+      static_cast<float *>(a.out)[o + r] = y;
   }
 }
 
-template <int NT, int MT, typename XT>
-__global__ __launch_bounds__(kThreads) void linear_skinny_kernel(LinearArgs a) {
+template <int NT, int MT, int WAVES, typename XT>
+__global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(LinearArgs a) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
   const int n_base = blockIdx.x * (NT * 16);
-  const int kso = blockIdx.y;
-  const int m_base = blockIdx.z * (MT * 16);
-  const int k_begin = (kso * kWaves + wave) * a.k_per_wave;
+  const int m_base = blockIdx.y * (MT * 16);
+  const int k_begin = wave * a.k_per_wave;
   const int k_end = min(k_begin + a.k_per_wave, a.K);
   const XT *x = static_cast<const XT *>(a.x);
 
@@ -167,8 +178,8 @@ __global__ __launch_bounds__(kThreads) void linear_skinny_kernel(LinearArgs a) {
           acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t][j], bf[u][j], acc[t][u], 0, 0, 0);
   }
 
-  // add the four K slices of this workgroup
-  __shared__ float4_t red[kWaves - 1][NT * MT][64];
+  // add the K slices of this workgroup: wavefronts 1.. park their fragments in LDS, wavefront 0 sums
+  __shared__ float4_t red[WAVES - 1][NT * MT][64];
   if (wave > 0) {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
@@ -183,56 +194,45 @@ __global__ __launch_bounds__(kThreads) void linear_skinny_kernel(LinearArgs a) {
     for (int u = 0; u < MT; ++u) {
       float4_t s = acc[t][u];
 #pragma unroll
-      for (int w = 0; w < kWaves - 1; ++w) s += red[w][t * MT + u][lane];
+      for (int w = 0; w < WAVES - 1; ++w) s += red[w][t * MT + u][lane];
       // fragment layout: this lane holds out[m = m_base + u*16 + r][n = n_base + t*16 + 4g + 0..3]
-      const int m = m_base + u * 16 + r;
-      const int n = n_base + t * 16 + 4 * g;
       const float v[4] = {s[0], s[1], s[2], s[3]};
-      if (a.ks_outer == 1) {
-        store_out4(a, m, n, v, true);
-      } else if (m < a.M) {
-        float *dst = a.partial + (static_cast<int64_t>(kso) * a.M + m) * a.N + n;
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (n + q < a.N) dst[q] = v[q];
-      }
+      store_out4(a, m_base + u * 16 + r, n_base + t * 16 + 4 * g, v);
     }
   }
 }
 
-__global__ __launch_bounds__(kThreads) void linear_reduce_kernel(LinearArgs a) {
-  const int64_t total = static_cast<int64_t>(a.M) * a.N;
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i >= total) return;
-  float s = 0.f;
-  for (int k = 0; k < a.ks_outer; ++k) s += a.partial[static_cast<int64_t>(k) * total + i];
-  if (a.bias) s += __half2float(a.bias[i % a.N]);
-  if (a.out_f16)
-    static_cast<__half *>(a.out)[i] = __float2half_rn(s);
-  else
-    static_cast<float *>(a.out)[i] = s;
+template <int NT, int MT, int WAVES, typename XT>
+void launch_skinny(const LinearArgs &a, hipStream_t st) {
+  const dim3 grid((a.N + NT * 16 - 1) / (NT * 16), (a.M + MT * 16 - 1) / (MT * 16));
+  hipLaunchKernelGGL((linear_skinny_kernel<NT, MT, WAVES, XT>), grid, dim3(WAVES * 64), 0, st, a);
 }
 
 template <int NT, int MT, typename XT>
-void launch_skinny(const LinearArgs &a, hipStream_t st) {
-  const dim3 grid((a.N + NT * 16 - 1) / (NT * 16), a.ks_outer, (a.M + MT * 16 - 1) / (MT * 16));
-  hipLaunchKernelGGL((linear_skinny_kernel<NT, MT, XT>), grid, dim3(kThreads), 0, st, a);
+void dispatch_waves(const LinearArgs &a, int waves, hipStream_t st) {
+  if constexpr (NT * MT == 1) {
+    if (waves >= 16) return launch_skinny<NT, MT, 16, XT>(a, st);
+  }
+  if constexpr (NT < 4) {
+    if (waves >= 8) return launch_skinny<NT, MT, 8, XT>(a, st);
+  }
+  launch_skinny<NT, MT, 4, XT>(a, st);
 }
 
 template <typename XT>
 void dispatch_skinny(const LinearArgs &a, const SkinnyPlan &p, hipStream_t st) {
   if (p.mt == 1) {
     if (p.nt == 4)
-      launch_skinny<4, 1, XT>(a, st);
+      dispatch_waves<4, 1, XT>(a, p.waves, st);
     else if (p.nt == 2)
-      launch_skinny<2, 1, XT>(a, st);
+      dispatch_waves<2, 1, XT>(a, p.waves, st);
     else
-      launch_skinny<1, 1, XT>(a, st);
+      dispatch_waves<1, 1, XT>(a, p.waves, st);
   } else {
     if (p.nt == 2)
-      launch_skinny<2, 2, XT>(a, st);
+      dispatch_waves<2, 2, XT>(a, p.waves, st);
     else
-      launch_skinny<1, 2, XT>(a, st);
+      dispatch_waves<1, 2, XT>(a, p.waves, st);
   }
 }
 
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void linear_gemm_kernel(LinearArgs a) {
         const int n = n0 + wn + i * 32 + blk * 8 + (lane >> 5) * 4;
         const float v[4] = {acc[i][j][blk * 4], acc[i][j][blk * 4 + 1], acc[i][j][blk * 4 + 2],
                             acc[i][j][blk * 4 + 3]};
-        store_out4(a, m, n, v, true);
+        store_out4(a, m, n, v);
       }
     }
   }
@@ -331,59 +331,52 @@ using namespace axhip;
 extern "C" {
 
 // Measurement hook for sweeps (0 restores a default).
-AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_ks_outer) {
+AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves) {
   g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
-  g_lin.force_ks_outer = force_ks_outer > 0 ? force_ks_outer : 0;
+  g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;
 }
 
+// Every shape is finished by one launch; no workspace is needed (the argument stays in the ABI for
+// callers that size buffers generically).
 AXHIP_API size_t axhip_linear_f16_workspace_bytes(int64_t M, int64_t K, int64_t N) {
-  if (M <= 0 || K <= 0 || N <= 0 || M > kSkinnyMaxM) return 0;
-  // enough for any split count the skinny kernel may choose
-  return static_cast<size_t>(kMaxOuterSplits) * M * N * sizeof(float);
+  (void)M;
+  (void)K;
+  (void)N;
+  return 0;
 }
 
 AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const void *bias, void *out,
                                int out_dtype, int64_t M, int64_t K, int64_t N, void *workspace,
                                size_t workspace_bytes, axhip_stream stream) {
+  (void)workspace;
+  (void)workspace_bytes;
   if (!is_float_dtype(x_dtype) || !is_float_dtype(out_dtype)) return AXHIP_UNSUPPORTED_TYPE;
   if (M < 0 || K <= 0 || N <= 0 || K % 8 != 0) return AXHIP_INVALID_ARGUMENT;
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
   if (M == 0) return AXHIP_OK;
   if (!x || !w || !out) return AXHIP_INVALID_PTR;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return AXHIP_INVALID_PTR;
+  if (reinterpret_cast<uintptr_t>(out) & 15) return AXHIP_INVALID_PTR;
   hipStream_t st = as_stream(stream);
   LinearArgs a;
   a.x = x;
   a.w = static_cast<const __half *>(w);
   a.bias = static_cast<const __half *>(bias);
   a.out = out;
-  a.partial = nullptr;
   a.M = static_cast<int>(M);
   a.K = static_cast<int>(K);
   a.N = static_cast<int>(N);
   a.out_f16 = out_dtype == AXHIP_FLOAT16;
-  a.ks_outer = 1;
   a.k_per_wave = 0;
 
   if (M <= kSkinnyMaxM) {
     const SkinnyPlan p = plan_skinny(M, K, N);
-    a.ks_outer = p.ks_outer;
     a.k_per_wave = p.k_per_wave;
-    if (p.ks_outer > 1) {
-      const size_t need = static_cast<size_t>(p.ks_outer) * M * N * sizeof(float);
-      if (!workspace || workspace_bytes < need) return AXHIP_INVALID_ARGUMENT;
-      a.partial = static_cast<float *>(workspace);
-    }
     if (x_dtype == AXHIP_FLOAT16)
       dispatch_skinny<__half>(a, p, st);
     else
       dispatch_skinny<float>(a, p, st);
-    if (p.ks_outer > 1) {
-      const int64_t total = M * N;
-      hipLaunchKernelGGL(linear_reduce_kernel, dim3(static_cast<unsigned>((total + kThreads - 1) / kThreads)),
-                         dim3(kThreads), 0, st, a);
-    }
     return launch_status();
   }
   const dim3 grid((a.N + kTN - 1) / kTN, (a.M + kTM - 1) / kTM);

@@ -27,11 +27,11 @@ inline unsigned blocks_for(int64_t items, int per_block) {
 // ------------------------------------------------------------------------------------------------
 constexpr int kRegChunks = 4;
 
-template <typename T, typename WT, int TPR, bool ADD>
+template <typename T, typename WT, typename OT, int TPR, bool ADD>
 __global__ __launch_bounds__(kBlock) void rms_norm_kernel(const T *__restrict__ x,
                                                           const T *__restrict__ res,
                                                           const WT *__restrict__ w, float eps,
-                                                          T *__restrict__ y, T *__restrict__ out,
+                                                          T *__restrict__ y, OT *__restrict__ out,
                                                           int64_t rows, int hidden, int vec_ok) {
   constexpr int RPB = kBlock / TPR;
   __shared__ float red[kBlock / 64];
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_kernel(const T *__restrict__ 
 #pragma unroll
       for (int j = 0; j < 8; ++j) o[j] = a[j] * rms;
     }
-    Row8<T>::store(out + off + i * 8, o);
+    Row8<OT>::store(out + off + i * 8, o);
   }
   for (int i = nvec * 8 + lane; i < hidden; i += TPR) {
     float a = ldf(x + off + i);
@@ -111,18 +111,21 @@ __global__ __launch_bounds__(kBlock) void rms_norm_kernel(const T *__restrict__ 
   }
 }
 
-template <typename T, typename WT, bool ADD>
+template <typename T, typename WT, typename OT, bool ADD>
 int launch_rms(const void *x, const void *res, const void *w, float eps, void *y, void *out,
                int64_t rows, int64_t hidden, hipStream_t st) {
-  const int vec_ok = (hidden * sizeof(T)) % 16 == 0;  // else every element goes through the scalar path
+  // rows of both element sizes must start on 16-byte boundaries, else every element goes through
+  // the scalar path
+  const int vec_ok = (hidden * sizeof(T)) % 16 == 0 && (hidden * sizeof(OT)) % 16 == 0;
   const T *xp = static_cast<const T *>(x), *rp = static_cast<const T *>(res);
   const WT *wp = static_cast<const WT *>(w);
-  T *yp = static_cast<T *>(y), *op = static_cast<T *>(out);
+  T *yp = static_cast<T *>(y);
+  OT *op = static_cast<OT *>(out);
   if (hidden <= 512) {
-    hipLaunchKernelGGL((rms_norm_kernel<T, WT, 64, ADD>), dim3(blocks_for(rows, kBlock / 64)),
+    hipLaunchKernelGGL((rms_norm_kernel<T, WT, OT, 64, ADD>), dim3(blocks_for(rows, kBlock / 64)),
                        dim3(kBlock), 0, st, xp, rp, wp, eps, yp, op, rows, static_cast<int>(hidden), vec_ok);
   } else {
-    hipLaunchKernelGGL((rms_norm_kernel<T, WT, kBlock, ADD>), dim3(static_cast<unsigned>(rows)),
+    hipLaunchKernelGGL((rms_norm_kernel<T, WT, OT, kBlock, ADD>), dim3(static_cast<unsigned>(rows)),
                        dim3(kBlock), 0, st, xp, rp, wp, eps, yp, op, rows, static_cast<int>(hidden), vec_ok);
   }
   return launch_status();
@@ -130,8 +133,10 @@ int launch_rms(const void *x, const void *res, const void *w, float eps, void *y
 
 template <bool ADD>
 int dispatch_rms(const void *x, const void *res, const void *w, float eps, void *y, void *out,
-                 int dtype, int w_dtype, int64_t rows, int64_t hidden, hipStream_t st) {
+                 int dtype, int w_dtype, int out_dtype, int64_t rows, int64_t hidden, hipStream_t st) {
   if (!is_float_dtype(dtype) || (w && !is_float_dtype(w_dtype))) return AXHIP_UNSUPPORTED_TYPE;
+  // the normalised output may be FLOAT16 while the activations are FLOAT32 (it feeds an fp16 Linear)
+  if (out_dtype != dtype && !(dtype == AXHIP_FLOAT32 && out_dtype == AXHIP_FLOAT16)) return AXHIP_UNSUPPORTED_TYPE;
   if (rows < 0 || hidden <= 0 || hidden > (1 << 24)) return AXHIP_INVALID_ARGUMENT;
   if (rows == 0) return AXHIP_OK;
   if (!x || !out || (ADD && (!res || !y))) return AXHIP_INVALID_PTR;
@@ -143,10 +148,13 @@ int dispatch_rms(const void *x, const void *res, const void *w, float eps, void 
   (void)esz;
   const bool wh = w && w_dtype == AXHIP_FLOAT16;
   if (dtype == AXHIP_FLOAT16)
-    return wh ? launch_rms<__half, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st)
-              : launch_rms<__half, float, ADD>(x, res, w, eps, y, out, rows, hidden, st);
-  return wh ? launch_rms<float, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st)
-            : launch_rms<float, float, ADD>(x, res, w, eps, y, out, rows, hidden, st);
+    return wh ? launch_rms<__half, __half, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st)
+              : launch_rms<__half, float, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st);
+  if (out_dtype == AXHIP_FLOAT16)
+    return wh ? launch_rms<float, __half, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st)
+              : launch_rms<float, float, __half, ADD>(x, res, w, eps, y, out, rows, hidden, st);
+  return wh ? launch_rms<float, __half, float, ADD>(x, res, w, eps, y, out, rows, hidden, st)
+            : launch_rms<float, float, float, ADD>(x, res, w, eps, y, out, rows, hidden, st);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -489,6 +497,81 @@ __global__ __launch_bounds__(kArgmaxBlock) void argmax_kernel(const T *__restric
   }
 }
 
+// Wide rows (a vocabulary): kArgmaxParts workgroups scan one row's column ranges, park their
+// (value, index) candidates in device scratch, and the workgroup that takes the last ticket of the row
+// picks the winner.  Ties go to the smaller index, as in the single-workgroup kernel.
+constexpr int kArgmaxParts = 64;
+constexpr int kArgmaxMaxRows = 1024;
+__device__ float g_argmax_val[kArgmaxMaxRows * kArgmaxParts];
+__device__ long long g_argmax_idx[kArgmaxMaxRows * kArgmaxParts];
+__device__ unsigned int g_argmax_ticket[kArgmaxMaxRows];
+
+__device__ __forceinline__ bool better(float ov, int64_t oi, float v, int64_t i) {
+  return oi != INT64_MAX && (i == INT64_MAX || ov > v || (ov == v && oi < i));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restrict__ x,
+                                                              int64_t *__restrict__ out, int64_t cols) {
+  __shared__ float s_val[kBlock / 64];
+  __shared__ int64_t s_idx[kBlock / 64];
+  __shared__ int s_last;
+  const int row = blockIdx.y, part = blockIdx.x;
+  const T *xr = x + static_cast<int64_t>(row) * cols;
+  const int64_t per = (cols + kArgmaxParts - 1) / kArgmaxParts;
+  const int64_t c0 = part * per, c1 = c0 + per < cols ? c0 + per : cols;
+  float best = -INFINITY;
+  int64_t bi = INT64_MAX;
+  for (int64_t c = c0 + threadIdx.x; c < c1; c += kBlock) {
+    const float v = ldf(xr + c);
+    if (v > best || bi == INT64_MAX) {
+      best = v;
+      bi = c;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int64_t oi = __shfl_xor(bi, off, 64);
+    if (better(ov, oi, best, bi)) {
+      best = ov;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_val[threadIdx.x >> 6] = best;
+    s_idx[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kBlock / 64; ++w)
+      if (better(s_val[w], s_idx[w], best, bi)) {
+        best = s_val[w];
+        bi = s_idx[w];
+      }
+    g_argmax_val[row * kArgmaxParts + part] = best;
+    g_argmax_idx[row * kArgmaxParts + part] = bi;
+    __threadfence();
+    const unsigned int t = atomicAdd(&g_argmax_ticket[row], 1u);
+    s_last = (t == kArgmaxParts - 1);
+    if (s_last) atomicExch(&g_argmax_ticket[row], 0u);
+  }
+  __syncthreads();
+  if (!s_last || threadIdx.x >= 64) return;
+  __threadfence();
+  // one wavefront: lane p takes part p (kArgmaxParts == 64)
+  best = __hip_atomic_load(&g_argmax_val[row * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  bi = __hip_atomic_load(&g_argmax_idx[row * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int64_t oi = __shfl_xor(bi, off, 64);
+    if (better(ov, oi, best, bi)) {
+      best = ov;
+      bi = oi;
+    }
+  }
+  if (threadIdx.x == 0) out[row] = bi == INT64_MAX ? 0 : bi;
+}
+
 }  // namespace
 }  // namespace axhip
 
@@ -500,13 +583,28 @@ AXHIP_API int axhip_add_rms_norm(const void *x, const void *residual, const void
                                  void *y, void *out, int dtype, int w_dtype, int64_t rows,
                                  int64_t hidden, axhip_stream stream) {
   if (!weight) return AXHIP_INVALID_PTR;
-  return dispatch_rms<true>(x, residual, weight, eps, y, out, dtype, w_dtype, rows, hidden,
+  return dispatch_rms<true>(x, residual, weight, eps, y, out, dtype, w_dtype, dtype, rows, hidden,
                             as_stream(stream));
+}
+
+AXHIP_API int axhip_add_rms_norm_ex(const void *x, const void *residual, const void *weight, float eps,
+                                    void *y, void *out, int dtype, int w_dtype, int out_dtype,
+                                    int64_t rows, int64_t hidden, axhip_stream stream) {
+  if (!weight) return AXHIP_INVALID_PTR;
+  return dispatch_rms<true>(x, residual, weight, eps, y, out, dtype, w_dtype, out_dtype, rows, hidden,
+                            as_stream(stream));
+}
+
+AXHIP_API int axhip_rms_norm_ex(const void *x, const void *weight, float eps, void *out, int dtype,
+                                int w_dtype, int out_dtype, int64_t rows, int64_t cols,
+                                axhip_stream stream) {
+  return dispatch_rms<false>(x, nullptr, weight, eps, nullptr, out, dtype, w_dtype, out_dtype, rows, cols,
+                             as_stream(stream));
 }
 
 AXHIP_API int axhip_rms_norm(const void *x, const void *weight, float eps, void *out, int dtype,
                              int w_dtype, int64_t rows, int64_t cols, axhip_stream stream) {
-  return dispatch_rms<false>(x, nullptr, weight, eps, nullptr, out, dtype, w_dtype, rows, cols,
+  return dispatch_rms<false>(x, nullptr, weight, eps, nullptr, out, dtype, w_dtype, dtype, rows, cols,
                              as_stream(stream));
 }
 
@@ -661,6 +759,16 @@ AXHIP_API int axhip_argmax(const void *x, int64_t *out, int dtype, int64_t rows,
   if (rows == 0) return AXHIP_OK;
   if (!x || !out) return AXHIP_INVALID_PTR;
   hipStream_t st = as_stream(stream);
+  if (cols >= 16384 && rows <= kArgmaxMaxRows) {
+    const dim3 pgrid(kArgmaxParts, static_cast<unsigned>(rows));
+    if (dtype == AXHIP_FLOAT16)
+      hipLaunchKernelGGL((argmax_parts_kernel<__half>), pgrid, dim3(kBlock), 0, st,
+                         static_cast<const __half *>(x), out, cols);
+    else
+      hipLaunchKernelGGL((argmax_parts_kernel<float>), pgrid, dim3(kBlock), 0, st,
+                         static_cast<const float *>(x), out, cols);
+    return launch_status();
+  }
   const dim3 grid(static_cast<unsigned>(rows));
   if (dtype == AXHIP_FLOAT16)
     hipLaunchKernelGGL((argmax_kernel<__half>), grid, dim3(kArgmaxBlock), 0, st,

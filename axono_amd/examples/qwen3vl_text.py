@@ -13,7 +13,9 @@ projections (their weights are the row-wise concatenation of the separate matric
 add at the end of a layer is folded into the next layer's fused add + RMSNorm; next-token argmax,
 the embedding lookup of that token and the position increment all run on the device, so a step has
 no host <-> device traffic.  Linear weights and the embedding table are FLOAT16; the residual
-stream and every Linear output are FLOAT32, as in the reference's fp16-Linear mode.
+stream and every Linear output are FLOAT32, as in the reference's fp16-Linear mode; a tensor that
+only feeds a Linear (norm outputs, the SiLU-mul result) is stored as FLOAT16 by its producer, which
+is the rounding the fp16 Linear applies to its input anyway.
 """
 from __future__ import annotations
 
@@ -110,7 +112,7 @@ class Qwen3VLTextDecoder(nn.Module):
 
     def _mlp(self, xn, p):
         gu = L.linear_nobias(xn, self._w(p + "mlp.gate_up_proj.weight"))
-        return L.linear_nobias(L.silu_mul_fused(gu), self._w(p + "mlp.down_proj.weight"))
+        return L.linear_nobias(L.silu_mul_fused(gu, DataType.FLOAT16), self._w(p + "mlp.down_proj.weight"))
 
     def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None):
         """One token per sequence.  ids INT64 [B]; pos INT64 [3,B]; appends to the cache at
@@ -121,7 +123,7 @@ class Qwen3VLTextDecoder(nn.Module):
         cache = self._cache
         max_len = attn_max_len or cache.max_len
         h = L.embedding(ids, self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)  # [B,H]
-        xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps)
+        xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
         # lengths that include the token being appended (the kernel reads them on the device)
         lens_now = self._lens_plus_one
         for i in range(cfg.num_hidden_layers):
@@ -134,11 +136,12 @@ class Qwen3VLTextDecoder(nn.Module):
             attn = L.gqa_decode_attention_cache(q, kc, vc, lens_now, max_len, workspace=self._attn_ws)
             attn_out = L.linear_nobias(attn.reshape([B, cfg.num_attention_heads * cfg.head_dim]),
                                        self._w(p + "self_attn.o_proj.weight"))
-            h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps)
+            h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
+                                    DataType.FLOAT16)
             mlp_out = self._mlp(xn2, p)
             nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
             # h = h + mlp_out folded into the following RMSNorm (next layer's input norm / final norm)
-            h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps)
+            h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps, DataType.FLOAT16)
         logits = L.linear_nobias(xn, self._w("embed_tokens.weight"))  # tied lm_head
         return logits, L.argmax(logits)
 
@@ -160,11 +163,11 @@ class Qwen3VLTextDecoder(nn.Module):
         vis = _dev(np.arange(1, S + 1, dtype=np.int32), dev)  # causal: row t sees t+1 keys
         wsb = lib.axhip_gqa_decode_workspace_bytes(S, nq, nkv, D, S)
         ws = Tensor(DataType.INT8, [max(wsb, 256)], dev, _zero=False)
-        last_h = Tensor(DataType.FLOAT32, [B, H], dev)
+        last_h = Tensor(DataType.FLOAT16, [B, H], dev)  # normalised hidden state of each sequence's last token
         esz = 2
         for b in range(B):
             h = L.embedding(_dev(ids[b].astype(np.int64), dev), self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)
-            xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps)
+            xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
             for i in range(cfg.num_hidden_layers):
                 p = f"layers.{i}."
                 qkv = L.linear_nobias(xn, self._w(p + "self_attn.qkv_proj.weight"))  # [S, width] fp32
@@ -185,12 +188,13 @@ class Qwen3VLTextDecoder(nn.Module):
                                            attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq, nkv,
                                            D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
                 attn_out = L.linear_nobias(attn, self._w(p + "self_attn.o_proj.weight"))
-                h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps)
+                h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
+                                    DataType.FLOAT16)
                 mlp_out = self._mlp(xn2, p)
                 nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
-                h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps)
+                h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps, DataType.FLOAT16)
             # keep the normalised hidden state of the last position for the lm_head
-            check(lib.axhip_memcpy_d2d(last_h.data_ptr + b * H * 4, xn.data_ptr + (S - 1) * H * 4, H * 4), "copy")
+            check(lib.axhip_memcpy_d2d(last_h.data_ptr + b * H * 2, xn.data_ptr + (S - 1) * H * 2, H * 2), "copy")
         self._cache.set_lengths(np.full(B, S, np.int32))
         logits = L.linear_nobias(last_h, self._w("embed_tokens.weight"))
         return logits, L.argmax(logits)

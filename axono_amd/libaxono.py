@@ -219,8 +219,9 @@ def silu_mul(gate: Tensor, up: Tensor) -> Tensor:
     return out
 
 
-def add_rms_norm(x: Tensor, residual: Tensor, weight: Tensor, eps: float = 1e-6):
-    """Returns (y, out).  nanobind_module.cpp:1053-1078 -> AddRmsNorm (src/ops/cuda/fused.cu:91-110)."""
+def add_rms_norm(x: Tensor, residual: Tensor, weight: Tensor, eps: float = 1e-6, out_dtype: DataType | None = None):
+    """Returns (y, out).  nanobind_module.cpp:1053-1078 -> AddRmsNorm (src/ops/cuda/fused.cu:91-110).
+    out_dtype FLOAT16 (FLOAT32 inputs only) stores the normalised result as fp16."""
     op = "add_rms_norm"
     _need_hip(op, x, residual, weight)
     if x.dtype not in _FLOATS or residual.dtype != x.dtype or x.shape != residual.shape:
@@ -230,15 +231,16 @@ def add_rms_norm(x: Tensor, residual: Tensor, weight: Tensor, eps: float = 1e-6)
     hidden = x.shape[-1]
     if weight.ndim != 1 or weight.shape[0] != hidden or weight.dtype not in _FLOATS:
         raise AxhipError(op, Status.SHAPE_MISMATCH)
-    y, out = _new(x.dtype, x.shape, x), _new(x.dtype, x.shape, x)
+    odt = DataType(out_dtype) if out_dtype is not None else x.dtype
+    y, out = _new(x.dtype, x.shape, x), _new(odt, x.shape, x)
     rows = x.num_elements // hidden if hidden else 0
-    check(_lib_().axhip_add_rms_norm(x.data_ptr, residual.data_ptr, weight.data_ptr, float(eps), y.data_ptr,
-                                     out.data_ptr, int(x.dtype), int(weight.dtype), rows, hidden,
-                                     current_stream()), op)
+    check(_lib_().axhip_add_rms_norm_ex(x.data_ptr, residual.data_ptr, weight.data_ptr, float(eps), y.data_ptr,
+                                        out.data_ptr, int(x.dtype), int(weight.dtype), int(odt), rows, hidden,
+                                        current_stream()), op)
     return y, out
 
 
-def rms_norm(x: Tensor, weight: Tensor | None, eps: float = 1e-5) -> Tensor:
+def rms_norm(x: Tensor, weight: Tensor | None, eps: float = 1e-5, out_dtype: DataType | None = None) -> Tensor:
     """nanobind_module.cpp:909-942 (llm ops) -> RmsNorm (src/ops/cpu/llm.cpp:240-264).  An empty or
     missing weight means no scaling."""
     op = "rms_norm"
@@ -251,11 +253,12 @@ def rms_norm(x: Tensor, weight: Tensor | None, eps: float = 1e-5) -> Tensor:
     cols = x.shape[-1]
     if has_w and (weight.ndim != 1 or weight.shape[0] != cols or weight.dtype not in _FLOATS):
         raise AxhipError(op, Status.SHAPE_MISMATCH)
-    out = _new(x.dtype, x.shape, x)
+    odt = DataType(out_dtype) if out_dtype is not None else x.dtype
+    out = _new(odt, x.shape, x)
     rows = x.num_elements // cols if cols else 0
-    check(_lib_().axhip_rms_norm(x.data_ptr, weight.data_ptr if has_w else None, float(eps), out.data_ptr,
-                                 int(x.dtype), int(weight.dtype) if has_w else int(DataType.FLOAT32), rows, cols,
-                                 current_stream()), op)
+    check(_lib_().axhip_rms_norm_ex(x.data_ptr, weight.data_ptr if has_w else None, float(eps), out.data_ptr,
+                                    int(x.dtype), int(weight.dtype) if has_w else int(DataType.FLOAT32), int(odt),
+                                    rows, cols, current_stream()), op)
     return out
 
 
@@ -425,16 +428,18 @@ def index_add(x: Tensor, delta: int) -> Tensor:
     return x
 
 
-def silu_mul_fused(gate_up: Tensor) -> Tensor:
-    """[rows, 2*cols] = [gate | up] -> silu(gate) * up, [rows, cols]."""
+def silu_mul_fused(gate_up: Tensor, out_dtype: DataType | None = None) -> Tensor:
+    """[rows, 2*cols] = [gate | up] -> silu(gate) * up, [rows, cols]; out_dtype FLOAT16 for a FLOAT32
+    input stores the result rounded once (for a result that only feeds an fp16 Linear)."""
     op = "silu_mul_fused"
     _need_hip(op, gate_up)
     if gate_up.dtype not in _FLOATS or gate_up.ndim < 1 or gate_up.shape[-1] % 2 != 0:
         raise AxhipError(op, Status.SHAPE_MISMATCH)
     cols = gate_up.shape[-1] // 2
     rows = gate_up.num_elements // (2 * cols) if cols else 0
-    out = _new(gate_up.dtype, gate_up.shape[:-1] + [cols], gate_up)
-    check(_lib_().axhip_silu_mul_fused(gate_up.data_ptr, out.data_ptr, int(gate_up.dtype), rows, cols,
+    odt = DataType(out_dtype) if out_dtype is not None else gate_up.dtype
+    out = _new(odt, gate_up.shape[:-1] + [cols], gate_up)
+    check(_lib_().axhip_silu_mul_fused(gate_up.data_ptr, out.data_ptr, int(gate_up.dtype), int(odt), rows, cols,
                                        current_stream()), op)
     return out
 

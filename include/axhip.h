@@ -217,6 +217,13 @@ AXHIP_API int axhip_add_rms_norm(const void *x, const void *residual, const void
                                  void *y, void *out, int dtype, int w_dtype, int64_t rows,
                                  int64_t hidden, axhip_stream stream);
 
+/* Same, with the normalised output stored as `out_dtype`: FLOAT16 while x / residual / y are
+ * FLOAT32, for a result that only feeds an fp16 Linear (which would round it to fp16 itself, so the
+ * values the Linear sees are identical).  No reference counterpart. */
+AXHIP_API int axhip_add_rms_norm_ex(const void *x, const void *residual, const void *weight, float eps,
+                                    void *y, void *out, int dtype, int w_dtype, int out_dtype,
+                                    int64_t rows, int64_t hidden, axhip_stream stream);
+
 /* y = gate / (1 + exp(-gate)) * up.  Replaces ops::cuda::SiluMul, src/ops/cuda/fused.cu:28-34,76-89. */
 AXHIP_API int axhip_silu_mul(const void *gate, const void *up, void *y, int dtype, int64_t n,
                              axhip_stream stream);
@@ -225,6 +232,10 @@ AXHIP_API int axhip_silu_mul(const void *gate, const void *up, void *y, int dtyp
  * Replaces ops::cuda::RmsNorm, src/ops/cuda/llm.cu:140-158. */
 AXHIP_API int axhip_rms_norm(const void *x, const void *weight, float eps, void *out, int dtype,
                              int w_dtype, int64_t rows, int64_t cols, axhip_stream stream);
+
+AXHIP_API int axhip_rms_norm_ex(const void *x, const void *weight, float eps, void *out, int dtype,
+                                int w_dtype, int out_dtype, int64_t rows, int64_t cols,
+                                axhip_stream stream);
 
 /* out = a + b.  Replaces ops::cuda::Add for equal shapes, src/ops/cuda/add.cu:17-24. */
 AXHIP_API int axhip_add(const void *a, const void *b, void *out, int dtype, int64_t n,
@@ -278,9 +289,10 @@ AXHIP_API int axhip_rope_with_cos_sin(const void *x, const float *cos_t, const f
  * M: at least axhip_linear_f16_workspace_bytes(M,K,N) bytes (may be 0, then pass NULL). */
 AXHIP_API size_t axhip_linear_f16_workspace_bytes(int64_t M, int64_t K, int64_t N);
 /* Measurement hook for the skinny-M kernel's plan (0 restores a default): wavefronts to aim for,
- * 16-row groups of W per wavefront (1, 2 or 4), K splits across workgroups.  No reference
+ * 16-row groups of W per wavefront (1, 2 or 4), wavefronts (K slices) per workgroup (4, 8, 16).
+ * No reference
  * counterpart (the reference leaves the choice to cuBLAS). */
-AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_ks_outer);
+AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves);
 AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const void *bias,
                                void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
                                void *workspace, size_t workspace_bytes, axhip_stream stream);
@@ -323,9 +335,10 @@ AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const
                                          int Hq, int Hkv, int D, int Lmax, axhip_stream stream);
 
 /* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
- * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0. */
-AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int64_t rows, int64_t cols,
-                                   axhip_stream stream);
+ * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0.  out_dtype
+ * may be FLOAT16 for FLOAT32 input (see axhip_add_rms_norm_ex). */
+AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int out_dtype, int64_t rows,
+                                   int64_t cols, axhip_stream stream);
 
 /* x[i] += delta in place for INT32 / INT64 device arrays (sequence lengths and positions that a
  * captured decode step advances on the device; the reference rebuilds them on the host each step,

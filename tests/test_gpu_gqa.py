@@ -140,3 +140,30 @@ def test_error_codes():
     assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 5, 128, 16, 0, 0, 0, None) == 4
     assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 3, 1, 16, 8, 128, 16, 0, 0, 0, None) == 3
     assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 8, 96, 16, 0, 0, 0, None) == 1
+
+
+def test_two_kernel_merge_mode_matches_fused_merge():
+    """The merge done by the last workgroup and the merge done by a second kernel give the same
+    result (both against the oracle), also with empty and single-split sequences in the batch."""
+    rng = np.random.default_rng(15)
+    B, Lmax = 6, 3000
+    lens = np.array([3000, 0, 1, 257, 1500, 2999], np.int32)
+    q = rng.standard_normal((B, 16, 128)).astype(np.float32).astype(np.float16)
+    k = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
+    v = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
+    want = port.gqa_decode_cache_native(q, k, v, lens)
+    fused = gqa_decode(q, k, v, lens).astype(np.float32)
+    lib().axhip_gqa_decode_tune(-1, 0)
+    two = gqa_decode(q, k, v, lens).astype(np.float32)
+    lib().axhip_gqa_decode_tune(0, 0)
+    assert np.abs(fused - want).max() <= TOL16 and np.abs(two - want).max() <= TOL16
+    assert np.all(fused[1] == 0) and np.all(two[1] == 0)
+    # repeated launches reuse the ticket counters: run the fused form several times
+    for _ in range(3):
+        again = gqa_decode(q, k, v, lens).astype(np.float32)
+        np.testing.assert_array_equal(again, fused)
+    # a single split and an empty sequence (the split-0 workgroup writes the zeros)
+    lib().axhip_gqa_decode_tune(0, 1)
+    one = gqa_decode(q, k, v, lens).astype(np.float32)
+    lib().axhip_gqa_decode_tune(0, 0)
+    assert np.abs(one - want).max() <= TOL16 and np.all(one[1] == 0)

@@ -219,3 +219,84 @@ def test_sdpa_prefill_and_small_heads():
     for t in (0, 17, 49):
         step = gu.sdpa(q[t:t + 1], k[:t + 1], v[:t + 1], False)
         np.testing.assert_allclose(step[0], full[t], rtol=0, atol=TOL32)
+
+
+def test_fp16_output_variants_round_once():
+    """Norm / SiLU-mul results stored as fp16 from fp32 inputs equal the fp32 result rounded once."""
+    rng = np.random.default_rng(30)
+    x = rng.standard_normal((16, 2048)).astype(np.float32)
+    r = rng.standard_normal((16, 2048)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(2048)).astype(np.float32)
+    dx, dr, dw = gu.dev(x), gu.dev(r), gu.dev(w)
+    dy, do = gu.DeviceBuffer(x.nbytes), gu.DeviceBuffer(x.size * 2)
+    gu._run("axhip_add_rms_norm_ex", dx.ptr, dr.ptr, dw.ptr, 1e-6, dy.ptr, do.ptr, gu.F32, gu.F32, gu.F16, 16, 2048, None)
+    gu.synchronize()
+    y32, o32 = gu.add_rms_norm(x, r, w, 1e-6)
+    np.testing.assert_array_equal(dy.download(np.float32, x.shape), y32)
+    np.testing.assert_array_equal(do.download(np.float16, x.shape).view(np.uint16), o32.astype(np.float16).view(np.uint16))
+    do2 = gu.DeviceBuffer(x.size * 2)
+    gu._run("axhip_rms_norm_ex", dx.ptr, dw.ptr, 1e-6, do2.ptr, gu.F32, gu.F32, gu.F16, 16, 2048, None)
+    gu.synchronize()
+    np.testing.assert_array_equal(do2.download(np.float16, x.shape).view(np.uint16),
+                                  gu.rms_norm(x, w, 1e-6).astype(np.float16).view(np.uint16))
+    g_u = rng.standard_normal((16, 2 * 6144)).astype(np.float32)
+    dg = gu.dev(g_u)
+    o_f32, o_f16 = gu.DeviceBuffer(16 * 6144 * 4), gu.DeviceBuffer(16 * 6144 * 2)
+    gu._run("axhip_silu_mul_fused", dg.ptr, o_f32.ptr, gu.F32, gu.F32, 16, 6144, None)
+    gu._run("axhip_silu_mul_fused", dg.ptr, o_f16.ptr, gu.F32, gu.F16, 16, 6144, None)
+    gu.synchronize()
+    want = port.silu_mul(np.ascontiguousarray(g_u[:, :6144]), np.ascontiguousarray(g_u[:, 6144:]))
+    got32 = o_f32.download(np.float32, (16, 6144))
+    np.testing.assert_allclose(got32, want, rtol=2e-6, atol=1e-6)
+    np.testing.assert_array_equal(o_f16.download(np.float16, (16, 6144)).view(np.uint16), got32.astype(np.float16).view(np.uint16))
+    assert gu.lib().axhip_silu_mul_fused(dg.ptr, o_f32.ptr, gu.F16, gu.F32, 16, 6144, None) == 3  # fp16 in, fp32 out: refused
+
+
+def test_qkv_norm_rope_append_equals_op_composition():
+    """The fused decode glue against rms_norm -> rope_thd -> round to fp16 -> append of the oracle."""
+    rng = np.random.default_rng(31)
+    B, S, nq, nkv, D, lmax = 3, 2, 4, 2, 128, 16
+    T = B * S
+    width = (nq + 2 * nkv) * D
+    qkv = rng.standard_normal((T, width)).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    pos = rng.integers(0, 8192, (3, T)).astype(np.int64)
+    inv = port.rope_inv_freq(1e6, D)
+    lens = np.array([5, 0, 13], np.int32)
+    kc = rng.standard_normal((B, nkv, lmax, D)).astype(np.float16)
+    vc = rng.standard_normal((B, nkv, lmax, D)).astype(np.float16)
+    dq, dqw, dkw, dp, di, dl, dkc, dvc = (gu.dev(a) for a in (qkv, qw, kw, pos, inv, lens, kc, vc))
+    qo = gu.DeviceBuffer(T * nq * D * 2)
+    gu._run("axhip_qkv_norm_rope_append", dq.ptr, width, dq.ptr + nq * D * 4, width, dq.ptr + (nq + nkv) * D * 4, width,
+            dqw.ptr, dkw.ptr, gu.F32, 1e-6, dp.ptr, di.ptr, 20, 20, dl.ptr, qo.ptr, dkc.ptr, dvc.ptr, gu.F16,
+            B, S, nq, nkv, D, lmax, None)
+    gu.synchronize()
+    q = port.rope_thd(port.rms_norm(qkv[:, : nq * D].reshape(T, nq, D), qw, 1e-6), pos, inv, [24, 20, 20])
+    k = port.rope_thd(port.rms_norm(qkv[:, nq * D:(nq + nkv) * D].reshape(T, nkv, D), kw, 1e-6), pos, inv, [24, 20, 20])
+    v = qkv[:, (nq + nkv) * D:].reshape(T, nkv, D)
+    got_q = qo.download(np.float16, (T, nq, D)).astype(np.float32)
+    assert np.abs(got_q - q).max() <= 2e-3
+    wk, wv = kc.copy(), vc.copy()
+    for t in range(T):
+        b, off = t // S, t % S
+        wk[b, :, lens[b] + off] = k[t].astype(np.float16)
+        wv[b, :, lens[b] + off] = v[t].astype(np.float16)
+    gk, gv = dkc.download(np.float16, kc.shape), dvc.download(np.float16, vc.shape)
+    np.testing.assert_array_equal(gv.view(np.uint16), wv.view(np.uint16))  # v: one exact rounding
+    assert np.abs(gk.astype(np.float32) - wk.astype(np.float32)).max() <= 2e-3
+    touched = np.zeros(kc.shape, bool)
+    for t in range(T):
+        touched[t // S, :, lens[t // S] + t % S] = True
+    np.testing.assert_array_equal(gk[~touched].view(np.uint16), kc[~touched].view(np.uint16))  # other rows untouched
+
+
+def test_index_add():
+    a32 = np.array([5, 0, -3], np.int32)
+    a64 = np.arange(6, dtype=np.int64).reshape(3, 2) * 1000
+    d32, d64 = gu.dev(a32), gu.dev(a64)
+    gu._run("axhip_index_add", d32.ptr, gu.I32, 3, 1, None)
+    gu._run("axhip_index_add", d64.ptr, gu.I64, 6, 7, None)
+    gu.synchronize()
+    np.testing.assert_array_equal(d32.download(np.int32, (3,)), a32 + 1)
+    np.testing.assert_array_equal(d64.download(np.int64, (3, 2)), a64 + 7)

@@ -147,7 +147,7 @@ def bench_rowops(lib, steps=200):
            "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 3)})
 
 
-def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512)):
+def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False):
     rng = np.random.default_rng(0)
     shapes = shapes or [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 151936)]
     for K, N in shapes:
@@ -162,8 +162,15 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512)):
                 n = min(w_host.nbytes, N * K * 2 - off)
                 wb.upload(w_host.reshape(-1)[: n // 2], off)
                 off += n
+            if packed:
+                pb = DeviceBuffer(lib.axhip_linear_f16_packed_bytes(N, K))
+                check(lib.axhip_linear_f16_pack(wb.ptr, pb.ptr, N, K, None), "pack")
+                check(lib.axhip_synchronize(), "sync")
+                wb = pb
             ws_.append(wb)
         for M in Ms:
+            if packed and M > 32:
+                continue
             x = DeviceBuffer.from_numpy(rng.standard_normal((M, K)).astype(np.float32).astype(np.float16))
             out = DeviceBuffer(M * N * 4)
             wsb = lib.axhip_linear_f16_workspace_bytes(M, K, N)
@@ -173,12 +180,15 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512)):
             def step():
                 wb = ws_[st["i"] % n_rot]
                 st["i"] += 1
-                check(lib.axhip_linear_f16(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, ws.ptr, wsb, None), "linear")
+                if packed:
+                    check(lib.axhip_linear_f16_packed(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, None), "linear")
+                else:
+                    check(lib.axhip_linear_f16(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, ws.ptr, wsb, None), "linear")
 
             us = _time(lib, step, steps)
             nb = 2 * K * N + 2 * M * K + 4 * M * N
             fl = 2.0 * M * K * N
-            _emit({"op": "linear_f16", "M": M, "K": K, "N": N, "us": round(us, 2), "bytes": nb,
+            _emit({"op": "linear_f16_packed" if packed else "linear_f16", "M": M, "K": K, "N": N, "us": round(us, 2), "bytes": nb,
                    "GBps": round(nb / us / 1e3, 1), "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 1),
                    "TFLOPs": round(fl / us / 1e6, 1), "pct_mfma_f16_peak": round(100 * fl / us / 1e6 / MFMA_F16_PEAK, 2),
                    "weight_copies": n_rot})
@@ -186,7 +196,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512)):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "copy", "rowops", "linear"])
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "copy", "rowops", "linear", "linear-packed"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -216,6 +226,8 @@ def main(argv=None):
         bench_rowops(lib)
     elif args.what == "linear":
         bench_linear(lib)
+    elif args.what == "linear-packed":
+        bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)], packed=True)
 
 
 if __name__ == "__main__":

@@ -15,9 +15,9 @@
 //
 // Scores are kept in the log2 domain (q.k * scale * log2 e) so that the exponentials are single
 // v_exp_f32 instructions.  Per-split results (unnormalised output, running max, running sum) go to
-// a workspace; the workgroup that finishes last for a (sequence, head group) - decided by a ticket
-// counter - merges them and writes the result, so one launch does the whole operator.  With one
-// split the workgroup normalises and writes the result itself.
+// a workspace and a second small kernel merges them; with one split the first kernel normalises
+// and writes the result itself.  (A single-launch form, in which the workgroup that takes the last
+// ticket of a (sequence, head group) merges, is kept behind the tuning hook: it measured no faster.)
 #include "common.hpp"
 
 namespace axhip {
@@ -32,7 +32,7 @@ constexpr int kMinChunk = 256;
 struct Tuning {
   int target_workgroups = 1024;  // 256 CUs x 4 resident workgroups
   int force_splits = 0;          // > 0: fixed split count (measurement sweeps)
-  int separate_merge = 0;        // 1: merge in a second kernel instead of the last workgroup
+  int separate_merge = 1;        // 1: merge in a second kernel; 0: the last workgroup merges
 };
 Tuning g_tuning;
 
@@ -132,10 +132,16 @@ struct DecodeArgs {
   int fused_merge;  // the last workgroup of a (sequence, head group) merges the splits
 };
 
-// Loads that must observe other workgroups' stores of this launch: served by L2, never by a stale
-// line of this CU's vector cache.
+// Split partials travel between workgroups that may sit on different XCDs, whose L2 caches are not
+// coherent with each other.  They are written and read with agent-scope atomic accesses (stores
+// written through, loads served past the local caches), which costs nothing for these few bytes; a
+// device-scope release fence instead would write back the whole L2 from every workgroup and was
+// measured to triple the kernel's time.
 __device__ __forceinline__ float ld_agent(const float *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int max_len) {
@@ -271,10 +277,10 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_split_kernel(DecodeArgs a
     if (a.n_splits == 1) {
       stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
     } else {
-      a.part_acc[(bh * a.n_splits + split) * D + d] = asum;
+      st_agent(&a.part_acc[(bh * a.n_splits + split) * D + d], asum);
       if (d == 0) {
-        a.part_ml[(bh * a.n_splits + split) * 2] = mx;
-        a.part_ml[(bh * a.n_splits + split) * 2 + 1] = lsum;
+        st_agent(&a.part_ml[(bh * a.n_splits + split) * 2], mx);
+        st_agent(&a.part_ml[(bh * a.n_splits + split) * 2 + 1], lsum);
       }
     }
   }
@@ -283,8 +289,7 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_split_kernel(DecodeArgs a
   // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
   const int n_valid = (len + a.chunk - 1) / a.chunk;  // splits that run for this sequence
   __shared__ int s_last;
-  __threadfence();   // this workgroup's partials are visible device-wide before its ticket is
-  __syncthreads();
+  __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
   if (tid == 0) {
     unsigned int *ticket = &g_tickets[b * gridDim.y + hg];
     const unsigned int t = atomicAdd(ticket, 1u);
@@ -293,7 +298,6 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_split_kernel(DecodeArgs a
   }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
   for (int o = tid; o < G * D; o += kThreads) {
     const int g = o / D, d = o % D;
     const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
@@ -377,8 +381,9 @@ extern "C" {
 
 // Measurement hook: overrides the split heuristics (0 restores the default).
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits) {
-  // a negative target selects the two-kernel form (split kernel + merge kernel)
-  g_tuning.separate_merge = target_workgroups < 0 ? 1 : 0;
+  // a negative target selects the single-launch form (the last workgroup merges); measured no
+  // faster than the second kernel (ticket + write-through latency at the tail), so not the default
+  g_tuning.separate_merge = target_workgroups < 0 ? 0 : 1;
   g_tuning.target_workgroups = target_workgroups > 0 ? target_workgroups : Tuning().target_workgroups;
   g_tuning.force_splits = force_splits > 0 ? force_splits : 0;
 }

@@ -323,6 +323,158 @@ __global__ __launch_bounds__(kThreads) void linear_gemm_kernel(LinearArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Packed weights.  W [N,K] row-major is re-ordered once into MFMA fragment order: the matrix is cut
+// into tiles of 16 rows x 32 K, and a tile is stored as the 1 KiB block a wavefront loads for one
+// v_mfma_f32_16x16x32_f16 (lane (r, g) = 8 halves W[16 t + r][32 c + 8 g ..]); the blocks of one
+// row tile are consecutive in c.  A wavefront streaming a row tile then reads consecutive memory,
+// 64 x 16 B per load instruction, the same pattern that lets the attention kernel run near HBM speed.
+// Rows and K are zero-padded to whole tiles.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pack_weight_kernel(const __half *__restrict__ w,
+                                                          __half *__restrict__ packed, int N, int K,
+                                                          int KC, int64_t frags) {
+  const int64_t f = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (f >= frags) return;
+  const int lane = static_cast<int>(f & 63);
+  const int64_t blk = f >> 6;
+  const int c = static_cast<int>(blk % KC);
+  const int64_t t = blk / KC;
+  const int64_t row = t * 16 + (lane & 15);
+  const int k = c * 32 + (lane >> 4) * 8;
+  Vec16 v;
+  v.w[0] = v.w[1] = v.w[2] = v.w[3] = 0u;
+  if (row < N && k + 8 <= K) v = ld16(w + row * K + k);
+  st16(packed + f * 8, v);
+}
+
+struct PackedArgs {
+  const void *x;
+  const __half *wp;
+  const __half *bias;
+  void *out;
+  int M, K, N, KC, chunks_per_wave, out_f16;
+};
+
+template <int NT, int MT, int WAVES, int U, typename XT>
+__global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(PackedArgs a) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int tile0 = blockIdx.x * NT;
+  const int n_tiles = (a.N + 15) / 16;
+  const int m_base = blockIdx.y * (MT * 16);
+  const int c_begin = wave * a.chunks_per_wave;
+  const int c_end = min(c_begin + a.chunks_per_wave, a.KC);
+  const XT *x = static_cast<const XT *>(a.x);
+
+  float4_t acc[NT][MT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const __half *wt[NT];
+  bool wok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    wok[t] = tile0 + t < n_tiles;
+    wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + lane * 8;
+  }
+  const XT *xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) {
+    const int m = m_base + u * 16 + r;
+    xok[u] = m < a.M;
+    xrow[u] = x + static_cast<int64_t>(xok[u] ? m : 0) * a.K + g * 8;
+  }
+
+  for (int c = c_begin; c < c_end; c += U) {
+    half8_t af[NT][U], bf[MT][U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const int cc = c + j;
+      const bool in = cc < c_end;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        af[t][j] = (in && wok[t]) ? load_h8(wt[t] + static_cast<int64_t>(cc) * 512) : zero_h8();
+      const bool kin = in && (cc * 32 + g * 8 + 8 <= a.K);
+#pragma unroll
+      for (int u = 0; u < MT; ++u) bf[u][j] = (kin && xok[u]) ? load_h8(xrow[u] + cc * 32) : zero_h8();
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int u = 0; u < MT; ++u)
+          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t][j], bf[u][j], acc[t][u], 0, 0, 0);
+  }
+
+  __shared__ float4_t red[WAVES - 1][NT * MT][64];
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int u = 0; u < MT; ++u) red[wave - 1][t * MT + u][lane] = acc[t][u];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  LinearArgs o;  // only the fields store_out4 reads
+  o.bias = a.bias;
+  o.out = a.out;
+  o.M = a.M;
+  o.N = a.N;
+  o.out_f16 = a.out_f16;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+      float4_t s = acc[t][u];
+#pragma unroll
+      for (int w = 0; w < WAVES - 1; ++w) s += red[w][t * MT + u][lane];
+      const float v[4] = {s[0], s[1], s[2], s[3]};
+      store_out4(o, m_base + u * 16 + r, (tile0 + t) * 16 + 4 * g, v);
+    }
+  }
+}
+
+template <int NT, int MT, int WAVES, typename XT>
+void launch_packed(const PackedArgs &a, hipStream_t st) {
+  constexpr int U = NT == 1 ? 8 : 4;
+  const int n_tiles = (a.N + 15) / 16;
+  const dim3 grid((n_tiles + NT - 1) / NT, (a.M + MT * 16 - 1) / (MT * 16));
+  hipLaunchKernelGGL((linear_skinny_packed_kernel<NT, MT, WAVES, U, XT>), grid, dim3(WAVES * 64), 0, st, a);
+}
+
+template <int NT, int MT, typename XT>
+void dispatch_packed_waves(const PackedArgs &a, int waves, hipStream_t st) {
+  if constexpr (NT * MT == 1) {
+    if (waves >= 16) return launch_packed<NT, MT, 16, XT>(a, st);
+  }
+  if constexpr (NT < 4) {
+    if (waves >= 8) return launch_packed<NT, MT, 8, XT>(a, st);
+  }
+  launch_packed<NT, MT, 4, XT>(a, st);
+}
+
+template <typename XT>
+void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  if (p.mt == 1) {
+    if (p.nt == 4)
+      dispatch_packed_waves<4, 1, XT>(a, p.waves, st);
+    else if (p.nt == 2)
+      dispatch_packed_waves<2, 1, XT>(a, p.waves, st);
+    else
+      dispatch_packed_waves<1, 1, XT>(a, p.waves, st);
+  } else {
+    if (p.nt == 2)
+      dispatch_packed_waves<2, 2, XT>(a, p.waves, st);
+    else
+      dispatch_packed_waves<1, 2, XT>(a, p.waves, st);
+  }
+}
+
 }  // namespace
 }  // namespace axhip
 
@@ -385,6 +537,57 @@ AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const 
     hipLaunchKernelGGL((linear_gemm_kernel<__half>), grid, dim3(kThreads), 0, st, a);
   else
     hipLaunchKernelGGL((linear_gemm_kernel<float>), grid, dim3(kThreads), 0, st, a);
+  return launch_status();
+}
+
+AXHIP_API size_t axhip_linear_f16_packed_bytes(int64_t N, int64_t K) {
+  if (N <= 0 || K <= 0) return 0;
+  const int64_t tiles = (N + 15) / 16, kc = (K + 31) / 32;
+  return static_cast<size_t>(tiles) * kc * 1024;
+}
+
+AXHIP_API int axhip_linear_f16_pack(const void *w, void *packed, int64_t N, int64_t K, axhip_stream stream) {
+  if (N <= 0 || K <= 0 || K % 8 != 0 || N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+  if (!w || !packed) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(packed)) & 15) return AXHIP_INVALID_PTR;
+  const int64_t tiles = (N + 15) / 16, kc = (K + 31) / 32;
+  const int64_t frags = tiles * kc * 64;
+  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>((frags + 255) / 256)), dim3(256), 0,
+                     as_stream(stream), static_cast<const __half *>(w), static_cast<__half *>(packed),
+                     static_cast<int>(N), static_cast<int>(K), static_cast<int>(kc), frags);
+  return launch_status();
+}
+
+AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *packed_w, const void *bias,
+                                      void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
+                                      axhip_stream stream) {
+  if (!is_float_dtype(x_dtype) || !is_float_dtype(out_dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (M < 0 || K <= 0 || N <= 0 || K % 8 != 0) return AXHIP_INVALID_ARGUMENT;
+  if (M > kSkinnyMaxM) return AXHIP_INVALID_ARGUMENT;  // larger M takes the row-major weight and the tiled GEMM
+  if (N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+  if (M == 0) return AXHIP_OK;
+  if (!x || !packed_w || !out) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed_w) | reinterpret_cast<uintptr_t>(out)) & 15)
+    return AXHIP_INVALID_PTR;
+  const SkinnyPlan p = plan_skinny(M, K, N);
+  PackedArgs a;
+  a.x = x;
+  a.wp = static_cast<const __half *>(packed_w);
+  a.bias = static_cast<const __half *>(bias);
+  a.out = out;
+  a.M = static_cast<int>(M);
+  a.K = static_cast<int>(K);
+  a.N = static_cast<int>(N);
+  a.KC = static_cast<int>((K + 31) / 32);
+  const int u = p.nt == 1 ? 8 : 4;
+  int cpw = (a.KC + p.waves - 1) / p.waves;
+  a.chunks_per_wave = (cpw + u - 1) / u * u;
+  a.out_f16 = out_dtype == AXHIP_FLOAT16;
+  hipStream_t st = as_stream(stream);
+  if (x_dtype == AXHIP_FLOAT16)
+    dispatch_packed<__half>(a, p, st);
+  else
+    dispatch_packed<float>(a, p, st);
   return launch_status();
 }
 

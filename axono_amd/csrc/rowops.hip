@@ -548,16 +548,17 @@ __global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restric
         best = s_val[w];
         bi = s_idx[w];
       }
-    g_argmax_val[row * kArgmaxParts + part] = best;
-    g_argmax_idx[row * kArgmaxParts + part] = bi;
-    __threadfence();
+    // agent-scope stores: written through, visible to a workgroup on another XCD (no L2 write-back)
+    __hip_atomic_store(&g_argmax_val[row * kArgmaxParts + part], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&g_argmax_idx[row * kArgmaxParts + part], static_cast<long long>(bi), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);  // both stores have completed before the ticket is taken
     const unsigned int t = atomicAdd(&g_argmax_ticket[row], 1u);
     s_last = (t == kArgmaxParts - 1);
     if (s_last) atomicExch(&g_argmax_ticket[row], 0u);
   }
   __syncthreads();
   if (!s_last || threadIdx.x >= 64) return;
-  __threadfence();
   // one wavefront: lane p takes part p (kArgmaxParts == 64)
   best = __hip_atomic_load(&g_argmax_val[row * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   bi = __hip_atomic_load(&g_argmax_idx[row * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

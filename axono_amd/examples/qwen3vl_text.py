@@ -90,6 +90,9 @@ class Qwen3VLTextDecoder(nn.Module):
         self._lib = _lib.load()
         for name, arr in weights.items():
             self._parameters[name] = _dev(arr, device)
+        # decode-sized Linear calls read packed copies of the weights (made once, here)
+        self._packed = {name: L.pack_linear_weight(t) for name, t in self._parameters.items()
+                        if name.endswith("_proj.weight") or name == "embed_tokens.weight"}
         self._inv_freq = _dev(inv_freq_table(cfg.rope_theta, cfg.head_dim), device)
         self._cache = nn.StaticKVCache(cfg.num_hidden_layers, batch, cfg.num_key_value_heads, max_len, cfg.head_dim,
                                        DataType.FLOAT16, device)
@@ -110,9 +113,17 @@ class Qwen3VLTextDecoder(nn.Module):
     def cache(self) -> nn.StaticKVCache:
         return self._cache
 
+    def _linear(self, x, name):
+        """x @ W^T: packed weights for decode-sized x, the row-major weight (tiled GEMM) otherwise."""
+        w = self._w(name)
+        rows = x.num_elements // w.shape[1]
+        if rows <= L.PACKED_MAX_ROWS:
+            return L.linear_packed(x, self._packed[name], w.shape[0])
+        return L.linear_nobias(x, w)
+
     def _mlp(self, xn, p):
-        gu = L.linear_nobias(xn, self._w(p + "mlp.gate_up_proj.weight"))
-        return L.linear_nobias(L.silu_mul_fused(gu, DataType.FLOAT16), self._w(p + "mlp.down_proj.weight"))
+        gu = self._linear(xn, p + "mlp.gate_up_proj.weight")
+        return self._linear(L.silu_mul_fused(gu, DataType.FLOAT16), p + "mlp.down_proj.weight")
 
     def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None):
         """One token per sequence.  ids INT64 [B]; pos INT64 [3,B]; appends to the cache at
@@ -128,21 +139,21 @@ class Qwen3VLTextDecoder(nn.Module):
         lens_now = self._lens_plus_one
         for i in range(cfg.num_hidden_layers):
             p = f"layers.{i}."
-            qkv = L.linear_nobias(xn, self._w(p + "self_attn.qkv_proj.weight"))
+            qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")
             kc, vc = cache.get(i)
             q = L.qkv_norm_rope_append(qkv, self._w(p + "self_attn.q_norm.weight"), self._w(p + "self_attn.k_norm.weight"),
                                        cfg.rms_norm_eps, pos, self._inv_freq, cfg.mrope_section, cache.seq_lens, kc, vc,
                                        cfg.num_attention_heads)
             attn = L.gqa_decode_attention_cache(q, kc, vc, lens_now, max_len, workspace=self._attn_ws)
-            attn_out = L.linear_nobias(attn.reshape([B, cfg.num_attention_heads * cfg.head_dim]),
-                                       self._w(p + "self_attn.o_proj.weight"))
+            attn_out = self._linear(attn.reshape([B, cfg.num_attention_heads * cfg.head_dim]),
+                                    p + "self_attn.o_proj.weight")
             h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                     DataType.FLOAT16)
             mlp_out = self._mlp(xn2, p)
             nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
             # h = h + mlp_out folded into the following RMSNorm (next layer's input norm / final norm)
             h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps, DataType.FLOAT16)
-        logits = L.linear_nobias(xn, self._w("embed_tokens.weight"))  # tied lm_head
+        logits = self._linear(xn, "embed_tokens.weight")  # tied lm_head
         return logits, L.argmax(logits)
 
     # ---- prefill -----------------------------------------------------------------------------
@@ -196,7 +207,7 @@ class Qwen3VLTextDecoder(nn.Module):
             # keep the normalised hidden state of the last position for the lm_head
             check(lib.axhip_memcpy_d2d(last_h.data_ptr + b * H * 2, xn.data_ptr + (S - 1) * H * 2, H * 2), "copy")
         self._cache.set_lengths(np.full(B, S, np.int32))
-        logits = L.linear_nobias(last_h, self._w("embed_tokens.weight"))
+        logits = self._linear(last_h, "embed_tokens.weight")
         return logits, L.argmax(logits)
 
     # ---- captured decode loop ------------------------------------------------------------------

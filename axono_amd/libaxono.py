@@ -378,6 +378,44 @@ def _linear_impl(x: Tensor, weight: Tensor, bias: Tensor | None, out_dtype: Data
     return out
 
 
+def pack_linear_weight(weight: Tensor) -> Tensor:
+    """FLOAT16 W [N,K] -> the packed (MFMA fragment order) copy that linear_packed reads.  Done once,
+    when a Linear's weights become resident fp16 (the build's extension of cast_linear_fp16)."""
+    op = "pack_linear_weight"
+    _need_hip(op, weight)
+    if weight.dtype != DataType.FLOAT16 or weight.ndim != 2:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    n, k = weight.shape
+    lib = _lib_()
+    nbytes = lib.axhip_linear_f16_packed_bytes(n, k)
+    packed = Tensor(DataType.FLOAT16, [nbytes // 2], weight.device, _zero=False)
+    check(lib.axhip_linear_f16_pack(weight.data_ptr, packed.data_ptr, n, k, current_stream()), op)
+    return packed
+
+
+def linear_packed(x: Tensor, packed: Tensor, n: int, bias: Tensor | None = None,
+                  out_dtype: DataType | None = None) -> Tensor:
+    """x (..., K) with at most 32 rows . packed W [n, K]^T (+ bias)."""
+    op = "linear"
+    has_b = bias is not None and bias.num_elements != 0
+    _need_hip(op, x, packed, bias if has_b else None)
+    if x.dtype not in _FLOATS or packed.dtype != DataType.FLOAT16 or x.ndim < 1:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    k = x.shape[-1]
+    rows = x.num_elements // k if k else 0
+    lib = _lib_()
+    if packed.num_bytes != lib.axhip_linear_f16_packed_bytes(n, k) or (has_b and bias.num_elements != n):
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    odt = DataType(out_dtype) if out_dtype is not None else DataType.FLOAT32
+    out = _new(odt, x.shape[:-1] + [n], x)
+    check(lib.axhip_linear_f16_packed(x.data_ptr, int(x.dtype), packed.data_ptr, bias.data_ptr if has_b else None,
+                                      out.data_ptr, int(odt), rows, k, n, current_stream()), op)
+    return out
+
+
+PACKED_MAX_ROWS = 32
+
+
 def linear(x: Tensor, weight: Tensor, bias: Tensor) -> Tensor:
     return _linear_impl(x, weight, bias)
 

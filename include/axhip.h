@@ -175,7 +175,8 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
 
 /* The split plan the launcher uses for these sizes (it depends on host-side sizes only), and a
  * measurement hook that overrides the heuristics: target_workgroups = resident workgroups to aim
- * for, force_splits > 0 fixes the split count; 0 restores a default.  No reference counterpart
+ * for (a negative value selects the single-launch form in which the last workgroup merges the
+ * splits), force_splits > 0 fixes the split count; 0 restores a default.  No reference counterpart
  * (the reference hard-codes min(256, ceil(L/64)), gqa.cu:158-160). */
 AXHIP_API void axhip_gqa_decode_plan(int B, int Hq, int Hkv, int max_len, int *n_splits, int *chunk);
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
@@ -296,6 +297,19 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
 AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const void *bias,
                                void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
                                void *workspace, size_t workspace_bytes, axhip_stream stream);
+
+/* Packed weights for skinny M.  axhip_linear_f16_pack re-orders a row-major FLOAT16 W [N,K] once
+ * into MFMA fragment order (1 KiB blocks of 16 rows x 32 K, consecutive along K; rows and K
+ * zero-padded to whole blocks) into a buffer of axhip_linear_f16_packed_bytes(N,K) bytes, so that
+ * every wavefront streams consecutive memory.  axhip_linear_f16_packed computes the same result as
+ * axhip_linear_f16 from it, for M <= 32.  The packing is the build's counterpart of what
+ * Module.cast_linear_fp16 does to a Linear's weights (axono/python/axono/nn/module.py:158-184): a
+ * one-off conversion into the resident format the inference kernels read. */
+AXHIP_API size_t axhip_linear_f16_packed_bytes(int64_t N, int64_t K);
+AXHIP_API int axhip_linear_f16_pack(const void *w, void *packed, int64_t N, int64_t K, axhip_stream stream);
+AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *packed_w, const void *bias,
+                                      void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
+                                      axhip_stream stream);
 
 /* ============================================================================================
  * Index operators of the decode step

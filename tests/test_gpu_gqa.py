@@ -152,16 +152,16 @@ def test_two_kernel_merge_mode_matches_fused_merge():
     k = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
     v = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
     want = port.gqa_decode_cache_native(q, k, v, lens)
+    two = gqa_decode(q, k, v, lens).astype(np.float32)       # default: split kernel + merge kernel
+    lib().axhip_gqa_decode_tune(-1, 0)                         # single launch, last workgroup merges
     fused = gqa_decode(q, k, v, lens).astype(np.float32)
-    lib().axhip_gqa_decode_tune(-1, 0)
-    two = gqa_decode(q, k, v, lens).astype(np.float32)
-    lib().axhip_gqa_decode_tune(0, 0)
-    assert np.abs(fused - want).max() <= TOL16 and np.abs(two - want).max() <= TOL16
-    assert np.all(fused[1] == 0) and np.all(two[1] == 0)
-    # repeated launches reuse the ticket counters: run the fused form several times
+    # repeated launches reuse the ticket counters: run the single-launch form several times
     for _ in range(3):
         again = gqa_decode(q, k, v, lens).astype(np.float32)
         np.testing.assert_array_equal(again, fused)
+    lib().axhip_gqa_decode_tune(0, 0)
+    assert np.abs(fused - want).max() <= TOL16 and np.abs(two - want).max() <= TOL16
+    assert np.all(fused[1] == 0) and np.all(two[1] == 0)
     # a single split and an empty sequence (the split-0 workgroup writes the zeros)
     lib().axhip_gqa_decode_tune(0, 1)
     one = gqa_decode(q, k, v, lens).astype(np.float32)

@@ -96,3 +96,44 @@ def test_error_codes():
     assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 60, 8, None, 0, None) == 1  # K % 8
     assert l.axhip_linear_f16(None, 2, None, None, None, 5, 4, 64, 8, None, 0, None) == 3  # x dtype
     assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 64, 8, None, 0, None) == 7  # null pointers
+
+
+@pytest.mark.parametrize("M", [1, 16, 32])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 4096)])
+def test_packed_weights_config4_shapes(M, K, N):
+    """The packed-weight kernels give the oracle's result and agree with the row-major path."""
+    rng = np.random.default_rng(M * 11 + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    out = gu.linear_f16_packed(x, w)
+    want = port.linear(x.astype(np.float32), w.astype(np.float32))
+    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
+    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag)
+    assert np.abs(out - gu.linear_f16(x, w)).max() <= 1e-4
+
+
+def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
+    rng = np.random.default_rng(8)
+    for (M, K, N) in [(3, 72, 50), (17, 136, 33), (32, 520, 130), (5, 8, 7), (16, 40, 16)]:
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        w = h16(0.05 * rng.standard_normal((N, K)))
+        b = h16(0.05 * rng.standard_normal(N))
+        want = port.linear(x.astype(np.float16).astype(np.float32), w.astype(np.float32), b.astype(np.float32))
+        np.testing.assert_allclose(gu.linear_f16_packed(x, w, b), want, rtol=0, atol=2e-5)
+        o16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16)
+        assert np.abs(o16.astype(np.float32) - want).max() <= 2e-3
+    l = gu.lib()
+    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 33, 64, 8, None) == 1  # M > 32
+    assert l.axhip_linear_f16_packed_bytes(17, 40) == 2 * 2 * 1024
+
+
+def test_packed_lm_head_M16():
+    rng = np.random.default_rng(98)
+    K, N = 2048, 151936
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    x = h16(rng.standard_normal((16, K)))
+    out = gu.linear_f16_packed(x, w)
+    cols = np.arange(0, N, 41)
+    want = port.linear(x.astype(np.float32), w[cols].astype(np.float32))
+    assert np.abs(out[:, cols] - want).max() <= 1e-4
+    assert np.abs(out[:, -7:] - port.linear(x.astype(np.float32), w[-7:].astype(np.float32))).max() <= 1e-4

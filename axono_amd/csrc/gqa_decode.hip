@@ -28,6 +28,7 @@ constexpr float kNegBig = -1.0e30f;   // "no key seen yet" in the log2 domain (f
 constexpr int kMaxSplits = 128;
 constexpr int kChunkAlign = 128;      // key ranges start on multiples of this
 constexpr int kMinChunk = 256;
+constexpr int kLongChunk = 1024;
 
 struct Tuning {
   int target_workgroups = 1024;  // 256 CUs x 4 resident workgroups
@@ -51,12 +52,23 @@ struct SplitPlan {
 // The key axis is cut into `n_splits` ranges of `chunk` keys.  The plan depends only on host-side
 // sizes so that a captured graph stays valid while the device-side lengths change.
 SplitPlan plan_splits(int B, int head_groups, int max_len) {
-  const long pairs = static_cast<long>(B) * head_groups;
-  long s = g_tuning.force_splits > 0
-               ? g_tuning.force_splits
-               : (g_tuning.target_workgroups + pairs - 1) / (pairs > 0 ? pairs : 1);
-  const long cap = (max_len + kMinChunk - 1) / kMinChunk;
-  if (s > cap) s = cap;
+  const long pairs = static_cast<long>(B) * head_groups > 0 ? static_cast<long>(B) * head_groups : 1;
+  long s;
+  if (g_tuning.force_splits > 0) {
+    s = g_tuning.force_splits;
+  } else {
+    // Measured on MI355X: a workgroup streams best over >= 1024 keys (prologue, LDS merge and the
+    // partial write are per workgroup), so aim for target_workgroups with chunks that long ...
+    s = (g_tuning.target_workgroups + pairs - 1) / pairs;
+    const long cap_long = max_len / kLongChunk > 0 ? max_len / kLongChunk : 1;
+    if (s > cap_long) s = cap_long;
+    // ... unless that leaves most of the 256 CUs idle: then shorter chunks, down to kMinChunk keys
+    if (pairs * s < g_tuning.target_workgroups / 2) {
+      s = (g_tuning.target_workgroups / 2 + pairs - 1) / pairs;
+      const long cap = (max_len + kMinChunk - 1) / kMinChunk;
+      if (s > cap) s = cap;
+    }
+  }
   if (s > kMaxSplits) s = kMaxSplits;
   if (s < 1) s = 1;
   long chunk = (max_len + s - 1) / s;
@@ -202,7 +214,7 @@ __device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t st
 }
 
 template <typename T, int D, int G, int U>
-__global__ __launch_bounds__(kThreads) void gqa_decode_split_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArgs a) {
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
   const int split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;

@@ -32,6 +32,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the headline split kernel, from the rocprofv3 --pmc runs recorded in
+# profiles/gqa_decode_split_B32_L8192_f16.md (a measured constant, not computed in this process)
+MEASURED_TRAFFIC_BYTES = 1075535872
 
 F16 = 4
 
@@ -265,9 +268,12 @@ def main():
                    "B": 32, "Hq": 16, "Hkv": 8, "D": 128, "L": 8192, "plan": wl.plan(),
                    "kv_buffers_rotated": len(wl.kv)},
         "pct_of_hbm_peak": round(100 * gbs_wall / HBM_PEAK_GBS, 2),
+        # achieved = algorithmic bytes per step / HIP-event time per step (split kernel + the 5 us merge
+        # kernel); traffic = HBM bytes per launch of the split kernel from rocprofv3 counters
+        # (FETCH_SIZE x 2.0000 + WRITE_SIZE x 1.0000, factors from a 1 GiB copy kernel), see profiles/
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gqa_decode_split_kernel<half,128,2> (+ merge)",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "gqa_decode_split_kernel<__half,128,2,8> (+ gqa_decode_merge_kernel)",
                      "avg_launch_us": round(ev_ms * 1e3, 2), "algorithmic_bytes": wl.bytes_per_step},
     }
     del wl

@@ -125,10 +125,12 @@ class Qwen3VLTextDecoder(nn.Module):
         gu = self._linear(xn, p + "mlp.gate_up_proj.weight")
         return self._linear(L.silu_mul_fused(gu, DataType.FLOAT16), p + "mlp.down_proj.weight")
 
-    def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None):
+    def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None, trace: list | None = None):
         """One token per sequence.  ids INT64 [B]; pos INT64 [3,B]; appends to the cache at
         cache.seq_lens and attends over seq_lens + 1 keys.  Returns (logits FLOAT32 [B,V], next ids
-        INT64 [B]).  Does not advance the lengths."""
+        INT64 [B]).  Does not advance the lengths.  `trace`, if given, receives the residual stream
+        entering every layer and the one leaving the last (FLOAT32 [B,H] tensors), for layer-wise
+        comparison with a reference evaluation."""
         cfg = self._cfg
         B = self._batch
         cache = self._cache
@@ -139,6 +141,8 @@ class Qwen3VLTextDecoder(nn.Module):
         lens_now = self._lens_plus_one
         for i in range(cfg.num_hidden_layers):
             p = f"layers.{i}."
+            if trace is not None:
+                trace.append(h)
             qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")
             kc, vc = cache.get(i)
             q = L.qkv_norm_rope_append(qkv, self._w(p + "self_attn.q_norm.weight"), self._w(p + "self_attn.k_norm.weight"),
@@ -153,6 +157,8 @@ class Qwen3VLTextDecoder(nn.Module):
             nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
             # h = h + mlp_out folded into the following RMSNorm (next layer's input norm / final norm)
             h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps, DataType.FLOAT16)
+        if trace is not None:
+            trace.append(h)
         logits = self._linear(xn, "embed_tokens.weight")  # tied lm_head
         return logits, L.argmax(logits)
 

@@ -163,28 +163,47 @@ def cpu_decode_step_hook(cfg, weights, model, first, pos, batch, max_len, log):
         cpu.k[i][:] = kc.numpy()
         cpu.v[i][:] = vc.numpy()
     cpu.lens[:] = ctx
-    # device: one eager step, then rewind
+    # device: one eager step with the residual stream of every layer kept, then rewind
     state = (model._ids.numpy().copy(), model._pos.numpy().copy(), model.cache.seq_lens.numpy().copy())
-    g_logits, g_next = model._step_fn()
+    trace = []
+    model._lens_plus_one.copy_from_numpy((state[2] + 1).astype(np.int32))
+    g_logits, g_next = model.decode_forward(model._ids, model._pos, trace=trace)
     g_logits, g_next = g_logits.to_numpy().copy(), g_next.to_numpy().copy()
-    model._ids.copy_from_numpy(state[0])
-    model._pos.copy_from_numpy(state[1])
-    model.cache.seq_lens.copy_from_numpy(state[2])
+    h_gpu = [t.to_numpy().copy() for t in trace]
+    del trace
     for name in list(weights):  # widen the weights outside the timed region
         if weights[name].dtype == np.float16:
             cpu.W(name)
+    # (1) free-running CPU step, timed: the baseline, and end-to-end logits
+    snap = [(cpu.k[i][:, :, ctx].copy(), cpu.v[i][:, :, ctx].copy()) for i in range(cfg.num_hidden_layers)]
     t0 = time.perf_counter()
     c_logits, c_next = cpu.decode_step(first, pos)
     cpu_s = time.perf_counter() - t0
     err = float(np.abs(g_logits - c_logits).max())
     chosen = c_logits[np.arange(batch), g_next]
-    agree = bool(np.all(chosen >= c_logits.max(-1) - 4e-3))
-    log(f"[decode] CPU restatement: one step in {cpu_s:.1f} s ({batch / cpu_s:.2f} tok/s, {oracle.port.num_threads()} threads); "
-        f"logits max abs err {err:.2e}, |logits| max {np.abs(c_logits).max():.2f}, greedy tokens agree: {agree}")
+    agree = bool(np.all(chosen >= c_logits.max(-1) - 2e-2))
+    # (2) layer-wise, every layer evaluated from the device's own input to that layer
+    cpu.lens[:] = ctx
+    for i, (kk, vv) in enumerate(snap):
+        cpu.k[i][:, :, ctx], cpu.v[i][:, :, ctx] = kk, vv
+    outs, tf_logits = cpu.decode_layers_teacher_forced(h_gpu, pos)
+    layer_err = max(float(np.abs(outs[i] - h_gpu[i + 1]).max()) for i in range(cfg.num_hidden_layers))
+    h_abs = max(float(np.abs(h).max()) for h in h_gpu)
+    tf_logit_err = float(np.abs(tf_logits - g_logits).max())
+    log(f"[decode] CPU restatement: one step in {cpu_s:.1f} s ({batch / cpu_s:.2f} tok/s, {oracle.port.num_threads()} threads)")
+    log(f"[decode] parity, each layer on identical inputs: max abs err of the residual stream {layer_err:.2e} "
+        f"(|h| max {h_abs:.1f}), logits from the same final state {tf_logit_err:.2e}; "
+        f"free-running end to end: logits {err:.2e} (|logits| max {np.abs(c_logits).max():.2f}), greedy tokens agree: {agree}")
     cpu.drop_cache()
     base = {"value": round(batch / cpu_s, 3), "unit": "tok/s", "cores": oracle.port.num_threads(), "kind": "port",
             "sample": f"1 decode step (batch {batch}, context {ctx}) of the C restatement from the post-prefill cache"}
-    par = {"logits_max_abs_err": err, "logits_abs_max": float(np.abs(c_logits).max()), "greedy_tokens_agree": agree}
+    par = {"per_layer_max_abs_err_identical_inputs": layer_err, "residual_abs_max": h_abs,
+           "logits_max_abs_err_identical_final_state": tf_logit_err,
+           "logits_max_abs_err_free_running": err, "logits_abs_max": float(np.abs(c_logits).max()),
+           "greedy_tokens_agree": agree,
+           "note": "fp16 storage points (activation entering each Linear, q, KV cache) round on different "
+                   "sides of an fp16 boundary for a few elements when two correct pipelines differ by 1e-7; "
+                   "free-running, these flips compound over 28 layers, layer-wise they cannot"}
     return {"cpu_baseline": base, "parity": par}
 
 

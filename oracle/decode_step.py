@@ -77,6 +77,25 @@ class OracleDecoder:
         # h + mlp_out, then the next RMSNorm: the reference does add (model.py:435) then rms_norm (:420 / :485)
         return ops.add_rms_norm(mlp_out, h, self.w[nxt], cfg.rms_norm_eps)
 
+    def decode_layers_teacher_forced(self, h_in, pos3):
+        """Layer-wise check of one decode step: layer i is evaluated from the residual stream the
+        build under test had at that layer's input (h_in[i], FLOAT32 [B,H]); returns the list of
+        residual streams each layer produces (to compare with h_in[i+1]) and the logits computed from
+        h_in[-1].  Each layer is then compared on identical inputs, so roundings that fall on
+        different sides of an fp16 boundary cannot compound through the depth of the model."""
+        cfg, ops = self.cfg, self.ops
+        rows_b, rows_t = np.arange(self.B), self.lens.copy()
+        outs = []
+        for i in range(cfg.num_hidden_layers):
+            h = np.asarray(h_in[i], np.float32)
+            wname = f"layers.{i}.input_layernorm.weight"
+            xn = ops.rms_norm(h, self.w[wname], cfg.rms_norm_eps)
+            h_next, _ = self._layer(i, h, xn, np.ascontiguousarray(pos3, dtype=np.int64), rows_b, rows_t)
+            outs.append(h_next)
+        self.lens += 1
+        xn = ops.rms_norm(np.asarray(h_in[-1], np.float32), self.w["norm.weight"], cfg.rms_norm_eps)
+        return outs, self._linear(xn, "embed_tokens.weight")
+
     def forward_rows(self, ids, pos3, rows_b, rows_t):
         cfg, ops = self.cfg, self.ops
         h = ops.embedding(np.asarray(ids, np.int64), self.W("embed_tokens.weight"))

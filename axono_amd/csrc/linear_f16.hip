@@ -356,16 +356,29 @@ struct PackedArgs {
   int M, K, N, KC, chunks_per_wave, out_f16;
 };
 
+// x fragments.  Loading the MFMA "B" fragments straight from global memory is a 16-row gather (64
+// bytes per row per instruction).  Instead, every iteration a wavefront copies the x columns it
+// needs next (MT*16 rows x U*32 columns) into a private LDS strip with coalesced 16-byte loads,
+// converting fp32 to fp16 on the way, and reads the fragments from LDS.  The strip has no padding;
+// the 16-byte unit index is XOR-ed with the row so that the 16 rows of a fragment read fall into
+// 16 different bank groups.
 template <int NT, int MT, int WAVES, int U, typename XT>
 __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(PackedArgs a) {
+  constexpr int ROWS = MT * 16;
+  constexpr int UNITS = U * 4;                 // 16-byte units per strip row
+  constexpr int STRIP_HALVES = ROWS * U * 32;  // per wavefront
+  constexpr int RED_BYTES = (WAVES - 1) * NT * MT * 64 * 16;
+  constexpr int STRIP_BYTES = WAVES * STRIP_HALVES * 2;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[STRIP_BYTES > RED_BYTES ? STRIP_BYTES : RED_BYTES];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
   const int tile0 = blockIdx.x * NT;
   const int n_tiles = (a.N + 15) / 16;
-  const int m_base = blockIdx.y * (MT * 16);
+  const int m_base = blockIdx.y * ROWS;
   const int c_begin = wave * a.chunks_per_wave;
   const int c_end = min(c_begin + a.chunks_per_wave, a.KC);
   const XT *x = static_cast<const XT *>(a.x);
+  _Float16 *strip = reinterpret_cast<_Float16 *>(smem) + wave * STRIP_HALVES;
 
   float4_t acc[NT][MT];
 #pragma unroll
@@ -380,28 +393,39 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
     wok[t] = tile0 + t < n_tiles;
     wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + lane * 8;
   }
-  const XT *xrow[MT];
-  bool xok[MT];
-#pragma unroll
-  for (int u = 0; u < MT; ++u) {
-    const int m = m_base + u * 16 + r;
-    xok[u] = m < a.M;
-    xrow[u] = x + static_cast<int64_t>(xok[u] ? m : 0) * a.K + g * 8;
-  }
 
   for (int c = c_begin; c < c_end; c += U) {
     half8_t af[NT][U], bf[MT][U];
 #pragma unroll
     for (int j = 0; j < U; ++j) {
-      const int cc = c + j;
-      const bool in = cc < c_end;
+      const bool in = c + j < c_end;
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        af[t][j] = (in && wok[t]) ? load_h8(wt[t] + static_cast<int64_t>(cc) * 512) : zero_h8();
-      const bool kin = in && (cc * 32 + g * 8 + 8 <= a.K);
-#pragma unroll
-      for (int u = 0; u < MT; ++u) bf[u][j] = (kin && xok[u]) ? load_h8(xrow[u] + cc * 32) : zero_h8();
+        af[t][j] = (in && wok[t]) ? load_h8(wt[t] + static_cast<int64_t>(c + j) * 512) : zero_h8();
     }
+    // stage x[m_base .. +ROWS)[32c .. 32(c+U)): ROWS*UNITS vectors, 64 per pass
+    half8_t xv[ROWS * UNITS / 64];
+#pragma unroll
+    for (int p = 0; p < ROWS * UNITS / 64; ++p) {
+      const int v = p * 64 + lane;
+      const int row = v / UNITS, unit = v % UNITS;
+      const int m = m_base + row, k = c * 32 + unit * 8;
+      xv[p] = (m < a.M && k + 8 <= a.K && c + unit / 4 < c_end) ? load_h8(x + static_cast<int64_t>(m) * a.K + k)
+                                                               : zero_h8();
+    }
+#pragma unroll
+    for (int p = 0; p < ROWS * UNITS / 64; ++p) {
+      const int v = p * 64 + lane;
+      const int row = v / UNITS, unit = v % UNITS;
+      *reinterpret_cast<half8_t *>(strip + row * (U * 32) + ((unit ^ (row & (UNITS - 1) & 15)) * 8)) = xv[p];
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j)
+#pragma unroll
+      for (int u = 0; u < MT; ++u) {
+        const int row = u * 16 + r, unit = j * 4 + g;
+        bf[u][j] = *reinterpret_cast<const half8_t *>(strip + row * (U * 32) + ((unit ^ (row & (UNITS - 1) & 15)) * 8));
+      }
 #pragma unroll
     for (int j = 0; j < U; ++j)
 #pragma unroll
@@ -411,12 +435,14 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
           acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[t][j], bf[u][j], acc[t][u], 0, 0, 0);
   }
 
-  __shared__ float4_t red[WAVES - 1][NT * MT][64];
+  // add the K slices: the x strips are dead by now, their LDS is reused for the fragments
+  __syncthreads();
+  float4_t *red = reinterpret_cast<float4_t *>(smem);  // [WAVES-1][NT*MT][64]
   if (wave > 0) {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int u = 0; u < MT; ++u) red[wave - 1][t * MT + u][lane] = acc[t][u];
+      for (int u = 0; u < MT; ++u) red[((wave - 1) * NT * MT + t * MT + u) * 64 + lane] = acc[t][u];
   }
   __syncthreads();
   if (wave != 0) return;
@@ -432,16 +458,23 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
     for (int u = 0; u < MT; ++u) {
       float4_t s = acc[t][u];
 #pragma unroll
-      for (int w = 0; w < WAVES - 1; ++w) s += red[w][t * MT + u][lane];
+      for (int w = 0; w < WAVES - 1; ++w) s += red[(w * NT * MT + t * MT + u) * 64 + lane];
       const float v[4] = {s[0], s[1], s[2], s[3]};
       store_out4(o, m_base + u * 16 + r, (tile0 + t) * 16 + 4 * g, v);
     }
   }
 }
 
+// Chunks of 32 K per loop iteration: bounded by the LDS the x strips take (WAVES * MT*16 * U*64 bytes
+// must stay within 64 KiB).
+template <int NT, int MT, int WAVES>
+constexpr int packed_unroll() {
+  return (WAVES * MT >= 16) ? 4 : ((NT == 1 && WAVES * MT <= 8) ? 8 : 4);
+}
+
 template <int NT, int MT, int WAVES, typename XT>
 void launch_packed(const PackedArgs &a, hipStream_t st) {
-  constexpr int U = NT == 1 ? 8 : 4;
+  constexpr int U = packed_unroll<NT, MT, WAVES>();
   const int n_tiles = (a.N + 15) / 16;
   const dim3 grid((n_tiles + NT - 1) / NT, (a.M + MT * 16 - 1) / (MT * 16));
   hipLaunchKernelGGL((linear_skinny_packed_kernel<NT, MT, WAVES, U, XT>), grid, dim3(WAVES * 64), 0, st, a);
@@ -579,9 +612,9 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
   a.K = static_cast<int>(K);
   a.N = static_cast<int>(N);
   a.KC = static_cast<int>((K + 31) / 32);
-  const int u = p.nt == 1 ? 8 : 4;
+  // any multiple of 4 works with every unroll the kernels use (a short last iteration is masked)
   int cpw = (a.KC + p.waves - 1) / p.waves;
-  a.chunks_per_wave = (cpw + u - 1) / u * u;
+  a.chunks_per_wave = (cpw + 3) / 4 * 4;
   a.out_f16 = out_dtype == AXHIP_FLOAT16;
   hipStream_t st = as_stream(stream);
   if (x_dtype == AXHIP_FLOAT16)

@@ -164,7 +164,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False):
                 off += n
             if packed:
                 pb = DeviceBuffer(lib.axhip_linear_f16_packed_bytes(N, K))
-                check(lib.axhip_linear_f16_pack(wb.ptr, pb.ptr, N, K, None), "pack")
+                check(lib.axhip_linear_f16_pack(wb.ptr, pb.ptr, N, K, 0, None), "pack")
                 check(lib.axhip_synchronize(), "sync")
                 wb = pb
             ws_.append(wb)
@@ -181,7 +181,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False):
                 wb = ws_[st["i"] % n_rot]
                 st["i"] += 1
                 if packed:
-                    check(lib.axhip_linear_f16_packed(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, None), "linear")
+                    check(lib.axhip_linear_f16_packed(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, 0, None), "linear")
                 else:
                     check(lib.axhip_linear_f16(x.ptr, F16, wb.ptr, None, out.ptr, F32, M, K, N, ws.ptr, wsb, None), "linear")
 
@@ -204,6 +204,9 @@ def main(argv=None):
     ap.add_argument("--ragged", action="store_true")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--target-wgs", type=int, default=0)
+    ap.add_argument("--nt", type=int, default=0, help="linear: 16-row groups of W per wavefront (1, 2, 4)")
+    ap.add_argument("--waves", type=int, default=0, help="linear: wavefronts (K slices) per workgroup (4, 8, 16)")
+    ap.add_argument("--M", type=int, default=0, help="linear: only this row count")
     args = ap.parse_args(argv)
     lib = _lib.load()
     if _lib.device_count() < 1:
@@ -225,9 +228,12 @@ def main(argv=None):
     elif args.what == "rowops":
         bench_rowops(lib)
     elif args.what == "linear":
-        bench_linear(lib)
+        lib.axhip_linear_f16_tune(0, args.nt, args.waves)
+        bench_linear(lib, Ms=(args.M,) if args.M else (1, 16, 32, 512))
     elif args.what == "linear-packed":
-        bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)], packed=True)
+        lib.axhip_linear_f16_tune(0, args.nt, args.waves)
+        bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)],
+                     Ms=(args.M,) if args.M else (1, 16, 32), packed=True)
 
 
 if __name__ == "__main__":

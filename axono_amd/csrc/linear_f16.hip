@@ -40,17 +40,20 @@ struct SkinnyPlan {
 // through LDS, so one launch finishes the product.  Small N gets more wavefronts per workgroup
 // (down to 128 of K each) so that the launch still fills the chip.
 SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
+  // Measured at M = 16 on MI355X (packed weights): two row tiles per wavefront win once N >= 8192
+  // (lm_head 2048 -> 151936: 109 us with NT=2 / 8 wavefronts against 125 us with NT=4 / 4), one tile
+  // with 8-16 K slices wins for the small matrices; every kernel costs about 3 us plus its bytes at
+  // 5.5-5.7 TB/s.
   SkinnyPlan p;
   p.mt = M <= 16 ? 1 : 2;
   if (g_lin.force_nt > 0)
     p.nt = g_lin.force_nt;
-  else if (p.mt == 2)
-    p.nt = 2;
   else
-    p.nt = N >= 32768 ? 4 : (N >= 8192 ? 2 : 1);
+    p.nt = (p.mt == 2 || N >= 8192) ? 2 : 1;
   if (p.mt == 2 && p.nt > 2) p.nt = 2;
   const int64_t ntiles = (N + p.nt * 16 - 1) / (p.nt * 16);
   int64_t want = g_lin.force_waves > 0 ? g_lin.force_waves : (g_lin.target_waves + ntiles - 1) / ntiles;
+  if (g_lin.force_waves == 0 && want < 8) want = 8;
   int waves = 4;
   while (waves < want && waves < kMaxWaves) waves *= 2;
   while (waves > 4 && K / waves < 128) waves /= 2;
@@ -333,14 +336,16 @@ __global__ __launch_bounds__(kThreads) void linear_gemm_kernel(LinearArgs a) {
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void pack_weight_kernel(const __half *__restrict__ w,
                                                           __half *__restrict__ packed, int N, int K,
-                                                          int KC, int64_t frags) {
+                                                          int KC, int64_t frags, int glu) {
   const int64_t f = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (f >= frags) return;
   const int lane = static_cast<int>(f & 63);
   const int64_t blk = f >> 6;
   const int c = static_cast<int>(blk % KC);
   const int64_t t = blk / KC;
-  const int64_t row = t * 16 + (lane & 15);
+  // glu: packed tile 2j takes rows [16j, 16j+16) of the first half of W (gate), tile 2j+1 the same
+  // rows of the second half (up)
+  const int64_t row = glu ? (t & 1) * (N / 2) + (t >> 1) * 16 + (lane & 15) : t * 16 + (lane & 15);
   const int k = c * 32 + (lane >> 4) * 8;
   Vec16 v;
   v.w[0] = v.w[1] = v.w[2] = v.w[3] = 0u;
@@ -354,6 +359,7 @@ struct PackedArgs {
   const __half *bias;
   void *out;
   int M, K, N, KC, chunks_per_wave, out_f16;
+  int glu;  // rows come in tile pairs (gate tile, up tile): the epilogue stores silu(gate) * up, N/2 columns
 };
 
 // x fragments.  Loading the MFMA "B" fragments straight from global memory is a 16-row gather (64
@@ -450,8 +456,9 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
   o.bias = a.bias;
   o.out = a.out;
   o.M = a.M;
-  o.N = a.N;
+  o.N = a.glu ? a.N / 2 : a.N;
   o.out_f16 = a.out_f16;
+  float4_t tot[NT][MT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -459,10 +466,34 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
       float4_t s = acc[t][u];
 #pragma unroll
       for (int w = 0; w < WAVES - 1; ++w) s += red[(w * NT * MT + t * MT + u) * 64 + lane];
-      const float v[4] = {s[0], s[1], s[2], s[3]};
-      store_out4(o, m_base + u * 16 + r, (tile0 + t) * 16 + 4 * g, v);
+      tot[t][u] = s;
     }
   }
+  if constexpr (NT % 2 == 0) {
+    if (a.glu) {
+      // tile 2j holds gate rows, tile 2j+1 the up rows of the same 16 output columns
+#pragma unroll
+      for (int t = 0; t < NT; t += 2)
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+          float v[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float gt = tot[t][u][q];
+            v[q] = gt / (1.0f + expf(-gt)) * tot[t + 1][u][q];
+          }
+          store_out4(o, m_base + u * 16 + r, ((tile0 + t) / 2) * 16 + 4 * g, v);
+        }
+      return;
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+      const float v[4] = {tot[t][u][0], tot[t][u][1], tot[t][u][2], tot[t][u][3]};
+      store_out4(o, m_base + u * 16 + r, (tile0 + t) * 16 + 4 * g, v);
+    }
 }
 
 // Chunks of 32 K per loop iteration: bounded by the LDS the x strips take (WAVES * MT*16 * U*64 bytes
@@ -579,31 +610,39 @@ AXHIP_API size_t axhip_linear_f16_packed_bytes(int64_t N, int64_t K) {
   return static_cast<size_t>(tiles) * kc * 1024;
 }
 
-AXHIP_API int axhip_linear_f16_pack(const void *w, void *packed, int64_t N, int64_t K, axhip_stream stream) {
+AXHIP_API int axhip_linear_f16_pack(const void *w, void *packed, int64_t N, int64_t K, int glu,
+                                    axhip_stream stream) {
   if (N <= 0 || K <= 0 || K % 8 != 0 || N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+  if (glu && N % 32 != 0) return AXHIP_INVALID_ARGUMENT;  // both halves must be whole 16-row tiles
   if (!w || !packed) return AXHIP_INVALID_PTR;
   if ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(packed)) & 15) return AXHIP_INVALID_PTR;
   const int64_t tiles = (N + 15) / 16, kc = (K + 31) / 32;
   const int64_t frags = tiles * kc * 64;
   hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>((frags + 255) / 256)), dim3(256), 0,
                      as_stream(stream), static_cast<const __half *>(w), static_cast<__half *>(packed),
-                     static_cast<int>(N), static_cast<int>(K), static_cast<int>(kc), frags);
+                     static_cast<int>(N), static_cast<int>(K), static_cast<int>(kc), frags, glu ? 1 : 0);
   return launch_status();
 }
 
 AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *packed_w, const void *bias,
-                                      void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
+                                      void *out, int out_dtype, int64_t M, int64_t K, int64_t N, int glu,
                                       axhip_stream stream) {
   if (!is_float_dtype(x_dtype) || !is_float_dtype(out_dtype)) return AXHIP_UNSUPPORTED_TYPE;
   if (M < 0 || K <= 0 || N <= 0 || K % 8 != 0) return AXHIP_INVALID_ARGUMENT;
+  if (glu && (N % 32 != 0 || bias)) return AXHIP_INVALID_ARGUMENT;
   if (M > kSkinnyMaxM) return AXHIP_INVALID_ARGUMENT;  // larger M takes the row-major weight and the tiled GEMM
   if (N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
   if (M == 0) return AXHIP_OK;
   if (!x || !packed_w || !out) return AXHIP_INVALID_PTR;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed_w) | reinterpret_cast<uintptr_t>(out)) & 15)
     return AXHIP_INVALID_PTR;
-  const SkinnyPlan p = plan_skinny(M, K, N);
+  SkinnyPlan p = plan_skinny(M, K, N);
+  if (glu && p.nt % 2 != 0) {  // the gated epilogue needs gate and up tiles in the same wavefront
+    p.nt = 2;
+    if (p.waves > 8) p.waves = 8;
+  }
   PackedArgs a;
+  a.glu = glu ? 1 : 0;
   a.x = x;
   a.wp = static_cast<const __half *>(packed_w);
   a.bias = static_cast<const __half *>(bias);

@@ -91,7 +91,9 @@ class Qwen3VLTextDecoder(nn.Module):
         for name, arr in weights.items():
             self._parameters[name] = _dev(arr, device)
         # decode-sized Linear calls read packed copies of the weights (made once, here)
-        self._packed = {name: L.pack_linear_weight(t) for name, t in self._parameters.items()
+        # (gate+up weights are packed as alternating gate / up tiles: the kernel's epilogue applies SiLU-mul)
+        self._packed = {name: L.pack_linear_weight(t, glu=name.endswith("gate_up_proj.weight"))
+                        for name, t in self._parameters.items()
                         if name.endswith("_proj.weight") or name == "embed_tokens.weight"}
         self._inv_freq = _dev(inv_freq_table(cfg.rope_theta, cfg.head_dim), device)
         self._cache = nn.StaticKVCache(cfg.num_hidden_layers, batch, cfg.num_key_value_heads, max_len, cfg.head_dim,
@@ -122,8 +124,14 @@ class Qwen3VLTextDecoder(nn.Module):
         return L.linear_nobias(x, w)
 
     def _mlp(self, xn, p):
-        gu = self._linear(xn, p + "mlp.gate_up_proj.weight")
-        return self._linear(L.silu_mul_fused(gu, DataType.FLOAT16), p + "mlp.down_proj.weight")
+        name = p + "mlp.gate_up_proj.weight"
+        w = self._w(name)
+        if xn.num_elements // w.shape[1] <= L.PACKED_MAX_ROWS:
+            # decode: the gate+up Linear applies SiLU-mul in its epilogue and stores fp16
+            act = L.linear_packed(xn, self._packed[name], w.shape[0], out_dtype=DataType.FLOAT16, glu=True)
+        else:
+            act = L.silu_mul_fused(L.linear_nobias(xn, w), DataType.FLOAT16)
+        return self._linear(act, p + "mlp.down_proj.weight")
 
     def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None, trace: list | None = None):
         """One token per sequence.  ids INT64 [B]; pos INT64 [3,B]; appends to the cache at

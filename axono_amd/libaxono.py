@@ -378,7 +378,7 @@ def _linear_impl(x: Tensor, weight: Tensor, bias: Tensor | None, out_dtype: Data
     return out
 
 
-def pack_linear_weight(weight: Tensor) -> Tensor:
+def pack_linear_weight(weight: Tensor, glu: bool = False) -> Tensor:
     """FLOAT16 W [N,K] -> the packed (MFMA fragment order) copy that linear_packed reads.  Done once,
     when a Linear's weights become resident fp16 (the build's extension of cast_linear_fp16)."""
     op = "pack_linear_weight"
@@ -389,13 +389,14 @@ def pack_linear_weight(weight: Tensor) -> Tensor:
     lib = _lib_()
     nbytes = lib.axhip_linear_f16_packed_bytes(n, k)
     packed = Tensor(DataType.FLOAT16, [nbytes // 2], weight.device, _zero=False)
-    check(lib.axhip_linear_f16_pack(weight.data_ptr, packed.data_ptr, n, k, current_stream()), op)
+    check(lib.axhip_linear_f16_pack(weight.data_ptr, packed.data_ptr, n, k, 1 if glu else 0, current_stream()), op)
     return packed
 
 
 def linear_packed(x: Tensor, packed: Tensor, n: int, bias: Tensor | None = None,
-                  out_dtype: DataType | None = None) -> Tensor:
-    """x (..., K) with at most 32 rows . packed W [n, K]^T (+ bias)."""
+                  out_dtype: DataType | None = None, glu: bool = False) -> Tensor:
+    """x (..., K) with at most 32 rows . packed W [n, K]^T (+ bias).  glu: W was packed as a fused
+    [gate ; up] projection and the result is silu(gate) * up, (..., n/2)."""
     op = "linear"
     has_b = bias is not None and bias.num_elements != 0
     _need_hip(op, x, packed, bias if has_b else None)
@@ -407,9 +408,9 @@ def linear_packed(x: Tensor, packed: Tensor, n: int, bias: Tensor | None = None,
     if packed.num_bytes != lib.axhip_linear_f16_packed_bytes(n, k) or (has_b and bias.num_elements != n):
         raise AxhipError(op, Status.SHAPE_MISMATCH)
     odt = DataType(out_dtype) if out_dtype is not None else DataType.FLOAT32
-    out = _new(odt, x.shape[:-1] + [n], x)
+    out = _new(odt, x.shape[:-1] + [n // 2 if glu else n], x)
     check(lib.axhip_linear_f16_packed(x.data_ptr, int(x.dtype), packed.data_ptr, bias.data_ptr if has_b else None,
-                                      out.data_ptr, int(odt), rows, k, n, current_stream()), op)
+                                      out.data_ptr, int(odt), rows, k, n, 1 if glu else 0, current_stream()), op)
     return out
 
 

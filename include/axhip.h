@@ -304,11 +304,16 @@ AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const 
  * every wavefront streams consecutive memory.  axhip_linear_f16_packed computes the same result as
  * axhip_linear_f16 from it, for M <= 32.  The packing is the build's counterpart of what
  * Module.cast_linear_fp16 does to a Linear's weights (axono/python/axono/nn/module.py:158-184): a
- * one-off conversion into the resident format the inference kernels read. */
+ * one-off conversion into the resident format the inference kernels read.
+ * glu != 0 (both calls): W is a fused [gate ; up] projection (N = 2*I rows, N % 32 == 0); the rows
+ * are packed as alternating gate / up tiles and the kernel stores silu(gate) * up, an [M, N/2]
+ * result, instead of the [M, N] projection (same arithmetic as axhip_silu_mul on the two halves;
+ * no bias). */
 AXHIP_API size_t axhip_linear_f16_packed_bytes(int64_t N, int64_t K);
-AXHIP_API int axhip_linear_f16_pack(const void *w, void *packed, int64_t N, int64_t K, axhip_stream stream);
+AXHIP_API int axhip_linear_f16_pack(const void *w, void *packed, int64_t N, int64_t K, int glu,
+                                    axhip_stream stream);
 AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *packed_w, const void *bias,
-                                      void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
+                                      void *out, int out_dtype, int64_t M, int64_t K, int64_t N, int glu,
                                       axhip_stream stream);
 
 /* ============================================================================================

@@ -159,19 +159,20 @@ def linear_f16(x, w, bias=None, out_dtype=np.float32):
     return do.download(out_dtype, (M, N))
 
 
-def linear_f16_packed(x, w, bias=None, out_dtype=np.float32):
+def linear_f16_packed(x, w, bias=None, out_dtype=np.float32, glu=False):
     M, K = x.shape
     N = w.shape[0]
     l = lib()
     dx, dw = dev(x), dev(w)
     dp = DeviceBuffer(l.axhip_linear_f16_packed_bytes(N, K))
-    _run("axhip_linear_f16_pack", dw.ptr, dp.ptr, N, K, None)
+    _run("axhip_linear_f16_pack", dw.ptr, dp.ptr, N, K, int(glu), None)
     db = dev(bias) if bias is not None else None
-    do = DeviceBuffer(M * N * np.dtype(out_dtype).itemsize)
+    n_out = N // 2 if glu else N
+    do = DeviceBuffer(M * n_out * np.dtype(out_dtype).itemsize)
     _run("axhip_linear_f16_packed", dx.ptr, dt(x), dp.ptr, db.ptr if db else None, do.ptr,
-         dt(np.empty(0, out_dtype)), M, K, N, None)
+         dt(np.empty(0, out_dtype)), M, K, N, int(glu), None)
     synchronize()
-    return do.download(out_dtype, (M, N))
+    return do.download(out_dtype, (M, n_out))
 
 
 def embedding(ids, table):

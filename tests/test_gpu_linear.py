@@ -12,6 +12,7 @@ import pytest
 from oracle import port
 
 import gpu_util as gu
+import gpu_util as gu_mod
 
 pytestmark = pytest.mark.gpu
 G = np.load(os.path.join(os.path.dirname(__file__), "golden", "decode_path_golden.npz"))
@@ -123,7 +124,7 @@ def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
         o16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16)
         assert np.abs(o16.astype(np.float32) - want).max() <= 2e-3
     l = gu.lib()
-    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 33, 64, 8, None) == 1  # M > 32
+    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 33, 64, 8, 0, None) == 1  # M > 32
     assert l.axhip_linear_f16_packed_bytes(17, 40) == 2 * 2 * 1024
 
 
@@ -137,3 +138,18 @@ def test_packed_lm_head_M16():
     want = port.linear(x.astype(np.float32), w[cols].astype(np.float32))
     assert np.abs(out[:, cols] - want).max() <= 1e-4
     assert np.abs(out[:, -7:] - port.linear(x.astype(np.float32), w[-7:].astype(np.float32))).max() <= 1e-4
+
+
+@pytest.mark.parametrize("M,K,I", [(16, 2048, 6144), (1, 2048, 6144), (32, 256, 96), (5, 72, 32)])
+def test_packed_gate_up_with_silu_mul_epilogue(M, K, I):
+    """Fused [gate ; up] projection with the SiLU-mul epilogue against Linear then silu_mul of the oracle."""
+    rng = np.random.default_rng(M + K + I)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((2 * I, K)))
+    gu = port.linear(x.astype(np.float32), w.astype(np.float32))
+    want = port.silu_mul(np.ascontiguousarray(gu[:, :I]), np.ascontiguousarray(gu[:, I:]))
+    got32 = gu_mod.linear_f16_packed(x, w, glu=True)
+    assert got32.shape == (M, I)
+    np.testing.assert_allclose(got32, want, rtol=0, atol=2e-5)
+    got16 = gu_mod.linear_f16_packed(x, w, out_dtype=np.float16, glu=True)
+    assert np.abs(got16.astype(np.float32) - want).max() <= 2e-3

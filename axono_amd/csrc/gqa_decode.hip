@@ -156,6 +156,17 @@ __device__ __forceinline__ void st_agent(float *p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Keys per split for a sequence of `len` keys: the sequence is cut into n_splits nearly equal
+// ranges (rounded up to 16 keys, at least kMinDevChunk), so that the workgroups of one sequence
+// finish together whatever its current length is; a range cut from the host-side upper bound would
+// leave the last split short (4100 keys in 4 splits: 1040/1040/1040/980 instead of 1152/1152/1152/644).
+constexpr int kMinDevChunk = 128;
+__device__ __forceinline__ int balanced_chunk(int len, int n_splits) {
+  int c = (len + n_splits - 1) / n_splits;
+  c = (c + 15) & ~15;
+  return c < kMinDevChunk ? kMinDevChunk : c;
+}
+
 __device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int max_len) {
   int len = seq_lens ? seq_lens[b] : max_len;
   len = len < 0 ? 0 : len;
@@ -219,7 +230,8 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   constexpr int RG = kThreads / LPR;
   const int split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
   const int len = clamped_len(a.seq_lens, b, a.max_len);
-  const int s0 = split * a.chunk;
+  const int chunk = balanced_chunk(len, a.n_splits);
+  const int s0 = split * chunk;
   const int tid = threadIdx.x;
   const int h0 = hg * G;            // first query head of this workgroup
   if (s0 >= len) {
@@ -231,7 +243,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
     }
     return;
   }
-  const int s1 = min(s0 + a.chunk, len);
+  const int s1 = min(s0 + chunk, len);
 
   const int rg = tid / LPR, dl = tid % LPR;
   const int hk = h0 / a.group;      // the kv head those G query heads share
@@ -299,7 +311,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   if (a.n_splits == 1 || !a.fused_merge) return;
 
   // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
-  const int n_valid = (len + a.chunk - 1) / a.chunk;  // splits that run for this sequence
+  const int n_valid = (len + chunk - 1) / chunk;  // splits that run for this sequence
   __shared__ int s_last;
   __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
   if (tid == 0) {
@@ -332,7 +344,8 @@ template <typename T, int D>
 __global__ __launch_bounds__(D) void gqa_decode_merge_kernel(DecodeArgs a) {
   const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const int len = clamped_len(a.seq_lens, b, a.max_len);
-  const int n_valid = (len + a.chunk - 1) / a.chunk;  // splits that wrote a partial
+  const int chunk = balanced_chunk(len, a.n_splits);
+  const int n_valid = (len + chunk - 1) / chunk;  // splits that wrote a partial
   const int64_t bh = static_cast<int64_t>(b) * a.Hq + h;
   T *out = static_cast<T *>(a.out) + bh * D + d;
   if (n_valid == 0) {

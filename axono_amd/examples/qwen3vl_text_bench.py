@@ -102,7 +102,12 @@ def main(argv=None):
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--gqa-single-launch", action="store_true",
+                    help="attention merges its splits in the last workgroup instead of a second kernel")
     args = ap.parse_args(argv)
+    if args.gqa_single_launch:
+        from .. import _lib
+        _lib.load().axhip_gqa_decode_tune(-1, 0)
     res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True))
     print(json.dumps(res), flush=True)
 

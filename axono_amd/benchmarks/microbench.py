@@ -169,8 +169,6 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False):
                 wb = pb
             ws_.append(wb)
         for M in Ms:
-            if packed and M > 32:
-                continue
             x = DeviceBuffer.from_numpy(rng.standard_normal((M, K)).astype(np.float32).astype(np.float16))
             out = DeviceBuffer(M * N * 4)
             wsb = lib.axhip_linear_f16_workspace_bytes(M, K, N)
@@ -233,7 +231,7 @@ def main(argv=None):
     elif args.what == "linear-packed":
         lib.axhip_linear_f16_tune(0, args.nt, args.waves)
         bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)],
-                     Ms=(args.M,) if args.M else (1, 16, 32), packed=True)
+                     Ms=(args.M,) if args.M else (1, 16, 32, 512, 4096), packed=True)
 
 
 if __name__ == "__main__":

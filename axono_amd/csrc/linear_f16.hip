@@ -539,6 +539,144 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// GEMM over packed weights (M > 32).  Workgroup tile: 256 rows of W (16 packed row tiles, 4 per
+// wavefront) x 128 rows of x; K advances 128 per step.  The W fragments come straight from the
+// packed buffer (1 KiB contiguous per load, no LDS); the x tile of a step (128 x 128 halves) is
+// staged once per workgroup into LDS (XOR-swizzled, double-buffered) with coalesced loads and read
+// back as MFMA "B" fragments by all four wavefronts.  Loads of step i+1 are issued before the 128
+// MFMAs of step i.  Workgroup ids are mapped so that the m-blocks sharing a block of W rows run on
+// the same XCD back to back: that XCD's L2 then serves W to all of them after one HBM read.
+// ------------------------------------------------------------------------------------------------
+constexpr int kGN = 256, kGM = 128, kGK = 128;  // workgroup tile
+constexpr int kXcds = 8;
+
+template <typename XT>
+__global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, int n_blocks, int m_blocks) {
+  __shared__ __attribute__((aligned(16))) _Float16 xs[2][kGM * kGK];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  // XCD-aware decode of the linear workgroup id (ids are dealt round-robin to the XCDs)
+  const int id = blockIdx.x;
+  const int xcd = id % kXcds, slot = id / kXcds;
+  const int nb = (slot / m_blocks) * kXcds + xcd, mb = slot % m_blocks;
+  if (nb >= n_blocks) return;
+  const int n_tiles = (a.N + 15) / 16;
+  const int tile0 = nb * (kGN / 16) + wave * 4;  // first of this wavefront's 4 row tiles
+  const int m0 = mb * kGM;
+  const XT *x = static_cast<const XT *>(a.x);
+  const int steps = (a.KC + 3) / 4;  // 4 chunks of 32 K per step
+
+  const __half *wt[4];
+  bool wok[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    wok[t] = tile0 + t < n_tiles;
+    wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + lane * 8;
+  }
+  auto load_w = [&](int t, int cc) -> half8_t {
+    return (wok[t] && cc < a.KC) ? load_h8(wt[t] + static_cast<int64_t>(cc) * 512) : zero_h8();
+  };
+  // x staging: 128 rows x 16 units of 16 bytes per step = 2048 vectors, 8 per thread
+  auto load_x = [&](int step, half8_t (&xv)[8]) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int v = p * 256 + tid;
+      const int row = v >> 4, unit = v & 15;
+      const int m = m0 + row, k = step * kGK + unit * 8;
+      xv[p] = (m < a.M && k + 8 <= a.K) ? load_h8(x + static_cast<int64_t>(m) * a.K + k) : zero_h8();
+    }
+  };
+  auto store_x = [&](int buf, const half8_t (&xv)[8]) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int v = p * 256 + tid;
+      const int row = v >> 4, unit = v & 15;
+      *reinterpret_cast<half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]) = xv[p];
+    }
+  };
+
+  float4_t acc[4][8];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  half8_t wf[4][4];  // [row tile][chunk within the step]
+  half8_t xv[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) wf[t][j] = load_w(t, j);
+  load_x(0, xv);
+  store_x(0, xv);
+  __syncthreads();
+
+  for (int i = 0; i < steps; ++i) {
+    const int buf = i & 1;
+    const bool more = i + 1 < steps;
+    if (more) load_x(i + 1, xv);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      half8_t bf[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int row = u * 16 + r, unit = j * 4 + g;
+        bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[t][j], bf[u], acc[t][u], 0, 0, 0);
+      // the fragments of chunk j are consumed: fetch chunk j of the next step into the same registers
+      if (more) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) wf[t][j] = load_w(t, (i + 1) * 4 + j);
+      }
+    }
+    if (more) store_x(buf ^ 1, xv);
+    __syncthreads();
+  }
+
+  LinearArgs o;
+  o.bias = a.bias;
+  o.out = a.out;
+  o.M = a.M;
+  o.N = a.glu ? a.N / 2 : a.N;
+  o.out_f16 = a.out_f16;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int m = m0 + u * 16 + r;
+    if (a.glu) {
+#pragma unroll
+      for (int t = 0; t < 4; t += 2) {
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float gt = acc[t][u][q];
+          v[q] = gt / (1.0f + expf(-gt)) * acc[t + 1][u][q];
+        }
+        store_out4(o, m, ((tile0 + t) / 2) * 16 + 4 * g, v);
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float v[4] = {acc[t][u][0], acc[t][u][1], acc[t][u][2], acc[t][u][3]};
+        store_out4(o, m, (tile0 + t) * 16 + 4 * g, v);
+      }
+    }
+  }
+}
+
+template <typename XT>
+void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
+  const int n_blocks = (a.N + kGN - 1) / kGN, m_blocks = (a.M + kGM - 1) / kGM;
+  const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;  // whole rounds over the XCDs
+  const dim3 grid(static_cast<unsigned>(nb_pad) * m_blocks);
+  hipLaunchKernelGGL((linear_gemm_packed_kernel<XT>), grid, dim3(256), 0, st, a, n_blocks, m_blocks);
+}
+
 }  // namespace
 }  // namespace axhip
 
@@ -630,12 +768,32 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
   if (!is_float_dtype(x_dtype) || !is_float_dtype(out_dtype)) return AXHIP_UNSUPPORTED_TYPE;
   if (M < 0 || K <= 0 || N <= 0 || K % 8 != 0) return AXHIP_INVALID_ARGUMENT;
   if (glu && (N % 32 != 0 || bias)) return AXHIP_INVALID_ARGUMENT;
-  if (M > kSkinnyMaxM) return AXHIP_INVALID_ARGUMENT;  // larger M takes the row-major weight and the tiled GEMM
-  if (N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
   if (M == 0) return AXHIP_OK;
   if (!x || !packed_w || !out) return AXHIP_INVALID_PTR;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed_w) | reinterpret_cast<uintptr_t>(out)) & 15)
     return AXHIP_INVALID_PTR;
+  if (M > kSkinnyMaxM) {  // MFMA-bound regime: tiled GEMM over the same packed buffer
+    PackedArgs ga;
+    ga.x = x;
+    ga.wp = static_cast<const __half *>(packed_w);
+    ga.bias = static_cast<const __half *>(bias);
+    ga.out = out;
+    ga.M = static_cast<int>(M);
+    ga.K = static_cast<int>(K);
+    ga.N = static_cast<int>(N);
+    ga.KC = static_cast<int>((K + 31) / 32);
+    ga.chunks_per_wave = 0;
+    ga.out_f16 = out_dtype == AXHIP_FLOAT16;
+    ga.glu = glu ? 1 : 0;
+    const int64_t wgs = ((N + kGN - 1) / kGN + kXcds - 1) / kXcds * kXcds * ((M + kGM - 1) / kGM);
+    if (wgs > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+    if (x_dtype == AXHIP_FLOAT16)
+      launch_gemm_packed<__half>(ga, as_stream(stream));
+    else
+      launch_gemm_packed<float>(ga, as_stream(stream));
+    return launch_status();
+  }
   SkinnyPlan p = plan_skinny(M, K, N);
   if (glu && p.nt % 2 != 0) {  // the gated epilogue needs gate and up tiles in the same wavefront
     p.nt = 2;

@@ -116,21 +116,13 @@ class Qwen3VLTextDecoder(nn.Module):
         return self._cache
 
     def _linear(self, x, name):
-        """x @ W^T: packed weights for decode-sized x, the row-major weight (tiled GEMM) otherwise."""
-        w = self._w(name)
-        rows = x.num_elements // w.shape[1]
-        if rows <= L.PACKED_MAX_ROWS:
-            return L.linear_packed(x, self._packed[name], w.shape[0])
-        return L.linear_nobias(x, w)
+        """x @ W^T over the packed copy of the weight (skinny kernels in decode, MFMA GEMM in prefill)."""
+        return L.linear_packed(x, self._packed[name], self._w(name).shape[0])
 
     def _mlp(self, xn, p):
         name = p + "mlp.gate_up_proj.weight"
-        w = self._w(name)
-        if xn.num_elements // w.shape[1] <= L.PACKED_MAX_ROWS:
-            # decode: the gate+up Linear applies SiLU-mul in its epilogue and stores fp16
-            act = L.linear_packed(xn, self._packed[name], w.shape[0], out_dtype=DataType.FLOAT16, glu=True)
-        else:
-            act = L.silu_mul_fused(L.linear_nobias(xn, w), DataType.FLOAT16)
+        # the gate+up Linear applies SiLU-mul in its epilogue and stores fp16
+        act = L.linear_packed(xn, self._packed[name], self._w(name).shape[0], out_dtype=DataType.FLOAT16, glu=True)
         return self._linear(act, p + "mlp.down_proj.weight")
 
     def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None, trace: list | None = None):

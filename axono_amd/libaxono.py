@@ -395,8 +395,9 @@ def pack_linear_weight(weight: Tensor, glu: bool = False) -> Tensor:
 
 def linear_packed(x: Tensor, packed: Tensor, n: int, bias: Tensor | None = None,
                   out_dtype: DataType | None = None, glu: bool = False) -> Tensor:
-    """x (..., K) with at most 32 rows . packed W [n, K]^T (+ bias).  glu: W was packed as a fused
-    [gate ; up] projection and the result is silu(gate) * up, (..., n/2)."""
+    """x (..., K) . packed W [n, K]^T (+ bias): the HBM-bound skinny kernels up to 32 rows, the
+    packed-weight MFMA GEMM above.  glu: W was packed as a fused [gate ; up] projection and the result
+    is silu(gate) * up, (..., n/2)."""
     op = "linear"
     has_b = bias is not None and bias.num_elements != 0
     _need_hip(op, x, packed, bias if has_b else None)

@@ -34,9 +34,8 @@ class Linear(Module):
         b = self._parameters["bias"]
         if w.dtype != DataType.FLOAT16:
             raise RuntimeError("linear: the hip operator takes FLOAT16 weights; call cast_linear_fp16() first")
-        rows = x.num_elements // self.in_features if self.in_features else 0
-        if w.is_hip and 0 < rows <= _l.PACKED_MAX_ROWS:
-            # decode-sized inputs read the packed copy of the weight (made once, on first use)
+        if w.is_hip and x.num_elements:
+            # the kernels read the packed copy of the weight (made once, on first use)
             packed = self.__dict__.get("_packed")
             if packed is None or self.__dict__.get("_packed_of") is not w:
                 packed = _l.pack_linear_weight(w)

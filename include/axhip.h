@@ -302,7 +302,7 @@ AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const 
  * into MFMA fragment order (1 KiB blocks of 16 rows x 32 K, consecutive along K; rows and K
  * zero-padded to whole blocks) into a buffer of axhip_linear_f16_packed_bytes(N,K) bytes, so that
  * every wavefront streams consecutive memory.  axhip_linear_f16_packed computes the same result as
- * axhip_linear_f16 from it, for M <= 32.  The packing is the build's counterpart of what
+ * axhip_linear_f16 from it: the HBM-bound skinny kernels for M <= 32, a 256x128-tile MFMA GEMM above.  The packing is the build's counterpart of what
  * Module.cast_linear_fp16 does to a Linear's weights (axono/python/axono/nn/module.py:158-184): a
  * one-off conversion into the resident format the inference kernels read.
  * glu != 0 (both calls): W is a fused [gate ; up] projection (N = 2*I rows, N % 32 == 0); the rows

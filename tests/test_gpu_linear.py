@@ -124,7 +124,7 @@ def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
         o16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16)
         assert np.abs(o16.astype(np.float32) - want).max() <= 2e-3
     l = gu.lib()
-    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 33, 64, 8, 0, None) == 1  # M > 32
+    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 33, 60, 8, 0, None) == 1  # K % 8
     assert l.axhip_linear_f16_packed_bytes(17, 40) == 2 * 2 * 1024
 
 
@@ -152,4 +152,34 @@ def test_packed_gate_up_with_silu_mul_epilogue(M, K, I):
     assert got32.shape == (M, I)
     np.testing.assert_allclose(got32, want, rtol=0, atol=2e-5)
     got16 = gu_mod.linear_f16_packed(x, w, out_dtype=np.float16, glu=True)
+    assert np.abs(got16.astype(np.float32) - want).max() <= 2e-3
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 2048, 2048), (512, 2048, 12288), (512, 6144, 2048), (33, 72, 50), (130, 264, 190),
+                                   (257, 136, 600), (4096, 256, 264)])
+def test_packed_gemm_large_M(M, K, N):
+    """M > 32 over packed weights (MFMA GEMM, 256 x 128 tiles, XCD-aware tile order)."""
+    rng = np.random.default_rng(M + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    b = h16(0.05 * rng.standard_normal(N))
+    out = gu.linear_f16_packed(x, w, b)
+    want = port.linear(x.astype(np.float32), w.astype(np.float32), b.astype(np.float32))
+    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
+    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag + 1e-3 * 2.0 ** -11)
+    x32 = rng.standard_normal((M, K)).astype(np.float32)  # fp32 activations are rounded to fp16 on the way in
+    out2 = gu.linear_f16_packed(x32, w)
+    want2 = port.linear(x32.astype(np.float16).astype(np.float32), w.astype(np.float32))
+    assert np.abs(out2 - want2).max() <= 1e-4
+
+
+def test_packed_gemm_glu_large_M():
+    rng = np.random.default_rng(77)
+    M, K, I = 300, 256, 160
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.05 * rng.standard_normal((2 * I, K)))
+    gu_ = port.linear(x.astype(np.float32), w.astype(np.float32))
+    want = port.silu_mul(np.ascontiguousarray(gu_[:, :I]), np.ascontiguousarray(gu_[:, I:]))
+    np.testing.assert_allclose(gu.linear_f16_packed(x, w, glu=True), want, rtol=0, atol=2e-5)
+    got16 = gu.linear_f16_packed(x, w, out_dtype=np.float16, glu=True)
     assert np.abs(got16.astype(np.float32) - want).max() <= 2e-3

@@ -147,13 +147,13 @@ def bench_rowops(lib, steps=200):
            "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 3)})
 
 
-def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False):
+def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, rot=0):
     rng = np.random.default_rng(0)
     shapes = shapes or [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 151936)]
     for K, N in shapes:
         w_host = (0.02 * rng.standard_normal((min(N, 4096), K))).astype(np.float32).astype(np.float16)
         # several weight copies are rotated when one is smaller than the Infinity Cache
-        n_rot = max(1, min(8, int(600e6 // (2 * K * N)) + 1))
+        n_rot = rot or max(1, min(8, int(600e6 // (2 * K * N)) + 1))
         ws_ = []
         for r in range(n_rot):
             wb = DeviceBuffer(N * K * 2)
@@ -205,6 +205,7 @@ def main(argv=None):
     ap.add_argument("--nt", type=int, default=0, help="linear: 16-row groups of W per wavefront (1, 2, 4)")
     ap.add_argument("--waves", type=int, default=0, help="linear: wavefronts (K slices) per workgroup (4, 8, 16)")
     ap.add_argument("--M", type=int, default=0, help="linear: only this row count")
+    ap.add_argument("--rot", type=int, default=0, help="linear: number of weight copies rotated through (1 = cache-hot)")
     args = ap.parse_args(argv)
     lib = _lib.load()
     if _lib.device_count() < 1:
@@ -227,11 +228,11 @@ def main(argv=None):
         bench_rowops(lib)
     elif args.what == "linear":
         lib.axhip_linear_f16_tune(0, args.nt, args.waves)
-        bench_linear(lib, Ms=(args.M,) if args.M else (1, 16, 32, 512))
+        bench_linear(lib, Ms=(args.M,) if args.M else (1, 16, 32, 512), rot=args.rot)
     elif args.what == "linear-packed":
         lib.axhip_linear_f16_tune(0, args.nt, args.waves)
         bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)],
-                     Ms=(args.M,) if args.M else (1, 16, 32, 512, 4096), packed=True)
+                     Ms=(args.M,) if args.M else (1, 16, 32, 512, 4096), packed=True, rot=args.rot)
 
 
 if __name__ == "__main__":

@@ -142,6 +142,18 @@ struct DecodeArgs {
   int64_t stride_b, stride_h, stride_s;
   float scale_log2e;
   int fused_merge;  // the last workgroup of a (sequence, head group) merges the splits
+  // Decode-step form (template parameter QKV): q, and the key / value row of the token being decoded,
+  // come straight from the fp32 output of the qkv projection; seq_lens holds the lengths before the
+  // append.  a.k / a.v are then the caches [B, Hkv, Lmax, D] and are written at row seq_lens[b].
+  int len_add;              // 1 in that form: the attended length is seq_lens[b] + 1
+  const float *pq, *pk, *pv;
+  int64_t pq_stride, pk_stride, pv_stride;
+  const void *qw, *kw;      // per-head RMSNorm weights [D] or null
+  int w_f16;
+  float eps;
+  const int64_t *pos;       // [3, B]
+  const float *inv_freq;    // [D/2]
+  int h_lim, w_lim, cache_rows;
 };
 
 // Split partials travel between workgroups that may sit on different XCDs, whose L2 caches are not
@@ -167,10 +179,54 @@ __device__ __forceinline__ int balanced_chunk(int len, int n_splits) {
   return c < kMinDevChunk ? kMinDevChunk : c;
 }
 
-__device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int max_len) {
+__device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int max_len, int len_add = 0) {
   int len = seq_lens ? seq_lens[b] : max_len;
   len = len < 0 ? 0 : len;
+  if (len_add && len < max_len) len += len_add;
   return len > max_len ? max_len : len;
+}
+
+// One head row of the qkv projection -> RMSNorm over the head (weights optional) -> interleaved
+// M-RoPE at this sequence's (t, h, w) position, in the evaluation order of the single operators
+// (rms_norm: (x * inv) * w; rope_thd: x0*c - x1*s, x1*c + x0*s).  One wavefront per row; the result
+// goes to `dst` (LDS) in the cache dtype and, when `gdst` is set, to the cache row as well.
+template <typename T, int D>
+__device__ __forceinline__ void norm_rope_row(const DecodeArgs &a, const float *src, const void *w, int b,
+                                              int B, int lane, T *dst, T *gdst) {
+  constexpr int HALF = D / 2;
+  float ss = 0.f;
+  for (int i = lane; i < HALF; i += 64) {
+    const float x0 = src[i], x1 = src[i + HALF];
+    ss = __builtin_fmaf(x0, x0, ss);
+    ss = __builtin_fmaf(x1, x1, ss);
+  }
+  ss = group_sum<64>(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(D) + a.eps);
+  const float pt = static_cast<float>(a.pos[b]);
+  const float ph = static_cast<float>(a.pos[B + b]);
+  const float pw = static_cast<float>(a.pos[2 * B + b]);
+  for (int i = lane; i < HALF; i += 64) {
+    float x0 = src[i] * inv, x1 = src[i + HALF] * inv;
+    if (w) {
+      x0 *= a.w_f16 ? __half2float(static_cast<const __half *>(w)[i]) : static_cast<const float *>(w)[i];
+      x1 *= a.w_f16 ? __half2float(static_cast<const __half *>(w)[i + HALF]) : static_cast<const float *>(w)[i + HALF];
+    }
+    const float f = a.inv_freq[i];
+    float ang = pt * f;
+    if (i % 3 == 1 && i < a.h_lim)
+      ang = ph * f;
+    else if (i % 3 == 2 && i < a.w_lim)
+      ang = pw * f;
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    const float y0 = x0 * cs - x1 * sn, y1 = x1 * cs + x0 * sn;
+    stf(dst + i, y0);
+    stf(dst + i + HALF, y1);
+    if (gdst) {
+      stf(gdst + i, y0);
+      stf(gdst + i + HALF, y1);
+    }
+  }
 }
 
 // One tile: U load instructions per lane for K and for V (U*RG key rows per workgroup).
@@ -224,12 +280,12 @@ __device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t st
   }
 }
 
-template <typename T, int D, int G, int U>
+template <typename T, int D, int G, int U, bool QKV>
 __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArgs a) {
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
   const int split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
-  const int len = clamped_len(a.seq_lens, b, a.max_len);
+  const int len = clamped_len(a.seq_lens, b, a.max_len, QKV ? a.len_add : 0);
   const int chunk = balanced_chunk(len, a.n_splits);
   const int s0 = split * chunk;
   const int tid = threadIdx.x;
@@ -248,14 +304,54 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   const int rg = tid / LPR, dl = tid % LPR;
   const int hk = h0 / a.group;      // the kv head those G query heads share
 
-  const T *q = static_cast<const T *>(a.q);
-  Frag8<T> qf[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) qf[g].load(q + (static_cast<int64_t>(b) * a.Hq + h0 + g) * D + dl * 8);
-
   const int64_t kv_off = b * a.stride_b + hk * a.stride_h + dl * 8;
   const T *kb = static_cast<const T *>(a.k) + kv_off;
   const T *vb = static_cast<const T *>(a.v) + kv_off;
+
+  Frag8<T> qf[G];
+  // Decode-step form: the token being decoded sits at row p_new; the workgroup whose key range holds
+  // that row prepares its key and value itself (from the projection output, rounded to the cache
+  // dtype exactly as the cache stores them) and attends to them from LDS, because the cache row is
+  // written in this same launch - by the first of the workgroups that share the kv head.
+  __shared__ __attribute__((aligned(16))) T s_q[QKV ? G : 1][D];
+  __shared__ __attribute__((aligned(16))) T s_kv[2][QKV ? D : 8];
+  bool mine = false;
+  int kv_end = s1;  // keys [s0, kv_end) come from the cache
+  if constexpr (QKV) {
+    int p_new = a.seq_lens[b];
+    p_new = p_new < 0 ? 0 : p_new;
+    mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
+    if (mine) kv_end = p_new;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int B = gridDim.z;
+    const bool writer = mine && (h0 % a.group == 0);
+    for (int job = wave; job < G + (mine ? 2 : 0); job += kThreads / 64) {
+      if (job < G) {
+        norm_rope_row<T, D>(a, a.pq + b * a.pq_stride + static_cast<int64_t>(h0 + job) * D, a.qw, b, B, lane, s_q[job],
+                            static_cast<T *>(nullptr));
+      } else {
+        T *crow = const_cast<T *>(static_cast<const T *>(job == G ? a.k : a.v)) + b * a.stride_b + hk * a.stride_h +
+                  static_cast<int64_t>(p_new) * a.stride_s;
+        if (job == G) {
+          norm_rope_row<T, D>(a, a.pk + b * a.pk_stride + static_cast<int64_t>(hk) * D, a.kw, b, B, lane, s_kv[0],
+                              writer ? crow : static_cast<T *>(nullptr));
+        } else {
+          const float *src = a.pv + b * a.pv_stride + static_cast<int64_t>(hk) * D;
+          for (int i = lane; i < D; i += 64) {
+            stf(&s_kv[1][i], src[i]);
+            if (writer) stf(crow + i, src[i]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; ++g) qf[g].load(&s_q[g][dl * 8]);
+  } else {
+    const T *q = static_cast<const T *>(a.q);
+#pragma unroll
+    for (int g = 0; g < G; ++g) qf[g].load(q + (static_cast<int64_t>(b) * a.Hq + h0 + g) * D + dl * 8);
+  }
 
   float m[G], l[G], acc[G][8];
 #pragma unroll
@@ -267,10 +363,31 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   }
 
   int base = s0;
-  for (; base + U * RG <= s1; base += U * RG)
-    decode_tile<T, D, G, U, false>(kb, vb, a.stride_s, base, rg, s1, a.scale_log2e, qf, m, l, acc);
-  for (; base < s1; base += U * RG)
-    decode_tile<T, D, G, U, true>(kb, vb, a.stride_s, base, rg, s1, a.scale_log2e, qf, m, l, acc);
+  for (; base + U * RG <= kv_end; base += U * RG)
+    decode_tile<T, D, G, U, false>(kb, vb, a.stride_s, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
+  for (; base < kv_end; base += U * RG)
+    decode_tile<T, D, G, U, true>(kb, vb, a.stride_s, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
+  if constexpr (QKV) {
+    if (mine) {  // the new token's key and value: one more row, taken by row group 0
+      Frag8<T> kn, vn;
+      kn.load(&s_kv[0][dl * 8]);
+      vn.load(&s_kv[1][dl * 8]);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const float d = group_sum<LPR>(qf[g].dot(kn)) * a.scale_log2e;
+        if (rg == 0) {
+          const float mn = fmaxf(m[g], d);
+          const float corr = __builtin_amdgcn_exp2f(m[g] - mn);
+          const float p = __builtin_amdgcn_exp2f(d - mn);
+          m[g] = mn;
+          l[g] = l[g] * corr + p;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[g][i] *= corr;
+          vn.axpy(p, acc[g]);
+        }
+      }
+    }
+  }
 
   // ---- merge the RG row-group states of this workgroup ----------------------------------------
   __shared__ float s_m[G][RG];
@@ -343,7 +460,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
 template <typename T, int D>
 __global__ __launch_bounds__(D) void gqa_decode_merge_kernel(DecodeArgs a) {
   const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-  const int len = clamped_len(a.seq_lens, b, a.max_len);
+  const int len = clamped_len(a.seq_lens, b, a.max_len, a.len_add);
   const int chunk = balanced_chunk(len, a.n_splits);
   const int n_valid = (len + chunk - 1) / chunk;  // splits that wrote a partial
   const int64_t bh = static_cast<int64_t>(b) * a.Hq + h;
@@ -369,7 +486,10 @@ template <typename T, int D, int G>
 int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   constexpr int U = (sizeof(T) == 2 ? 8 : 4) / (G >= 4 ? 2 : 1);
   const dim3 grid(a.n_splits, a.Hq / G, B);
-  hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U>), grid, dim3(kThreads), 0, st, a);
+  if (a.len_add)
+    hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, true>), grid, dim3(kThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, false>), grid, dim3(kThreads), 0, st, a);
   if (a.n_splits > 1 && !a.fused_merge)
     hipLaunchKernelGGL((gqa_decode_merge_kernel<T, D>), dim3(a.Hq, B), dim3(D), 0, st, a);
   return launch_status();
@@ -401,6 +521,34 @@ int heads_per_workgroup(int group) { return group % 4 == 0 ? 4 : (group % 2 == 0
 }  // namespace axhip
 
 using namespace axhip;
+
+namespace {
+// Split plan, workspace carve-up and launch shared by the entry points.
+int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int dtype, int B, int Hq, int Hkv,
+                    int D, int max_len, axhip_stream stream) {
+  const int group = Hq / Hkv;
+  const int G = heads_per_workgroup(group);
+  const SplitPlan plan = plan_splits(B, Hq / G, max_len);
+  a.Hq = Hq;
+  a.group = group;
+  a.max_len = max_len;
+  a.chunk = plan.chunk;
+  a.n_splits = plan.n_splits;
+  a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
+  a.part_acc = nullptr;
+  a.part_ml = nullptr;
+  a.fused_merge = (!g_tuning.separate_merge && static_cast<long>(B) * (Hq / G) <= kTicketSlots) ? 1 : 0;
+  if (plan.n_splits > 1) {
+    const size_t acc_elems = static_cast<size_t>(B) * Hq * plan.n_splits * D;
+    const size_t need = (acc_elems + static_cast<size_t>(B) * Hq * plan.n_splits * 2) * sizeof(float);
+    if (!workspace || workspace_bytes < need) return AXHIP_INVALID_ARGUMENT;
+    a.part_acc = static_cast<float *>(workspace);
+    a.part_ml = a.part_acc + acc_elems;
+  }
+  hipStream_t st = as_stream(stream);
+  return dtype == AXHIP_FLOAT16 ? dispatch_dim<__half>(a, D, G, B, st) : dispatch_dim<float>(a, D, G, B, st);
+}
+}  // namespace
 
 extern "C" {
 
@@ -444,38 +592,60 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v, cons
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) & 15)
     return AXHIP_INVALID_PTR;
 
-  const int group = Hq / Hkv;
-  const int G = heads_per_workgroup(group);
-  const SplitPlan plan = plan_splits(B, Hq / G, max_len);
-
-  DecodeArgs a;
+  DecodeArgs a{};
   a.q = q;
   a.k = k;
   a.v = v;
   a.seq_lens = seq_lens;
   a.out = out;
-  a.Hq = Hq;
-  a.group = group;
-  a.max_len = max_len;
-  a.chunk = plan.chunk;
-  a.n_splits = plan.n_splits;
   a.stride_b = stride_b;
   a.stride_h = stride_h;
   a.stride_s = stride_s;
-  a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
-  a.part_acc = nullptr;
-  a.part_ml = nullptr;
-  a.fused_merge = (!g_tuning.separate_merge && static_cast<long>(B) * (Hq / G) <= kTicketSlots) ? 1 : 0;
-  if (plan.n_splits > 1) {
-    const size_t acc_elems = static_cast<size_t>(B) * Hq * plan.n_splits * D;
-    const size_t need = (acc_elems + static_cast<size_t>(B) * Hq * plan.n_splits * 2) * sizeof(float);
-    if (!workspace || workspace_bytes < need) return AXHIP_INVALID_ARGUMENT;
-    a.part_acc = static_cast<float *>(workspace);
-    a.part_ml = a.part_acc + acc_elems;
-  }
-  hipStream_t st = as_stream(stream);
-  return dtype == AXHIP_FLOAT16 ? dispatch_dim<__half>(a, D, G, B, st)
-                                : dispatch_dim<float>(a, D, G, B, st);
+  return plan_and_launch(a, workspace, workspace_bytes, dtype, B, Hq, Hkv, D, max_len, stream);
+}
+
+AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float *k, int64_t k_stride,
+                                   const float *v, int64_t v_stride, const void *q_weight,
+                                   const void *k_weight, int w_dtype, float eps, const int64_t *pos,
+                                   const float *inv_freq, int h_sec, int w_sec, const int32_t *seq_lens,
+                                   void *k_cache, void *v_cache, void *out, void *workspace,
+                                   size_t workspace_bytes, int cache_dtype, int B, int Hq, int Hkv, int D,
+                                   int cache_rows, int max_len, axhip_stream stream) {
+  if (cache_dtype != AXHIP_FLOAT16 && cache_dtype != AXHIP_FLOAT32) return AXHIP_UNSUPPORTED_TYPE;
+  if ((q_weight || k_weight) && !is_float_dtype(w_dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || Hq <= 0 || Hkv <= 0 || max_len <= 0 || cache_rows <= 0 || max_len > cache_rows)
+    return AXHIP_INVALID_ARGUMENT;
+  if (Hq % Hkv != 0) return AXHIP_SHAPE_MISMATCH;
+  if (D != 64 && D != 128 && D != 256) return AXHIP_INVALID_ARGUMENT;
+  if (B == 0) return AXHIP_OK;
+  if (B > 65535) return AXHIP_INVALID_ARGUMENT;
+  if (!q || !k || !v || !pos || !inv_freq || !seq_lens || !k_cache || !v_cache || !out) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15) return AXHIP_INVALID_PTR;
+  DecodeArgs a{};
+  a.k = k_cache;
+  a.v = v_cache;
+  a.seq_lens = seq_lens;
+  a.out = out;
+  a.stride_b = static_cast<int64_t>(Hkv) * cache_rows * D;
+  a.stride_h = static_cast<int64_t>(cache_rows) * D;
+  a.stride_s = D;
+  a.len_add = 1;
+  a.pq = q;
+  a.pk = k;
+  a.pv = v;
+  a.pq_stride = q_stride;
+  a.pk_stride = k_stride;
+  a.pv_stride = v_stride;
+  a.qw = q_weight;
+  a.kw = k_weight;
+  a.w_f16 = w_dtype == AXHIP_FLOAT16;
+  a.eps = eps;
+  a.pos = pos;
+  a.inv_freq = inv_freq;
+  a.h_lim = h_sec * 3;
+  a.w_lim = w_sec * 3;
+  a.cache_rows = cache_rows;
+  return plan_and_launch(a, workspace, workspace_bytes, cache_dtype, B, Hq, Hkv, D, max_len, stream);
 }
 
 }  // extern "C"

@@ -137,18 +137,17 @@ class Qwen3VLTextDecoder(nn.Module):
         max_len = attn_max_len or cache.max_len
         h = L.embedding(ids, self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)  # [B,H]
         xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
-        # lengths that include the token being appended (the kernel reads them on the device)
-        lens_now = self._lens_plus_one
         for i in range(cfg.num_hidden_layers):
             p = f"layers.{i}."
             if trace is not None:
                 trace.append(h)
             qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")
             kc, vc = cache.get(i)
-            q = L.qkv_norm_rope_append(qkv, self._w(p + "self_attn.q_norm.weight"), self._w(p + "self_attn.k_norm.weight"),
-                                       cfg.rms_norm_eps, pos, self._inv_freq, cfg.mrope_section, cache.seq_lens, kc, vc,
-                                       cfg.num_attention_heads)
-            attn = L.gqa_decode_attention_cache(q, kc, vc, lens_now, max_len, workspace=self._attn_ws)
+            # q/k RMSNorm + M-RoPE + KV append + attention over seq_lens + 1 keys: one launch (+ the merge)
+            attn = L.gqa_decode_attention_qkv(qkv, self._w(p + "self_attn.q_norm.weight"),
+                                              self._w(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, pos,
+                                              self._inv_freq, cfg.mrope_section, cache.seq_lens, kc, vc,
+                                              cfg.num_attention_heads, max_len, workspace=self._attn_ws)
             attn_out = self._linear(attn.reshape([B, cfg.num_attention_heads * cfg.head_dim]),
                                     p + "self_attn.o_proj.weight")
             h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
@@ -224,12 +223,8 @@ class Qwen3VLTextDecoder(nn.Module):
         self._ids.copy_from_numpy(np.ascontiguousarray(first_ids, dtype=np.int64).reshape(B))
         self._pos.copy_from_numpy(np.ascontiguousarray(first_pos, dtype=np.int64).reshape(3, B))
         bound = min(self._cache.max_len, len(self._cache) + max_new_tokens + 1)
-        self._lens_plus_one = Tensor(DataType.INT32, [B], self._device)
 
         def step():
-            # lens_plus_one = seq_lens + 1 (keys visible to this step's query, incl. the new token)
-            check(self._lib.axhip_memcpy_d2d(self._lens_plus_one.data_ptr, self._cache.seq_lens.data_ptr, 4 * B), "copy")
-            L.index_add(self._lens_plus_one, 1)
             logits, nxt = self.decode_forward(self._ids, self._pos, bound)
             # feed the device-side state of the next step
             check(self._lib.axhip_memcpy_d2d(self._ids.data_ptr, nxt.data_ptr, 8 * B), "copy")

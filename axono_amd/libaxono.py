@@ -518,6 +518,49 @@ def qkv_norm_rope_append(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, eps: f
     return q_out
 
 
+def gqa_decode_attention_qkv(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, eps: float, pos: Tensor, inv_freq: Tensor,
+                             mrope_section, seq_lens: Tensor, k_cache: Tensor, v_cache: Tensor, n_q_heads: int,
+                             max_len: int | None = None, workspace: Tensor | None = None) -> Tensor:
+    """The attention block of one decode step in one launch: qkv FLOAT32 [B, (Hq + 2*Hkv) * D] (fused
+    projection) is normalised per head, rotated, its k / v rows appended to the caches at seq_lens[b],
+    and the query attends over seq_lens[b] + 1 keys.  Equals qkv_norm_rope_append followed by
+    gqa_decode_attention_cache.  Returns [B, Hq, D] in the cache dtype."""
+    op = "gqa_decode_attention"
+    _need_hip(op, qkv, q_weight, k_weight, pos, inv_freq, seq_lens, k_cache, v_cache, workspace)
+    if qkv.dtype != DataType.FLOAT32 or k_cache.ndim != 4 or k_cache.dtype not in _FLOATS or v_cache.dtype != k_cache.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    B, hkv, rows, d = k_cache.shape
+    hq = int(n_q_heads)
+    width = (hq + 2 * hkv) * d
+    if qkv.num_elements != B * width or v_cache.shape != k_cache.shape:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if pos.dtype != DataType.INT64 or pos.shape != [3, B] or seq_lens.dtype != DataType.INT32 or seq_lens.num_elements != B:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if inv_freq.dtype != DataType.FLOAT32 or inv_freq.num_elements != d // 2:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    for w in (q_weight, k_weight):
+        if w is not None and (w.num_elements != d or w.dtype not in _FLOATS):
+            raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    _, h_sec, w_sec = (list(mrope_section) + [0, 0, 0])[:3]
+    bound = int(max_len) if max_len else rows
+    lib = _lib_()
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, hq, hkv, d, bound)
+    if workspace is None:
+        workspace = _new(DataType.INT8, [max(wsb, 256)], qkv)
+    out = _new(k_cache.dtype, [B, hq, d], qkv)
+    base = qkv.data_ptr
+    wdt = int(q_weight.dtype) if q_weight is not None else int(DataType.FLOAT32)
+    check(lib.axhip_gqa_decode_qkv(
+        base, width, base + hq * d * 4, width, base + (hq + hkv) * d * 4, width,
+        q_weight.data_ptr if q_weight is not None else None, k_weight.data_ptr if k_weight is not None else None,
+        wdt, float(eps), pos.data_ptr, inv_freq.data_ptr, int(h_sec), int(w_sec), seq_lens.data_ptr,
+        k_cache.data_ptr, v_cache.data_ptr, out.data_ptr, workspace.data_ptr, workspace.num_bytes, int(k_cache.dtype),
+        B, hq, hkv, d, rows, bound, current_stream()), op)
+    return out
+
+
 # ---- graph capture -------------------------------------------------------------------------------
 class HIPGraph:
     """The binding-level graph object (the reference's CUDAGraph class, nanobind_module.cpp:1228-1324):

@@ -166,7 +166,6 @@ def cpu_decode_step_hook(cfg, weights, model, first, pos, batch, max_len, log):
     # device: one eager step with the residual stream of every layer kept, then rewind
     state = (model._ids.numpy().copy(), model._pos.numpy().copy(), model.cache.seq_lens.numpy().copy())
     trace = []
-    model._lens_plus_one.copy_from_numpy((state[2] + 1).astype(np.int32))
     g_logits, g_next = model.decode_forward(model._ids, model._pos, trace=trace)
     g_logits, g_next = g_logits.to_numpy().copy(), g_next.to_numpy().copy()
     h_gpu = [t.to_numpy().copy() for t in trace]

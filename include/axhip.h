@@ -353,6 +353,24 @@ AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const
                                          void *k_cache, void *v_cache, int cache_dtype, int B, int S,
                                          int Hq, int Hkv, int D, int Lmax, axhip_stream stream);
 
+/* The attention block of one decode step in one launch (plus the split merge): equals
+ * axhip_qkv_norm_rope_append with S = 1 followed by axhip_gqa_decode over seq_lens[b] + 1 keys of the
+ * caches [B,Hkv,cache_rows,D], without materialising q and without a second read of the row just
+ * appended.  q / k / v, their strides, the norm weights, pos [3,B], inv_freq, h_sec / w_sec as in
+ * axhip_qkv_norm_rope_append; seq_lens int32 [B] holds the lengths BEFORE the append (required); the new
+ * row is written at seq_lens[b] when that is < max_len, otherwise nothing is appended and max_len cached
+ * keys are attended.  max_len <= cache_rows bounds the attended length (the split plan is made from it, so a
+ * captured launch stays valid while seq_lens grows).  out [B,Hq,D] in the cache dtype.  Workspace as for
+ * axhip_gqa_decode.  No reference counterpart (the reference's layer runs these as separate operators,
+ * examples/vlm/qwen3vl/model.py:330-373). */
+AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float *k, int64_t k_stride,
+                                   const float *v, int64_t v_stride, const void *q_weight,
+                                   const void *k_weight, int w_dtype, float eps, const int64_t *pos,
+                                   const float *inv_freq, int h_sec, int w_sec, const int32_t *seq_lens,
+                                   void *k_cache, void *v_cache, void *out, void *workspace,
+                                   size_t workspace_bytes, int cache_dtype, int B, int Hq, int Hkv, int D,
+                                   int cache_rows, int max_len, axhip_stream stream);
+
 /* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
  * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0.  out_dtype
  * may be FLOAT16 for FLOAT32 input (see axhip_add_rms_norm_ex). */

@@ -11,6 +11,7 @@ import pytest
 import oracle
 from oracle import port
 
+import gpu_util as gu
 from gpu_util import gqa_decode, lib
 
 pytestmark = pytest.mark.gpu
@@ -167,3 +168,67 @@ def test_two_kernel_merge_mode_matches_fused_merge():
     one = gqa_decode(q, k, v, lens).astype(np.float32)
     lib().axhip_gqa_decode_tune(0, 0)
     assert np.abs(one - want).max() <= TOL16 and np.all(one[1] == 0)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (8, 1, 64), (3, 3, 256)])
+def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
+    """axhip_gqa_decode_qkv (q/k norm + M-RoPE + append + attention in the split kernel) against the
+    oracle's rms_norm -> rope_thd -> fp16 rounding -> append -> attention over len + 1 keys; sequences
+    that put the new row in the first split, in the last split, and alone in a split of its own."""
+    rng = np.random.default_rng(77)
+    rows, max_len = 1300, 1280
+    lens = np.array([0, 5, 255, 256, 700, 1279, 1280], np.int32)   # 1280: cache bound reached, nothing appended
+    B = len(lens)
+    width = (Hq + 2 * Hkv) * D
+    qkv = rng.standard_normal((B, width)).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    pos = rng.integers(0, 8192, (3, B)).astype(np.int64)
+    inv = port.rope_inv_freq(1e6, D)
+    hw = 10 if D == 64 else 20
+    sec = [D // 2 - 2 * hw, hw, hw]
+    kc = (0.5 * rng.standard_normal((B, Hkv, rows, D))).astype(np.float16)
+    vc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
+    l = gu.lib()
+    dq, dqw, dkw, dp, di, dl, dkc, dvc = (gu.dev(a) for a in (qkv, qw, kw, pos, inv, lens, kc, vc))
+    out = gu.DeviceBuffer(B * Hq * D * 2)
+    for force_splits in (0, 5):
+        l.axhip_gqa_decode_tune(0, force_splits)
+        dkc.upload(kc.reshape(-1))
+        dvc.upload(vc.reshape(-1))
+        wsb = l.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, max_len)
+        ws = gu.DeviceBuffer(max(wsb, 256))
+        gu._run("axhip_gqa_decode_qkv", dq.ptr, width, dq.ptr + Hq * D * 4, width, dq.ptr + (Hq + Hkv) * D * 4, width,
+                dqw.ptr, dkw.ptr, gu.F32, 1e-6, dp.ptr, di.ptr, hw, hw, dl.ptr, dkc.ptr, dvc.ptr, out.ptr, ws.ptr, wsb,
+                gu.F16, B, Hq, Hkv, D, rows, max_len, None)
+        gu.synchronize()
+        q = port.rope_thd(port.rms_norm(qkv[:, : Hq * D].reshape(B, Hq, D), qw, 1e-6), pos, inv, sec)
+        k = port.rope_thd(port.rms_norm(qkv[:, Hq * D:(Hq + Hkv) * D].reshape(B, Hkv, D), kw, 1e-6), pos, inv, sec)
+        v = qkv[:, (Hq + Hkv) * D:].reshape(B, Hkv, D)
+        wk, wv = kc.copy(), vc.copy()
+        attended = lens.copy()
+        for b in range(B):
+            if lens[b] < max_len:
+                wk[b, :, lens[b]] = k[b].astype(np.float16)
+                wv[b, :, lens[b]] = v[b].astype(np.float16)
+                attended[b] += 1
+        gk, gv = dkc.download(np.float16, kc.shape), dvc.download(np.float16, vc.shape)
+        np.testing.assert_array_equal(gv.view(np.uint16), wv.view(np.uint16))
+        assert np.abs(gk.astype(np.float32) - wk.astype(np.float32)).max() <= 2e-3
+        untouched = np.ones(kc.shape, bool)
+        for b in range(B):
+            if lens[b] < max_len:
+                untouched[b, :, lens[b]] = False
+        np.testing.assert_array_equal(gk[untouched].view(np.uint16), kc[untouched].view(np.uint16))
+        # attention of the oracle over the cache as the device wrote it, with q rounded to the cache dtype
+        want = port.gqa_decode_cache_native(q.astype(np.float16).astype(np.float32), gk.astype(np.float32),
+                                              gv.astype(np.float32), attended)
+        got = out.download(np.float16, (B, Hq, D)).astype(np.float32)
+        assert np.abs(got - want).max() <= 2e-3, (force_splits, np.abs(got - want).max())
+    l.axhip_gqa_decode_tune(0, 0)
+    # argument checks: seq_lens is required; max_len may not exceed the cache
+    args = [dq.ptr, width, dq.ptr, width, dq.ptr, width, None, None, gu.F32, 1e-6, dp.ptr, di.ptr, hw, hw]
+    assert l.axhip_gqa_decode_qkv(*args, None, dkc.ptr, dvc.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows,
+                                  max_len, None) == 7
+    assert l.axhip_gqa_decode_qkv(*args, dl.ptr, dkc.ptr, dvc.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows,
+                                  rows + 1, None) == 1

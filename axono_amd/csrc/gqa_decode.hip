@@ -230,14 +230,10 @@ __device__ __forceinline__ void norm_rope_row(const DecodeArgs &a, const float *
 }
 
 // One tile: U load instructions per lane for K and for V (U*RG key rows per workgroup).
-template <typename T, int D, int G, int U, bool CHECK>
-__device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t stride_s, int base,
-                                            int rg, int s1, float scale_log2e,
-                                            const Frag8<T> (&qf)[G], float (&m)[G], float (&l)[G],
-                                            float (&acc)[G][8]) {
-  constexpr int LPR = D / 8;
-  constexpr int RG = kThreads / LPR;
-  Frag8<T> kr[U], vr[U];
+template <typename T, int D, int U, bool CHECK>
+__device__ __forceinline__ void tile_load(const T *kb, const T *vb, int64_t stride_s, int base, int rg, int s1,
+                                          Frag8<T> (&kr)[U], Frag8<T> (&vr)[U]) {
+  constexpr int RG = kThreads / (D / 8);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int row = base + u * RG + rg;
@@ -249,6 +245,14 @@ __device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t st
       vr[u].zero();
     }
   }
+}
+
+template <typename T, int D, int G, int U, bool CHECK>
+__device__ __forceinline__ void tile_update(const Frag8<T> (&kr)[U], const Frag8<T> (&vr)[U], int base, int rg,
+                                            int s1, float scale_log2e, const Frag8<T> (&qf)[G], float (&m)[G],
+                                            float (&l)[G], float (&acc)[G][8]) {
+  constexpr int LPR = D / 8;
+  constexpr int RG = kThreads / LPR;
   float sc[G][U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -278,6 +282,16 @@ __device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t st
       vr[u].axpy(p, acc[g]);
     }
   }
+}
+
+template <typename T, int D, int G, int U, bool CHECK>
+__device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t stride_s, int base,
+                                            int rg, int s1, float scale_log2e,
+                                            const Frag8<T> (&qf)[G], float (&m)[G], float (&l)[G],
+                                            float (&acc)[G][8]) {
+  Frag8<T> kr[U], vr[U];
+  tile_load<T, D, U, CHECK>(kb, vb, stride_s, base, rg, s1, kr, vr);
+  tile_update<T, D, G, U, CHECK>(kr, vr, base, rg, s1, scale_log2e, qf, m, l, acc);
 }
 
 template <typename T, int D, int G, int U, bool QKV>
@@ -317,11 +331,14 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   __shared__ __attribute__((aligned(16))) T s_kv[2][QKV ? D : 8];
   bool mine = false;
   int kv_end = s1;  // keys [s0, kv_end) come from the cache
+  Frag8<T> kr0[QKV ? U : 1], vr0[QKV ? U : 1];
   if constexpr (QKV) {
     int p_new = a.seq_lens[b];
     p_new = p_new < 0 ? 0 : p_new;
     mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
     if (mine) kv_end = p_new;
+    // the first tile of cached keys is requested before q is prepared: those loads do not need it
+    tile_load<T, D, U, true>(kb, vb, a.stride_s, s0, rg, kv_end, kr0, vr0);
     const int wave = tid >> 6, lane = tid & 63;
     const int B = gridDim.z;
     const bool writer = mine && (h0 % a.group == 0);
@@ -363,6 +380,10 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   }
 
   int base = s0;
+  if constexpr (QKV) {
+    tile_update<T, D, G, U, true>(kr0, vr0, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
+    base += U * RG;
+  }
   for (; base + U * RG <= kv_end; base += U * RG)
     decode_tile<T, D, G, U, false>(kb, vb, a.stride_s, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
   for (; base < kv_end; base += U * RG)

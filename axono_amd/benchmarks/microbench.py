@@ -205,6 +205,7 @@ def main(argv=None):
     ap.add_argument("--nt", type=int, default=0, help="linear: 16-row groups of W per wavefront (1, 2, 4)")
     ap.add_argument("--waves", type=int, default=0, help="linear: wavefronts (K slices) per workgroup (4, 8, 16)")
     ap.add_argument("--M", type=int, default=0, help="linear: only this row count")
+    ap.add_argument("--gemm-rows", type=int, default=0, help="linear: rows of x per GEMM workgroup (64 or 128)")
     ap.add_argument("--rot", type=int, default=0, help="linear: number of weight copies rotated through (1 = cache-hot)")
     args = ap.parse_args(argv)
     lib = _lib.load()
@@ -227,10 +228,10 @@ def main(argv=None):
     elif args.what == "rowops":
         bench_rowops(lib)
     elif args.what == "linear":
-        lib.axhip_linear_f16_tune(0, args.nt, args.waves)
+        lib.axhip_linear_f16_tune(0, args.nt, args.waves, args.gemm_rows)
         bench_linear(lib, Ms=(args.M,) if args.M else (1, 16, 32, 512), rot=args.rot)
     elif args.what == "linear-packed":
-        lib.axhip_linear_f16_tune(0, args.nt, args.waves)
+        lib.axhip_linear_f16_tune(0, args.nt, args.waves, args.gemm_rows)
         bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)],
                      Ms=(args.M,) if args.M else (1, 16, 32, 512, 4096), packed=True, rot=args.rot)
 

@@ -73,7 +73,9 @@ __device__ __forceinline__ half8_t zero_h8() {
 }
 
 __device__ __forceinline__ half8_t load_h8(const __half *p) {
-  return __builtin_bit_cast(half8_t, ld16(p));
+  // a plain vector load: going through an integer struct makes the compiler touch the loaded
+  // registers at once, which puts a wait right behind every load
+  return *reinterpret_cast<const half8_t *>(p);
 }
 
 // 8 fp32 activations -> fp16 round-to-nearest-even (the conversion the reference applies to x
@@ -548,12 +550,21 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
 // MFMAs of step i.  Workgroup ids are mapped so that the m-blocks sharing a block of W rows run on
 // the same XCD back to back: that XCD's L2 then serves W to all of them after one HBM read.
 // ------------------------------------------------------------------------------------------------
-constexpr int kGN = 256, kGM = 128, kGK = 128;  // workgroup tile
+constexpr int kGN = 256, kGK = 128;  // workgroup tile: kGN weight rows x GM rows of x, K in steps of kGK
+int g_gemm_rows = 0;                 // measurement hook: 64 or 128 rows of x per workgroup (0 = default)
 constexpr int kXcds = 8;
 
-template <typename XT>
-__global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, int n_blocks, int m_blocks) {
-  __shared__ __attribute__((aligned(16))) _Float16 xs[2][kGM * kGK];
+// FULL: K is a multiple of the 128-column step, so no load needs a predicate (rows and tiles past
+// the edge are clamped to valid memory and their results never stored).  Predicated loads compile to
+// branches, after which the compiler waits for every outstanding load before each MFMA group.
+// GM: rows of x per workgroup.  128 gives the larger tile (one workgroup per CU, 87 flop per byte
+// moved from L2); 64 halves the registers so that two workgroups share a CU and one's loads hide
+// behind the other's MFMAs.
+template <typename XT, bool FULL, int GM>
+__global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kernel(PackedArgs a, int n_blocks, int m_blocks) {
+  constexpr int MT = GM / 16;        // x row tiles per wavefront
+  constexpr int XV = GM * 16 / 256;  // 16-byte x vectors staged per thread and step
+  __shared__ __attribute__((aligned(16))) _Float16 xs[2][GM * kGK];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
   // XCD-aware decode of the linear workgroup id (ids are dealt round-robin to the XCDs)
@@ -563,7 +574,7 @@ __global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, i
   if (nb >= n_blocks) return;
   const int n_tiles = (a.N + 15) / 16;
   const int tile0 = nb * (kGN / 16) + wave * 4;  // first of this wavefront's 4 row tiles
-  const int m0 = mb * kGM;
+  const int m0 = mb * GM;
   const XT *x = static_cast<const XT *>(a.x);
   const int steps = (a.KC + 3) / 4;  // 4 chunks of 32 K per step
 
@@ -575,35 +586,39 @@ __global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, i
     wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + lane * 8;
   }
   auto load_w = [&](int t, int cc) -> half8_t {
+    if constexpr (FULL) return load_h8(wt[t] + static_cast<int64_t>(cc) * 512);
     return (wok[t] && cc < a.KC) ? load_h8(wt[t] + static_cast<int64_t>(cc) * 512) : zero_h8();
   };
-  // x staging: 128 rows x 16 units of 16 bytes per step = 2048 vectors, 8 per thread
-  auto load_x = [&](int step, half8_t (&xv)[8]) {
+  // x staging: GM rows x 16 units of 16 bytes per step, XV per thread
+  auto load_x = [&](int step, half8_t (&xv)[XV]) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < XV; ++p) {
       const int v = p * 256 + tid;
       const int row = v >> 4, unit = v & 15;
       const int m = m0 + row, k = step * kGK + unit * 8;
-      xv[p] = (m < a.M && k + 8 <= a.K) ? load_h8(x + static_cast<int64_t>(m) * a.K + k) : zero_h8();
+      if constexpr (FULL)
+        xv[p] = load_h8(x + static_cast<int64_t>(min(m, a.M - 1)) * a.K + k);
+      else
+        xv[p] = (m < a.M && k + 8 <= a.K) ? load_h8(x + static_cast<int64_t>(m) * a.K + k) : zero_h8();
     }
   };
-  auto store_x = [&](int buf, const half8_t (&xv)[8]) {
+  auto store_x = [&](int buf, const half8_t (&xv)[XV]) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < XV; ++p) {
       const int v = p * 256 + tid;
       const int row = v >> 4, unit = v & 15;
       *reinterpret_cast<half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]) = xv[p];
     }
   };
 
-  float4_t acc[4][8];
+  float4_t acc[4][MT];
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
-    for (int u = 0; u < 8; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < MT; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   half8_t wf[4][4];  // [row tile][chunk within the step]
-  half8_t xv[8];
+  half8_t xv[XV];
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -614,26 +629,33 @@ __global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, i
 
   for (int i = 0; i < steps; ++i) {
     const int buf = i & 1;
-    const bool more = i + 1 < steps;
-    if (more) load_x(i + 1, xv);
+    // FULL: the loop body is branch-free - the last step fetches its own data once more instead of
+    // skipping the prefetch, so the compiler can count outstanding loads exactly
+    const bool more = FULL || i + 1 < steps;
+    const int nxt = FULL ? min(i + 1, steps - 1) : i + 1;
+    if (more) load_x(nxt, xv);
+    // keep the prefetches where they are written: left alone, the scheduler sinks them to the end of
+    // the step (shorter live ranges) and the step then waits out a full memory latency
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      half8_t bf[8];
+      half8_t bf[MT];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < MT; ++u) {
         const int row = u * 16 + r, unit = j * 4 + g;
         bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
       }
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+        for (int u = 0; u < MT; ++u)
           acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[t][j], bf[u], acc[t][u], 0, 0, 0);
       // the fragments of chunk j are consumed: fetch chunk j of the next step into the same registers
       if (more) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) wf[t][j] = load_w(t, (i + 1) * 4 + j);
+        for (int t = 0; t < 4; ++t) wf[t][j] = load_w(t, nxt * 4 + j);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (more) store_x(buf ^ 1, xv);
     __syncthreads();
@@ -646,7 +668,7 @@ __global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, i
   o.N = a.glu ? a.N / 2 : a.N;
   o.out_f16 = a.out_f16;
 #pragma unroll
-  for (int u = 0; u < 8; ++u) {
+  for (int u = 0; u < MT; ++u) {
     const int m = m0 + u * 16 + r;
     if (a.glu) {
 #pragma unroll
@@ -671,10 +693,19 @@ __global__ __launch_bounds__(256) void linear_gemm_packed_kernel(PackedArgs a, i
 
 template <typename XT>
 void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
-  const int n_blocks = (a.N + kGN - 1) / kGN, m_blocks = (a.M + kGM - 1) / kGM;
+  const int gm = g_gemm_rows > 0 ? g_gemm_rows : 64;
+  const int n_blocks = (a.N + kGN - 1) / kGN, m_blocks = (a.M + gm - 1) / gm;
   const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;  // whole rounds over the XCDs
   const dim3 grid(static_cast<unsigned>(nb_pad) * m_blocks);
-  hipLaunchKernelGGL((linear_gemm_packed_kernel<XT>), grid, dim3(256), 0, st, a, n_blocks, m_blocks);
+  const bool full = a.K % kGK == 0;
+#define AXHIP_GEMM_LAUNCH(F, G) \
+  hipLaunchKernelGGL((linear_gemm_packed_kernel<XT, F, G>), grid, dim3(256), 0, st, a, n_blocks, m_blocks)
+  if (gm == 128) {
+    if (full) AXHIP_GEMM_LAUNCH(true, 128); else AXHIP_GEMM_LAUNCH(false, 128);
+  } else {
+    if (full) AXHIP_GEMM_LAUNCH(true, 64); else AXHIP_GEMM_LAUNCH(false, 64);
+  }
+#undef AXHIP_GEMM_LAUNCH
 }
 
 }  // namespace
@@ -685,7 +716,8 @@ using namespace axhip;
 extern "C" {
 
 // Measurement hook for sweeps (0 restores a default).
-AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves) {
+AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows) {
+  g_gemm_rows = (gemm_rows == 64 || gemm_rows == 128) ? gemm_rows : 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;
@@ -786,7 +818,7 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
     ga.chunks_per_wave = 0;
     ga.out_f16 = out_dtype == AXHIP_FLOAT16;
     ga.glu = glu ? 1 : 0;
-    const int64_t wgs = ((N + kGN - 1) / kGN + kXcds - 1) / kXcds * kXcds * ((M + kGM - 1) / kGM);
+    const int64_t wgs = ((N + kGN - 1) / kGN + kXcds - 1) / kXcds * kXcds * ((M + 63) / 64);
     if (wgs > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
     if (x_dtype == AXHIP_FLOAT16)
       launch_gemm_packed<__half>(ga, as_stream(stream));

@@ -5,7 +5,7 @@ the host-side mirror of the reference's Python surface for that path: the same n
 `axono` (axono/python/axono/__init__.py:46-113) for the operators, `nn`, `fused`, `gqa`, `compile`
 and graph capture, on the device strings "hip" / "hip:<id>".
 """
-from . import fused, gqa, nn  # noqa: F401
+from . import format, fused, gqa, nn  # noqa: F401,A004
 from .core import DataType, Status, Tensor, cuda_available, get_default_device, hip_available, set_default_device
 from .core.backend import get_backend, set_backend
 from .core.compile import compile  # noqa: A004

@@ -77,6 +77,65 @@ def random_weights(cfg: TextConfig, seed: int = 0) -> dict:
     return w
 
 
+# ---- AXM1 weight files --------------------------------------------------------------------------
+# The reference stores the text tower under "model.language_model." with separate q/k/v and gate/up
+# projections (examples/vlm/qwen3vl/model.py:323-326,379-381,595-621); this model keeps them fused.
+AXM_TEXT_PREFIX = "model.language_model."
+
+
+def weights_to_axm(weights: dict, cfg: TextConfig, path: str, prefix: str = AXM_TEXT_PREFIX) -> None:
+    """Writes `weights` (this module's fused naming) as an .axm file in the reference's naming."""
+    from ..format import save_axm
+
+    D, nq, nkv, I = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.intermediate_size
+    out = {}
+    for name, arr in weights.items():
+        if name.endswith("self_attn.qkv_proj.weight"):
+            base = name[: -len("qkv_proj.weight")]
+            out[prefix + base + "q_proj.weight"] = arr[: nq * D]
+            out[prefix + base + "k_proj.weight"] = arr[nq * D: (nq + nkv) * D]
+            out[prefix + base + "v_proj.weight"] = arr[(nq + nkv) * D:]
+        elif name.endswith("mlp.gate_up_proj.weight"):
+            base = name[: -len("gate_up_proj.weight")]
+            out[prefix + base + "gate_proj.weight"] = arr[:I]
+            out[prefix + base + "up_proj.weight"] = arr[I:]
+        else:
+            out[prefix + name] = arr
+    save_axm(out, path, meta={"text_config": dict(cfg.__dict__)})
+
+
+def weights_from_axm(path: str, cfg: TextConfig, prefix: str = AXM_TEXT_PREFIX) -> dict:
+    """Reads the text tower of an .axm file into this module's naming and storage formats: Linear and
+    embedding weights fp16 (what `cast_linear_fp16` makes of them, nn/module.py:158-184), norm weights
+    fp32, q/k/v and gate/up concatenated along the output axis.  Tensors outside `prefix` are
+    ignored (the vision tower); a missing tensor raises KeyError."""
+    from ..format import AxmReader
+
+    r = AxmReader(path)
+    have = {n[len(prefix):]: n for n in r.names() if n.startswith(prefix)}
+
+    def get(name, dtype):
+        return np.asarray(r.get(have[name])).astype(dtype, copy=False)
+
+    def fused(base, parts, whole):
+        if base + whole in have:
+            return get(base + whole, np.float16)
+        return np.concatenate([get(base + p, np.float16) for p in parts], axis=0)
+
+    w = {"embed_tokens.weight": get("embed_tokens.weight", np.float16), "norm.weight": get("norm.weight", np.float32)}
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        w[p + "self_attn.qkv_proj.weight"] = fused(p + "self_attn.", ["q_proj.weight", "k_proj.weight", "v_proj.weight"],
+                                                   "qkv_proj.weight")
+        w[p + "mlp.gate_up_proj.weight"] = fused(p + "mlp.", ["gate_proj.weight", "up_proj.weight"], "gate_up_proj.weight")
+        for n in ("self_attn.o_proj.weight", "mlp.down_proj.weight"):
+            w[p + n] = get(p + n, np.float16)
+        for n in ("self_attn.q_norm.weight", "self_attn.k_norm.weight", "input_layernorm.weight",
+                  "post_attention_layernorm.weight"):
+            w[p + n] = get(p + n, np.float32)
+    return w
+
+
 def _dev(arr, device):
     return Tensor.from_numpy_ref(np.ascontiguousarray(arr)).to(device)
 

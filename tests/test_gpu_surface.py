@@ -196,6 +196,54 @@ def test_dynamic_kv_cache_with_attention():
         np.testing.assert_allclose(step.to_numpy()[0], full[i], rtol=1e-4, atol=1e-5)
 
 
+def test_custom_sliding_window_cache_component():
+    """tests/nn/test_kv_cache.py:75-114 of the reference: a user-written KVCache that keeps the last
+    two steps with concat + slice_; also get() before update() and independent layers (:60-73)."""
+
+    class SlidingWindowCache(nn.KVCache):
+        def __init__(self, window=2):
+            self.window, self.k, self.v = window, None, None
+
+        def update(self, layer_idx, k_new, v_new):
+            if self.k is None:
+                self.k, self.v = k_new, v_new
+            else:
+                self.k, self.v = axono.concat(self.k, k_new, 0), axono.concat(self.v, v_new, 0)
+            extra = int(self.k.shape[0]) - self.window
+            if extra > 0:
+                self.k = axono.slice_(self.k, 0, extra, self.window)
+                self.v = axono.slice_(self.v, 0, extra, self.window)
+
+        def get(self, layer_idx):
+            return self.k, self.v
+
+        def reset(self):
+            self.k = self.v = None
+
+        def __len__(self):
+            return 0 if self.k is None else int(self.k.shape[0])
+
+    def kv(seed, steps=1):
+        return np.random.RandomState(seed).randn(steps, 1, 4).astype(np.float32)
+
+    cache = SlidingWindowCache(window=2)
+    for i in range(4):
+        cache.update(0, t(kv(i)), t(kv(i + 10)))
+    assert len(cache) == 2
+    np.testing.assert_array_equal(cache.get(0)[0].to_numpy(), np.concatenate([kv(2), kv(3)]))
+    np.testing.assert_array_equal(cache.get(0)[1].to_numpy(), np.concatenate([kv(12), kv(13)]))
+    cache.reset()
+    assert len(cache) == 0
+
+    dyn = nn.DynamicKVCache(2, device=DEV)
+    with pytest.raises(RuntimeError):
+        dyn.get(0)
+    dyn.update(0, t(kv(0, 2)), t(kv(1, 2)))
+    dyn.update(1, t(kv(2, 5)), t(kv(3, 5)))
+    assert len(dyn) == 2                      # the first non-empty layer's length
+    assert dyn.get(0)[0].to_numpy().shape == (2, 1, 4) and dyn.get(1)[0].to_numpy().shape == (5, 1, 4)
+
+
 def test_static_kv_cache_matches_dynamic():
     rng = np.random.default_rng(5)
     B, hkv, d, lmax = 3, 2, 64, 16
@@ -317,3 +365,24 @@ def test_allocator_cache_and_budget():
     del z
     assert L.cached_bytes() <= 1 << 20
     L.set_cache_budget(64 << 30)
+
+
+def test_axm_weights_go_straight_to_the_device(tmp_path):
+    """save_axm -> load_axm_to_device: values arrive unchanged; dtype="float16" converts floating
+    tensors on the way (one IEEE rounding) and leaves integer tensors alone."""
+    from axono_amd.format import load_axm_to_device, save_axm
+
+    rng = np.random.default_rng(3)
+    sd = {"w": rng.standard_normal((33, 70)).astype(np.float32), "h": rng.standard_normal((5, 8)).astype(np.float16),
+          "ids": np.arange(12, dtype=np.int64)}
+    p = str(tmp_path / "w.axm")
+    save_axm(sd, p)
+    dev = load_axm_to_device(p, "hip")
+    assert set(dev) == set(sd)
+    for k, v in sd.items():
+        assert dev[k].device.startswith("hip") and dev[k].shape == list(v.shape)
+        np.testing.assert_array_equal(dev[k].numpy(), v)
+    dev16 = load_axm_to_device(p, "hip", dtype="float16", names=["w", "ids"])
+    assert set(dev16) == {"w", "ids"}
+    np.testing.assert_array_equal(dev16["w"].numpy(), sd["w"].astype(np.float16))
+    np.testing.assert_array_equal(dev16["ids"].numpy(), sd["ids"])

@@ -1,0 +1,281 @@
+// Causal attention for prefill on the matrix cores: S query tokens per sequence attend to the keys
+// already written to the static KV cache [B, Hkv, rows, D] (fp16), query i of sequence b sitting at
+// absolute position start[b] + i and seeing keys 0 .. start[b] + i.
+//
+// Work decomposition.  One workgroup (4 wavefronts) owns 64 consecutive positions of one sequence
+// and the G query heads of one kv-head group; a wavefront owns 16 of those positions for all G
+// heads, i.e. G "query tiles" of 16 rows that share every K and V fragment it reads.  K and V
+// travel through LDS in stages of 64 keys (double-buffered, 16-byte units XOR-swizzled by key so
+// that fragment reads of 16 keys hit 16 different bank groups).
+//
+// Everything is computed transposed so that no operand ever has to change layout in registers:
+//   S^T = K . Q^T   A = K rows (16 keys x 32 d), B = Q rows       -> C: lane owns query l%16,
+//                                                                     keys 4*(l/16) + e
+//   O^T = V^T . P^T A = V^T (16 d x 32 keys),    B = P^T           -> C: lane owns query l%16,
+//                                                                     d = 4*(l/16) + e
+// P^T in the B layout needs, per lane, 8 keys of its own query: exactly what the lane holds after
+// two S^T tiles (keys 4g+e of each), if the 32 keys of a block are taken in the order
+// k' = 8g + j <-> key 4g + j (j < 4), 16 + 4g + (j - 4) (j >= 4).  V^T fragments in that same key
+// order come from row-major V in LDS through the transposing LDS read of gfx950
+// (ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of 4 consecutive elements and
+// receives element i of each of the 4 rows of 16 elements the group addressed).  The running
+// maximum and the rescale factor of a query live in the lanes that own that query in both products.
+//
+// Softmax: online, log2 domain, fp32; P is rounded to fp16 for the second product (values in
+// [0, 1]); the row sum is kept per lane and reduced once at the end.
+#include "common.hpp"
+
+namespace axhip {
+namespace {
+
+constexpr int kPThreads = 256;
+constexpr int kPosPerWg = 64;   // query positions per workgroup (16 per wavefront)
+constexpr int kStageKeys = 64;  // keys per LDS stage
+constexpr float kMasked = -1.0e30f;
+
+struct PrefillArgs {
+  const __half *q;   // [B, S, Hq, D]
+  const __half *k;   // [B, Hkv, rows, D]
+  const __half *v;
+  const int32_t *start;  // [B] absolute position of query 0 (null: 0)
+  __half *out;       // [B, S, Hq, D]
+  int S, Hq, Hkv, rows, group;
+  float scale_log2e;
+};
+
+__device__ __forceinline__ half8_t lds_h8(const _Float16 *p) { return *reinterpret_cast<const half8_t *>(p); }
+
+// 4 keys x 16 d of row-major V, delivered transposed: this lane gets V[key0 .. key0+3][d0 + lane%16].
+// `row_base` points at V[key0][0] of the stage in LDS for this lane's group; rows are 2*D bytes.
+template <int D>
+__device__ __forceinline__ half4_t lds_v_tr(const _Float16 *stage, int key0, int d0, int c) {
+  const int key = key0 + (c >> 2);           // the row this lane addresses
+  const int unit = (d0 >> 3) + ((c & 3) >> 1);  // 16-byte unit within the row
+  const _Float16 *p = stage + key * D + ((unit ^ (key & (D / 8 - 1))) << 3) + ((c & 1) << 2);
+  typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+  const fp16x4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p));
+  return __builtin_bit_cast(half4_t, r);
+}
+
+template <int D, int G>
+__global__ __launch_bounds__(kPThreads) void prefill_attn_kernel(PrefillArgs a) {
+  constexpr int KK = D / 32;   // MFMA steps over d for S^T
+  constexpr int DT = D / 16;   // d tiles of O^T
+  constexpr int UPR = D / 8;   // 16-byte units per K/V row
+  constexpr int VEC = kStageKeys * UPR / kPThreads;  // staging vectors per thread, per tensor
+  __shared__ __attribute__((aligned(16))) _Float16 ks[2][kStageKeys * D];
+  __shared__ __attribute__((aligned(16))) _Float16 vs[2][kStageKeys * D];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const int pb = gridDim.x - 1 - blockIdx.x;  // long rows first
+  const int hg = blockIdx.y, b = blockIdx.z;
+  const int h0 = hg * G, hk = h0 / a.group;
+  const int start = a.start ? max(a.start[b], 0) : 0;
+  const int p0 = pb * kPosPerWg;
+  const int pr = p0 + wave * 16 + c;           // this lane's query (as B column), relative position
+  const int pos = start + pr;                  // its absolute position = last visible key
+  const int wave_last = start + p0 + wave * 16 + 15;
+  int k_end = start + min(p0 + kPosPerWg, a.S);  // keys the workgroup needs: [0, k_end)
+  k_end = min(k_end, a.rows);
+
+  // Q fragments stay in registers for the whole kernel
+  half8_t qf[G][KK];
+  {
+    const int prc = min(pr, a.S - 1);
+    const __half *qrow = a.q + ((static_cast<int64_t>(b) * a.S + prc) * a.Hq + h0) * D;
+#pragma unroll
+    for (int t = 0; t < G; ++t)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+        qf[t][kk] = *reinterpret_cast<const half8_t *>(qrow + t * D + kk * 32 + g * 8);
+  }
+
+  const __half *kbase = a.k + (static_cast<int64_t>(b) * a.Hkv + hk) * a.rows * D;
+  const __half *vbase = a.v + (static_cast<int64_t>(b) * a.Hkv + hk) * a.rows * D;
+  half8_t kst[VEC], vst[VEC];
+  auto load_stage = [&](int key0) {
+#pragma unroll
+    for (int p = 0; p < VEC; ++p) {
+      const int vi = p * kPThreads + tid;
+      const int row = vi / UPR, unit = vi % UPR;
+      const int64_t off = static_cast<int64_t>(min(key0 + row, a.rows - 1)) * D + unit * 8;
+      kst[p] = *reinterpret_cast<const half8_t *>(kbase + off);
+      vst[p] = *reinterpret_cast<const half8_t *>(vbase + off);
+    }
+  };
+  // V rows past the last key any query of this workgroup may see are stored as zeros: their
+  // probabilities are zero, but 0 * (whatever bits the unwritten cache holds) must stay 0
+  auto store_stage = [&](int buf, int key0) {
+#pragma unroll
+    for (int p = 0; p < VEC; ++p) {
+      const int vi = p * kPThreads + tid;
+      const int row = vi / UPR, unit = vi % UPR;
+      const int o = row * D + ((unit ^ (row & (UPR - 1))) << 3);
+      *reinterpret_cast<half8_t *>(&ks[buf][o]) = kst[p];
+      half8_t vv = vst[p];
+      if (key0 + row >= k_end) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      *reinterpret_cast<half8_t *>(&vs[buf][o]) = vv;
+    }
+  };
+
+  float4_t o[G][DT];
+  float m[G], lsum[G];
+#pragma unroll
+  for (int t = 0; t < G; ++t) {
+    m[t] = kMasked;
+    lsum[t] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[t][dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int n_stages = (k_end + kStageKeys - 1) / kStageKeys;
+  load_stage(0);
+  store_stage(0, 0);
+  __syncthreads();
+
+  for (int s = 0; s < n_stages; ++s) {
+    const int buf = s & 1;
+    const int nxt = min(s + 1, n_stages - 1);  // the last stage fetches itself again: no branch
+    load_stage(nxt * kStageKeys);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int sub = 0; sub < kStageKeys / 32; ++sub) {
+      const int kb = s * kStageKeys + sub * 32;      // first key of this block of 32
+      if (kb <= wave_last && kb < k_end) {           // wave-uniform: otherwise every key is masked
+        const _Float16 *kst_l = &ks[buf][sub * 32 * D];
+        // ---- S^T = K . Q^T for two tiles of 16 keys ----
+        float4_t sc[G][2];
+#pragma unroll
+        for (int t = 0; t < G; ++t) sc[t][0] = sc[t][1] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) {
+            const int row = tk * 16 + c, unit = kk * 4 + g;  // row & 15 == c
+            const half8_t kf = lds_h8(kst_l + row * D + ((unit ^ (c & (UPR - 1))) << 3));
+#pragma unroll
+            for (int t = 0; t < G; ++t)
+              sc[t][tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][kk], sc[t][tk], 0, 0, 0);
+          }
+        // ---- mask, online softmax ----
+        const bool diag = kb + 31 > start + p0 + wave * 16;  // some key of the block may be masked
+        half8_t pf[G];
+#pragma unroll
+        for (int t = 0; t < G; ++t) {
+          float x[8];
+#pragma unroll
+          for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int key = kb + tk * 16 + 4 * g + e;
+              float v = sc[t][tk][e] * a.scale_log2e;
+              if (diag && key > pos) v = kMasked;
+              x[tk * 4 + e] = v;
+            }
+          float mx = x[0];
+#pragma unroll
+          for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
+          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          const float mn = fmaxf(m[t], mx);
+          const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
+          m[t] = mn;
+          float ps = 0.f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            float p = __builtin_amdgcn_exp2f(x[j] - mn);
+            if (x[j] <= kMasked) p = 0.f;  // a fully masked row keeps m == kMasked: exp2(0) would count
+            ps += p;
+            pf[t][j] = static_cast<_Float16>(p);
+          }
+          lsum[t] = lsum[t] * corr + ps;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
+        }
+        // ---- O^T += V^T . P^T ----
+        const _Float16 *vst_l = &vs[buf][sub * 32 * D];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const half4_t lo = lds_v_tr<D>(vst_l, 4 * g, dt * 16, c);
+          const half4_t hi = lds_v_tr<D>(vst_l, 16 + 4 * g, dt * 16, c);
+          const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+          for (int t = 0; t < G; ++t)
+            o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][dt], 0, 0, 0);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    store_stage(buf ^ 1, nxt * kStageKeys);
+    __syncthreads();
+  }
+
+  if (pr >= a.S) return;
+  __half *orow = a.out + ((static_cast<int64_t>(b) * a.S + pr) * a.Hq + h0) * D;
+#pragma unroll
+  for (int t = 0; t < G; ++t) {
+    float l = lsum[t];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      half4_t h;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(o[t][dt][e] * inv);
+      *reinterpret_cast<half4_t *>(reinterpret_cast<_Float16 *>(orow) + t * D + dt * 16 + 4 * g) = h;
+    }
+  }
+}
+
+template <int D>
+int launch_prefill(const PrefillArgs &a, int B, int G, hipStream_t st) {
+  const dim3 grid((a.S + kPosPerWg - 1) / kPosPerWg, a.Hq / G, B);
+  switch (G) {
+    case 4: hipLaunchKernelGGL((prefill_attn_kernel<D, 4>), grid, dim3(kPThreads), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((prefill_attn_kernel<D, 2>), grid, dim3(kPThreads), 0, st, a); break;
+    default: hipLaunchKernelGGL((prefill_attn_kernel<D, 1>), grid, dim3(kPThreads), 0, st, a); break;
+  }
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace axhip
+
+using namespace axhip;
+
+extern "C" {
+
+AXHIP_API int axhip_prefill_attention(const void *q, const void *k_cache, const void *v_cache,
+                                      const int32_t *start, void *out, int dtype, int B, int S, int Hq,
+                                      int Hkv, int D, int cache_rows, axhip_stream stream) {
+  if (dtype != AXHIP_FLOAT16) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || S < 0 || Hq <= 0 || Hkv <= 0 || cache_rows <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (Hq % Hkv != 0) return AXHIP_SHAPE_MISMATCH;
+  if (D != 64 && D != 128) return AXHIP_INVALID_ARGUMENT;
+  if (B == 0 || S == 0) return AXHIP_OK;
+  if (B > 65535 || Hq > 65535) return AXHIP_INVALID_ARGUMENT;
+  if (!q || !k_cache || !v_cache || !out) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache) |
+       reinterpret_cast<uintptr_t>(out)) & 15)
+    return AXHIP_INVALID_PTR;
+  const int group = Hq / Hkv;
+  const int G = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  PrefillArgs a;
+  a.q = static_cast<const __half *>(q);
+  a.k = static_cast<const __half *>(k_cache);
+  a.v = static_cast<const __half *>(v_cache);
+  a.start = start;
+  a.out = static_cast<__half *>(out);
+  a.S = S;
+  a.Hq = Hq;
+  a.Hkv = Hkv;
+  a.rows = cache_rows;
+  a.group = group;
+  a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
+  hipStream_t st = as_stream(stream);
+  return D == 128 ? launch_prefill<128>(a, B, G, st) : launch_prefill<64>(a, B, G, st);
+}
+
+}  // extern "C"

@@ -258,10 +258,16 @@ class Qwen3VLTextDecoder(nn.Module):
                     vc.data_ptr + seq_off, int(DataType.FLOAT16), 1, S, nq, nkv, D, lmax, current_stream()),
                     "qkv_norm_rope_append")
                 attn = Tensor(DataType.FLOAT16, [S, nq * D], dev, _zero=False)
-                # every query row is a "sequence" of the decode kernel over this sequence's cache rows
-                check(lib.axhip_gqa_decode(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, vis.data_ptr,
-                                           attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq, nkv,
-                                           D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
+                if D in (64, 128):
+                    # causal attention over the rows just appended, on the matrix cores
+                    check(lib.axhip_prefill_attention(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, None,
+                                                      attn.data_ptr, int(DataType.FLOAT16), 1, S, nq, nkv, D, lmax,
+                                                      current_stream()), "prefill_attention")
+                else:
+                    # every query row is a "sequence" of the decode kernel over this sequence's cache rows
+                    check(lib.axhip_gqa_decode(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, vis.data_ptr,
+                                               attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq,
+                                               nkv, D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
                 attn_out = L.linear_nobias(attn, self._w(p + "self_attn.o_proj.weight"))
                 h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                     DataType.FLOAT16)

@@ -518,6 +518,29 @@ def qkv_norm_rope_append(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, eps: f
     return q_out
 
 
+def prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, start: Tensor | None = None) -> Tensor:
+    """Causal attention of S new tokens per sequence over a static cache that already holds their
+    keys / values: q FLOAT16 [B,S,Hq,D], caches FLOAT16 [B,Hkv,rows,D], start INT32 [B] = absolute
+    position of query 0 (None: 0).  Returns FLOAT16 [B,S,Hq,D]."""
+    op = "scaled_dot_product_attention"
+    _need_hip(op, q, k_cache, v_cache, start)
+    if q.dtype != DataType.FLOAT16 or k_cache.dtype != DataType.FLOAT16 or v_cache.dtype != DataType.FLOAT16:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    if q.ndim != 4 or k_cache.ndim != 4 or v_cache.shape != k_cache.shape:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    B, S, hq, d = q.shape
+    if k_cache.shape[0] != B or k_cache.shape[3] != d:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if start is not None and (start.dtype != DataType.INT32 or start.num_elements != B):
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    out = _new(DataType.FLOAT16, [B, S, hq, d], q)
+    check(_lib_().axhip_prefill_attention(q.data_ptr, k_cache.data_ptr, v_cache.data_ptr,
+                                          start.data_ptr if start is not None else None, out.data_ptr,
+                                          int(DataType.FLOAT16), B, S, hq, k_cache.shape[1], d, k_cache.shape[2],
+                                          current_stream()), op)
+    return out
+
+
 def gqa_decode_attention_qkv(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, eps: float, pos: Tensor, inv_freq: Tensor,
                              mrope_section, seq_lens: Tensor, k_cache: Tensor, v_cache: Tensor, n_q_heads: int,
                              max_len: int | None = None, workspace: Tensor | None = None) -> Tensor:

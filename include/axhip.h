@@ -353,6 +353,16 @@ AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const
                                          void *k_cache, void *v_cache, int cache_dtype, int B, int S,
                                          int Hq, int Hkv, int D, int Lmax, axhip_stream stream);
 
+/* Causal attention for prefill on the matrix cores: q [B,S,Hq,D] fp16, keys / values already in the
+ * caches [B,Hkv,cache_rows,D] fp16; query i of sequence b sits at absolute position start[b] + i
+ * (start NULL: 0) and attends to cache rows 0 .. start[b] + i.  out [B,S,Hq,D] fp16.  D = 64 or 128.
+ * Same result as ops::cuda::ScaledDotProductAttention with is_causal (src/ops/cuda/sequence.cu:105-163,
+ * 451-472) on each sequence, with fp32 softmax statistics and probabilities rounded to fp16 for the
+ * second product. */
+AXHIP_API int axhip_prefill_attention(const void *q, const void *k_cache, const void *v_cache,
+                                      const int32_t *start, void *out, int dtype, int B, int S, int Hq,
+                                      int Hkv, int D, int cache_rows, axhip_stream stream);
+
 /* The attention block of one decode step in one launch (plus the split merge): equals
  * axhip_qkv_norm_rope_append with S = 1 followed by axhip_gqa_decode over seq_lens[b] + 1 keys of the
  * caches [B,Hkv,cache_rows,D], without materialising q and without a second read of the row just

@@ -232,3 +232,46 @@ def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
                                   max_len, None) == 7
     assert l.axhip_gqa_decode_qkv(*args, dl.ptr, dkc.ptr, dvc.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows,
                                   rows + 1, None) == 1
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,S,start", [(4, 2, 128, 200, [0, 37]), (2, 2, 128, 64, [0, 0]), (8, 2, 64, 130, [5, 300]),
+                                               (16, 8, 128, 257, [0, 1])])
+def test_prefill_attention_matches_causal_oracle(Hq, Hkv, D, S, start):
+    """axhip_prefill_attention (MFMA, fp16 probabilities) against the CPU operator with the causal
+    mask, per sequence: query i at absolute position start + i sees cache rows 0 .. start + i.  Cache
+    rows past the last visible key hold NaN bit patterns: they must not leak into the result."""
+    rng = np.random.default_rng(11)
+    B = len(start)
+    rows = max(start) + S + 70
+    q = rng.standard_normal((B, S, Hq, D)).astype(np.float16)
+    kc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
+    vc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
+    for b in range(B):
+        kc[b, :, start[b] + S:] = np.float16(np.nan)
+        vc[b, :, start[b] + S:] = np.float16(np.nan)
+    st = np.asarray(start, np.int32)
+    dq, dk, dv, ds = (gu.dev(a) for a in (q, kc, vc, st))
+    out = gu.DeviceBuffer(q.nbytes)
+    gu._run("axhip_prefill_attention", dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F16, B, S, Hq, Hkv, D, rows, None)
+    gu.synchronize()
+    got = out.download(np.float16, q.shape).astype(np.float32)
+    assert np.isfinite(got).all()
+    worst = 0.0
+    for b in range(B):
+        L = start[b] + S
+        k = np.ascontiguousarray(np.transpose(kc[b, :, :L], (1, 0, 2)), dtype=np.float32)   # [L, Hkv, D]
+        v = np.ascontiguousarray(np.transpose(vc[b, :, :L], (1, 0, 2)), dtype=np.float32)
+        for i in sorted({0, 1, 15, 16, 63, min(64, S - 1), S // 2, S - 2, S - 1}):
+            vis = start[b] + i + 1
+            want = port.sdpa(q[b, i:i + 1].astype(np.float32), k[:vis], v[:vis], False)[0]
+            worst = max(worst, float(np.abs(got[b, i] - want).max()))
+    assert worst <= 2e-3, worst
+    if max(start) == 0:   # whole sequences through the operator's own causal path
+        for b in range(B):
+            k = np.ascontiguousarray(np.transpose(kc[b, :, :S], (1, 0, 2)), dtype=np.float32)
+            v = np.ascontiguousarray(np.transpose(vc[b, :, :S], (1, 0, 2)), dtype=np.float32)
+            want = port.sdpa(q[b].astype(np.float32), k, v, True)
+            assert np.abs(got[b] - want).max() <= 2e-3
+    l = gu.lib()
+    assert l.axhip_prefill_attention(dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F32, B, S, Hq, Hkv, D, rows, None) == 3
+    assert l.axhip_prefill_attention(dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F16, B, S, Hq, Hkv, 256, rows, None) == 1

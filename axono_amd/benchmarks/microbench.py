@@ -94,6 +94,23 @@ def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag=
     return us
 
 
+def bench_prefill_attn(lib, B, S, steps, Hq=16, Hkv=8, D=128):
+    """Causal prefill attention: 4*D flops per visible (query, key) pair and query head."""
+    n = B * Hkv * S * D
+    q = DeviceBuffer(B * S * Hq * D * 2)
+    k, v, out = DeviceBuffer(n * 2), DeviceBuffer(n * 2), DeviceBuffer(B * S * Hq * D * 2)
+    for i, buf in enumerate((q, k, v)):
+        _rand_fill(buf, buf.nbytes, 100 + i)
+
+    def step():
+        check(lib.axhip_prefill_attention(q.ptr, k.ptr, v.ptr, None, out.ptr, F16, B, S, Hq, Hkv, D, S, None), "prefill")
+
+    us = _time(lib, step, steps)
+    fl = 4.0 * D * Hq * B * (S * (S + 1) / 2)
+    _emit({"op": "prefill_attention", "B": B, "S": S, "Hq": Hq, "Hkv": Hkv, "D": D, "us": round(us, 1),
+           "TFLOPs": round(fl / us / 1e6, 1), "pct_mfma_f16_peak": round(100 * fl / us / 1e6 / MFMA_F16_PEAK, 2)})
+
+
 def bench_copy(lib, mib, steps):
     n = mib * 2**20
     a, b = DeviceBuffer(n), DeviceBuffer(n)
@@ -194,7 +211,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "copy", "rowops", "linear", "linear-packed"])
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -223,6 +240,9 @@ def main(argv=None):
                 bench_gqa(lib, B, L, max(10, min(args.steps, int(2e9 // (B * L * 4096)) + 10)))
         lens = np.random.default_rng(0).integers(512, 32769, 32)
         bench_gqa(lib, 32, 32768, 20, lens, tag="gqa_ragged_512_32768")
+    elif args.what == "prefill-attn":
+        for S in (1024, 4096, 16384):
+            bench_prefill_attn(lib, max(1, min(args.B, 65536 // S)), S, max(5, min(args.steps, 20)))
     elif args.what == "copy":
         bench_copy(lib, args.mib, args.steps)
     elif args.what == "rowops":

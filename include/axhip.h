@@ -381,6 +381,28 @@ AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float
                                    size_t workspace_bytes, int cache_dtype, int B, int Hq, int Hkv, int D,
                                    int cache_rows, int max_len, axhip_stream stream);
 
+/* Everything of a decoder layer behind the attention, for M <= 16 rows, in one persistent launch:
+ *   h_mid = attn . Wo^T + h_in;  act = silu(g) * u with [g | u] = rmsnorm(h_mid, w_post) . Wgu^T;
+ *   h_out = act . Wd^T + h_mid;  y = rmsnorm(h_out, w_next) . Wn^T
+ * i.e. o_proj, AddRmsNorm, gate/up + SiluMul, down_proj, AddRmsNorm and the next Linear (the next layer's
+ * qkv projection or the lm_head) of examples/vlm/qwen3vl/model.py:371-373,384,408-436,483-486, with the
+ * arithmetic of the single operators.  attn fp16 [M,K1]; h_in / h_mid / h_out fp32 [M,H]; act fp16 [M,I]
+ * scratch; y fp32 [M,N_next]; norm weights fp32 [H]; the four weight matrices packed by
+ * axhip_linear_f16_pack (gate+up with glu = 1).  H <= 2048 and a multiple of 2048 / ... see the checks:
+ * H, K1 and I must be multiples of 2048 (K slices of whole 128-column steps for 16 wavefronts), N_next a
+ * multiple of 16.  The workgroups of the launch synchronise among themselves and must all be resident
+ * (one per CU is launched): launches of this entry point must not overlap on a device.  No reference
+ * counterpart. */
+AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const void *w_o, const float *w_post,
+                                      const void *w_gate_up, const void *w_down, const float *w_next,
+                                      const void *w_next_linear, float *h_mid, void *act, float *h_out, float *y,
+                                      int M, int H, int K1, int I, int N_next, float eps, axhip_stream stream);
+/* Barrier waits of axhip_decode_layer_tail that ran out (0 in a healthy process); reset != 0 also clears the
+ * barrier state (only while no such launch is in flight).  Measurement hook: workgroups to launch (0 = one
+ * per CU, at most 256). */
+AXHIP_API int axhip_decode_layer_tail_status(int reset, unsigned *failed_waits);
+AXHIP_API void axhip_decode_layer_tail_tune(int workgroups);
+
 /* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
  * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0.  out_dtype
  * may be FLOAT16 for FLOAT32 input (see axhip_add_rms_norm_ex). */

@@ -81,7 +81,7 @@ PROTOTYPES = {
     "axhip_argmax": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
     "axhip_decode_layer_tail": (c_i, [c_vp] * 12 + [c_i] * 5 + [c_f, c_vp]),
     "axhip_decode_layer_tail_status": (c_i, [c_i, c_vp]),
-    "axhip_decode_layer_tail_tune": (None, [c_i]),
+    "axhip_decode_layer_tail_tune": (None, [c_i, c_i]),
     "axhip_prefill_attention": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_gqa_decode_qkv": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i, c_i, c_vp,
                                    c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),

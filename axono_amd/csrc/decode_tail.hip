@@ -9,9 +9,14 @@
 //
 // The same arithmetic as the single operators (fp16 Linear with fp32 accumulation, add_rms_norm
 // with evaluation order (x * rstd) * w, SiLU-mul) - only the five kernel boundaries between them are
-// replaced by barriers across the resident workgroups.  At 16 rows every one of those launches is
-// bounded by its start-up, one HBM round trip and its drain, not by bandwidth; a barrier costs
-// about 2 us.
+// replaced by barriers across the resident workgroups.
+//
+// Measured on MI355X at the 2B shape (16 rows, H 2048, I 6144, next N 4096, cold weights): 61 us per
+// launch - 16 us for the launch and its three barriers (2.5 us each plus 1.5 us for the cache
+// invalidate behind it), 6 / 20 / 10 / 9 us for the four phases - against about 51 us for the seven
+// launches it replaces inside a captured graph.  A phase still pays what a small kernel pays (one
+// HBM round trip for its weights, one write-through drain), and a kernel boundary inside a graph
+// turns out to be as cheap as a barrier, so the example model keeps this path switched off.
 //
 // One workgroup per CU (1024 threads = 16 wavefronts), workgroups stride over 16-row tiles of the
 // weight matrix; the wavefronts of a team split K and add their fragments through LDS (as in the
@@ -54,8 +59,7 @@ __device__ TailBarrier g_tail_bar;
 #define TAIL_ADD(p, v) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
 // k-th barrier of this launch (k = 1, 2, ...).  Returns false when the wait ran out.
-__device__ __forceinline__ bool grid_sync(unsigned k, int *s_ok) {
-  __builtin_amdgcn_s_waitcnt(0);  // this thread's write-through stores have completed
+__device__ __forceinline__ bool grid_sync(unsigned k, int *s_ok, bool fence = true) {
   __syncthreads();
   if (threadIdx.x == 0) {
     const unsigned n_wg = gridDim.x, wg = blockIdx.x;
@@ -77,10 +81,13 @@ __device__ __forceinline__ bool grid_sync(unsigned k, int *s_ok) {
         TAIL_ADD(&g_tail_bar.fail, 1u);
       }
     }
+    // one invalidate per workgroup (the vector L1 belongs to the CU, the non-coherent L2 lines to the
+    // XCD): later loads of any wavefront see the other workgroups' stores.  Issued by every wavefront
+    // it costs about 2 us apiece.
+    if (fence) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     *s_ok = ok;
   }
   __syncthreads();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // later loads see the other workgroups' stores
   return *s_ok != 0;
 }
 
@@ -99,6 +106,7 @@ struct TailArgs {
   float *y;             // [M, N_next] out
   int M, H, K1, I, N_next;
   float eps;
+  int skip;  // measurement: bit p set = phase p + 1 does no work (results are then meaningless)
 };
 
 // Loads through pointers known to be global memory: the phase functions are not inlined, so their
@@ -273,23 +281,27 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
   __shared__ int s_ok;
 
   // phase 1: o_proj + residual
-  linear_phase<1, 16, false, 0>(a.attn, a.M, a.K1, a.w_o, a.H, a.h_in, a.h_mid, a.H);
-  if (!grid_sync(1, &s_ok)) return;
+  if (!(a.skip & 1)) linear_phase<1, 16, false, 0>(a.attn, a.M, a.K1, a.w_o, a.H, a.h_in, a.h_mid, a.H);
+  __builtin_amdgcn_s_waitcnt(0);  // this thread's write-through stores have completed
+  if (!grid_sync(1, &s_ok, !(a.skip & 64))) return;
 
   // phase 2: post-attention norm, gate+up, SiLU-mul
-  stage_norm(a.h_mid, a.w_post, a.M, a.H, a.eps);
+  if (!(a.skip & 16)) stage_norm(a.h_mid, a.w_post, a.M, a.H, a.eps);
   __syncthreads();
-  linear_phase<2, 8, true, 1>(nullptr, a.M, a.H, a.w_gu, 2 * a.I, nullptr, a.act, a.I);
-  if (!grid_sync(2, &s_ok)) return;
+  if (!(a.skip & 2)) linear_phase<2, 8, true, 1>(nullptr, a.M, a.H, a.w_gu, 2 * a.I, nullptr, a.act, a.I);
+  __builtin_amdgcn_s_waitcnt(0);
+  if (!grid_sync(2, &s_ok, !(a.skip & 64))) return;
 
   // phase 3: down_proj + residual
-  linear_phase<1, 16, false, 0>(a.act, a.M, a.I, a.w_down, a.H, a.h_mid, a.h_out, a.H);
-  if (!grid_sync(3, &s_ok)) return;
+  if (!(a.skip & 4)) linear_phase<1, 16, false, 0>(a.act, a.M, a.I, a.w_down, a.H, a.h_mid, a.h_out, a.H);
+  __builtin_amdgcn_s_waitcnt(0);
+  if (!grid_sync(3, &s_ok, !(a.skip & 64))) return;
 
   // phase 4: the next norm and the Linear behind it
-  stage_norm(a.h_out, a.w_next, a.M, a.H, a.eps);
+  if (!(a.skip & 16)) stage_norm(a.h_out, a.w_next, a.M, a.H, a.eps);
   __syncthreads();
-  if (a.N_next >= 8192)
+  if (a.skip & 8) {
+  } else if (a.N_next >= 8192)
     linear_phase<2, 8, true, 2>(nullptr, a.M, a.H, a.w_nl, a.N_next, nullptr, a.y, a.N_next);
   else
     linear_phase<1, 16, true, 2>(nullptr, a.M, a.H, a.w_nl, a.N_next, nullptr, a.y, a.N_next);
@@ -307,6 +319,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
 }
 
 int g_tail_wgs = 0;  // resident workgroups to launch (0: one per CU, at most 256)
+int g_tail_skip = 0;
 
 }  // namespace
 }  // namespace axhip
@@ -363,6 +376,7 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
   a.I = I;
   a.N_next = N_next;
   a.eps = eps;
+  a.skip = g_tail_skip;
   static bool lds_set = false;  // more dynamic LDS than the default limit: raised once per process
   if (!lds_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tail_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -388,6 +402,9 @@ AXHIP_API int axhip_decode_layer_tail_status(int reset, unsigned *failed_waits) 
   return AXHIP_OK;
 }
 
-AXHIP_API void axhip_decode_layer_tail_tune(int workgroups) { g_tail_wgs = workgroups > 0 ? workgroups : 0; }
+AXHIP_API void axhip_decode_layer_tail_tune(int workgroups, int skip_phases) {
+  g_tail_wgs = workgroups > 0 ? workgroups : 0;
+  g_tail_skip = skip_phases;
+}
 
 }  // extern "C"

@@ -399,9 +399,10 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
                                       int M, int H, int K1, int I, int N_next, float eps, axhip_stream stream);
 /* Barrier waits of axhip_decode_layer_tail that ran out (0 in a healthy process); reset != 0 also clears the
  * barrier state (only while no such launch is in flight).  Measurement hook: workgroups to launch (0 = one
- * per CU, at most 256). */
+ * per CU, at most 256); skip_phases: bit p set = phase p + 1 does no work, bit 4 = no norm staging, bit 6 =
+ * no cache invalidate behind the barriers (timing only: results are then meaningless). */
 AXHIP_API int axhip_decode_layer_tail_status(int reset, unsigned *failed_waits);
-AXHIP_API void axhip_decode_layer_tail_tune(int workgroups);
+AXHIP_API void axhip_decode_layer_tail_tune(int workgroups, int skip_phases);
 
 /* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
  * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0.  out_dtype

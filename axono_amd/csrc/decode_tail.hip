@@ -194,7 +194,8 @@ __device__ __attribute__((noinline)) void linear_phase(const __half *xg, int M, 
 #pragma unroll
       for (int j = 0; j < kU; ++j)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) af[t][j] = tail_ld8(wt[t] + static_cast<int64_t>(c + j) * 512);
+        for (int t = 0; t < NT; ++t)
+          af[t][j] = __builtin_nontemporal_load((const TAIL_GLOBAL half8_t *)(wt[t] + static_cast<int64_t>(c + j) * 512));
       if constexpr (XLDS) {
 #pragma unroll
         for (int j = 0; j < kU; ++j) {

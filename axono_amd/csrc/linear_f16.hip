@@ -78,6 +78,11 @@ __device__ __forceinline__ half8_t load_h8(const __half *p) {
   return *reinterpret_cast<const half8_t *>(p);
 }
 
+// weight fragments are read once per launch: streaming (non-temporal) loads
+__device__ __forceinline__ half8_t load_h8_stream(const __half *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(p));
+}
+
 // 8 fp32 activations -> fp16 round-to-nearest-even (the conversion the reference applies to x
 // before its GEMM)
 __device__ __forceinline__ half8_t load_h8(const float *p) {
@@ -170,7 +175,7 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(LinearArgs a)
       const int kc = kk + (j * 4 + g) * 8;
       const bool kin = kc < k_end;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) af[t][j] = (kin && wok[t]) ? load_h8(wrow[t] + kc) : zero_h8();
+      for (int t = 0; t < NT; ++t) af[t][j] = (kin && wok[t]) ? load_h8_stream(wrow[t] + kc) : zero_h8();
 #pragma unroll
       for (int u = 0; u < MT; ++u) bf[u][j] = (kin && xok[u]) ? load_h8(xrow[u] + kc) : zero_h8();
     }
@@ -409,7 +414,7 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
       const bool in = c + j < c_end;
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        af[t][j] = (in && wok[t]) ? load_h8(wt[t] + static_cast<int64_t>(c + j) * 512) : zero_h8();
+        af[t][j] = (in && wok[t]) ? load_h8_stream(wt[t] + static_cast<int64_t>(c + j) * 512) : zero_h8();
     }
     // stage x[m_base .. +ROWS)[32c .. 32(c+U)): ROWS*UNITS vectors, 64 per pass
     half8_t xv[ROWS * UNITS / 64];

@@ -48,13 +48,13 @@ __global__ __launch_bounds__(kBlock) void rms_norm_kernel(const T *__restrict__ 
     int c = 0;
     for (int i = lane; i < nvec; i += TPR, ++c) {
       float a[8];
-      Row8<T>::load(x + off + i * 8, a);
+      Row8<T>::load_stream(x + off + i * 8, a);
       if (ADD) {
         float r[8];
-        Row8<T>::load(res + off + i * 8, r);
+        Row8<T>::load_stream(res + off + i * 8, r);
 #pragma unroll
         for (int j = 0; j < 8; ++j) a[j] += r[j];
-        Row8<T>::store(y + off + i * 8, a);  // the only rounding of y; the norm uses the fp32 sum
+        Row8<T>::store_stream(y + off + i * 8, a);  // the only rounding of y; the norm uses the fp32 sum
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(a[j], a[j], ss);
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_kernel(const T *__restrict__ 
 #pragma unroll
       for (int j = 0; j < 8; ++j) o[j] = a[j] * rms;
     }
-    Row8<OT>::store(out + off + i * 8, o);
+    Row8<OT>::store_stream(out + off + i * 8, o);
   }
   for (int i = nvec * 8 + lane; i < hidden; i += TPR) {
     float a = ldf(x + off + i);
@@ -215,8 +215,8 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ src,
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += stride) {
     float f[8];
-    Row8<S>::load(src + i * 8, f);
-    Row8<Dt>::store(dst + i * 8, f);
+    Row8<S>::load_stream(src + i * 8, f);
+    Row8<Dt>::store_stream(dst + i * 8, f);
   }
   if (blockIdx.x == 0) {
     for (int64_t i = nvec * 8 + threadIdx.x; i < n; i += kBlock) stf(dst + i, ldf(src + i));
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kBlock) void copy_bytes_kernel(const uint8_t *__res
   const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   if (vec_ok) {
     const int64_t nvec = n / 16;
-    for (int64_t i = t; i < nvec; i += stride) st16(dst + i * 16, ld16(src + i * 16));
+    for (int64_t i = t; i < nvec; i += stride) st16_stream(dst + i * 16, ld16_stream(src + i * 16));
     for (int64_t i = nvec * 16 + t; i < n; i += stride) dst[i] = src[i];
   } else {
     for (int64_t i = t; i < n; i += stride) dst[i] = src[i];

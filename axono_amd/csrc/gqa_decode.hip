@@ -28,12 +28,13 @@ constexpr float kNegBig = -1.0e30f;   // "no key seen yet" in the log2 domain (f
 constexpr int kMaxSplits = 128;
 constexpr int kChunkAlign = 128;      // key ranges start on multiples of this
 constexpr int kMinChunk = 256;
-constexpr int kLongChunk = 1024;
 
 struct Tuning {
-  int target_workgroups = 1024;  // 256 CUs x 4 resident workgroups
-  int force_splits = 0;          // > 0: fixed split count (measurement sweeps)
-  int separate_merge = 1;        // 1: merge in a second kernel; 0: the last workgroup merges
+  int target_workgroups = 256;  // workgroups that stream at a time: one per CU keeps HBM busy with
+                                // streaming loads (measured: 256 workgroups 153 us, 1024 163 us at
+                                // B=32 L=8192), and nothing has to be merged when a sequence is one
+  int force_splits = 0;         // > 0: fixed split count for every sequence (measurement sweeps)
+  int separate_merge = 0;       // 1: merge in a second kernel; 0: the last workgroup of a sequence merges
 };
 Tuning g_tuning;
 
@@ -44,30 +45,53 @@ Tuning g_tuning;
 constexpr int kTicketSlots = 1 << 16;
 __device__ unsigned int g_tickets[kTicketSlots];
 
+constexpr int kMaxDynBatch = 64;  // batches up to this size deal their workgroups by sequence length
+
+// How the key axis is cut.  The plan depends only on host-side sizes, so that a captured launch stays
+// valid while the device-side lengths change.
+//   dynamic (B <= kMaxDynBatch, no forced split count): the grid holds `active` workgroups per head
+//     group (one workgroup per CU over all head groups); on the device they are dealt to the
+//     sequences in proportion to their current lengths, so that every workgroup streams about
+//     (sum of lengths) / active keys whatever the mix of lengths is.  A batch of equal lengths gets
+//     active / B splits per sequence.  The launch is one-dimensional with the slot index slowest, so
+//     that the slots a launch leaves unused are the last workgroups dispatched: measured, a CU that
+//     gets two streaming workgroups while another gets none costs 28 % (B=8, L=8192: 56 us against
+//     44 us) - the memory pipeline of a CU holds about one workgroup's worth of loads in flight.
+//   static: every sequence is cut into n_splits ranges.
 struct SplitPlan {
-  int n_splits;
-  int chunk;
+  int n_splits;  // grid.x: workgroups per (sequence, head group) slot
+  int chunk;     // nominal keys per workgroup for max_len (reporting only)
+  int dynamic;
+  int active;    // dynamic: streaming workgroups per head group
+  int stride;    // splits a sequence can have at most (workspace stride)
 };
 
-// The key axis is cut into `n_splits` ranges of `chunk` keys.  The plan depends only on host-side
-// sizes so that a captured graph stays valid while the device-side lengths change.
 SplitPlan plan_splits(int B, int head_groups, int max_len) {
-  const long pairs = static_cast<long>(B) * head_groups > 0 ? static_cast<long>(B) * head_groups : 1;
+  SplitPlan p{};
+  const long hgs = head_groups > 0 ? head_groups : 1;
+  const long Bc = B > 0 ? B : 1;
+  if (g_tuning.force_splits == 0 && Bc <= kMaxDynBatch) {
+    long active = (g_tuning.target_workgroups + hgs - 1) / hgs;
+    const long cap = (Bc * max_len + kMinChunk - 1) / kMinChunk;  // no point in ranges shorter than kMinChunk
+    if (active > cap) active = cap;
+    if (active < 1) active = 1;
+    if (active < Bc) active = Bc;  // every sequence needs a workgroup of its own
+    p.dynamic = 1;
+    p.active = static_cast<int>(active);
+    p.n_splits = static_cast<int>((active + Bc - 1) / Bc);  // reporting: splits of a sequence when all are equal
+    p.stride = static_cast<int>(active < kMaxSplits ? active : kMaxSplits);
+    long c = (Bc * max_len + active - 1) / active;
+    p.chunk = static_cast<int>(c);
+    return p;
+  }
   long s;
   if (g_tuning.force_splits > 0) {
     s = g_tuning.force_splits;
   } else {
-    // Measured on MI355X: a workgroup streams best over >= 1024 keys (prologue, LDS merge and the
-    // partial write are per workgroup), so aim for target_workgroups with chunks that long ...
+    const long pairs = Bc * hgs;
     s = (g_tuning.target_workgroups + pairs - 1) / pairs;
-    const long cap_long = max_len / kLongChunk > 0 ? max_len / kLongChunk : 1;
-    if (s > cap_long) s = cap_long;
-    // ... unless that leaves most of the 256 CUs idle: then shorter chunks, down to kMinChunk keys
-    if (pairs * s < g_tuning.target_workgroups / 2) {
-      s = (g_tuning.target_workgroups / 2 + pairs - 1) / pairs;
-      const long cap = (max_len + kMinChunk - 1) / kMinChunk;
-      if (s > cap) s = cap;
-    }
+    const long cap = (max_len + kMinChunk - 1) / kMinChunk;
+    if (s > cap) s = cap;
   }
   if (s > kMaxSplits) s = kMaxSplits;
   if (s < 1) s = 1;
@@ -76,7 +100,10 @@ SplitPlan plan_splits(int B, int head_groups, int max_len) {
   if (chunk < kChunkAlign) chunk = kChunkAlign;
   s = (max_len + chunk - 1) / chunk;
   if (s < 1) s = 1;
-  return {static_cast<int>(s), static_cast<int>(chunk)};
+  p.n_splits = static_cast<int>(s);
+  p.chunk = static_cast<int>(chunk);
+  p.stride = p.n_splits;
+  return p;
 }
 
 // ---- 8 consecutive K or V elements as they come from memory --------------------------------------
@@ -148,6 +175,7 @@ struct DecodeArgs {
   float *part_acc;  // [B, Hq, n_splits, D]
   float *part_ml;   // [B, Hq, n_splits, 2]  (running max in log2 units, running sum)
   int Hq, group, max_len, chunk, n_splits;
+  int dynamic, active, split_stride, B, n_hg;  // see SplitPlan; split_stride = partial slots per (sequence, head)
   int64_t stride_b, stride_h, stride_s;
   float scale_log2e;
   int fused_merge;  // the last workgroup of a (sequence, head group) merges the splits
@@ -193,6 +221,62 @@ __device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int m
   len = len < 0 ? 0 : len;
   if (len_add && len < max_len) len += len_add;
   return len > max_len ? max_len : len;
+}
+
+// Which (sequence, split, head group) a workgroup works on, and how many splits that sequence has.
+// Static plan: straight from the grid.  Dynamic plan: workgroup id = slot * n_hg + head group; the
+// `active` slots of a head group are dealt by length - with c keys per workgroup, sequence b takes
+// max(1, ceil(len_b / c)) consecutive slots (the workgroup of an empty sequence writes zeros), and c
+// starts at ceil(sum of lengths / active) and grows until the slots suffice (a few rounds: the count
+// falls as c grows, and c = max_len needs B <= active slots).  Slots left over exit at once.  Every
+// wavefront builds the table in its registers: lane i holds sequence i (B <= 64), one vector load
+// for the lengths, wave sums, a wave prefix sum, one ballot.
+struct Work {
+  int b, k, n, hg;
+};
+__device__ __forceinline__ int dyn_splits_of(int len, int c, int stride) {
+  const int n = len > 0 ? (len + c - 1) / c : 1;
+  return n < stride ? n : stride;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ Work map_work(const DecodeArgs &a) {
+  if (!a.dynamic)
+    return Work{static_cast<int>(blockIdx.z), static_cast<int>(blockIdx.x), a.n_splits, static_cast<int>(blockIdx.y)};
+  const int lane = threadIdx.x & 63;
+  const int j = static_cast<int>(blockIdx.x) / a.n_hg, hg = static_cast<int>(blockIdx.x) % a.n_hg;
+  const bool live = lane < a.B;
+  const int len = live ? clamped_len(a.seq_lens, lane, a.max_len, a.len_add) : 0;
+  // sum of lengths in units of 64 keys (rounded up per sequence): fits an int for any supported size
+  const int total64 = wave_sum_i((len + 63) >> 6);
+  long long c64 = (static_cast<long long>(total64) * 64 + a.active - 1) / a.active;
+  int c = static_cast<int>(c64 < kMinDevChunk ? kMinDevChunk : (c64 > a.max_len ? a.max_len : c64));
+  int n = 0;
+#pragma unroll 1
+  for (int round = 0; round < 8; ++round) {
+    n = live ? dyn_splits_of(len, c, a.split_stride) : 0;
+    const int used = wave_sum_i(n);
+    if (used <= a.active) break;
+    // too many slots: grow c by the overshoot (at least one key), the last round takes one range each
+    const long long grown = (static_cast<long long>(c) * used + a.active - 1) / a.active;
+    c = round == 6 ? a.max_len : static_cast<int>(grown > a.max_len ? a.max_len : (grown > c ? grown : c + 1));
+  }
+  int incl = n;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  const int first = incl - n;
+  const unsigned long long hit = __ballot(j >= first && j < first + n);
+  if (hit == 0ull) return Work{-1, 0, 0, hg};
+  const int b = __ffsll(hit) - 1;
+  // the same in every lane: say so, so that everything derived from it lives in scalar registers
+  return Work{__builtin_amdgcn_readfirstlane(b), __builtin_amdgcn_readfirstlane(j - __shfl(first, b, 64)),
+              __builtin_amdgcn_readfirstlane(__shfl(n, b, 64)), hg};
 }
 
 // One head row of the qkv projection -> RMSNorm over the head (weights optional) -> interleaved
@@ -307,16 +391,19 @@ template <typename T, int D, int G, int U, bool QKV>
 __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArgs a) {
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
-  const int split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
-  const int len = clamped_len(a.seq_lens, b, a.max_len, QKV ? a.len_add : 0);
-  const int chunk = balanced_chunk(len, a.n_splits);
+  const Work wk = map_work(a);
+  if (wk.b < 0) return;  // a slot the lengths of this launch leave unused
+  const int split = wk.k, hg = wk.hg, b = wk.b;
+  const int len = clamped_len(a.seq_lens, b, a.max_len, a.len_add);
+  const int chunk = balanced_chunk(len, wk.n);
+  const int n_valid = (len + chunk - 1) / chunk;  // splits of this sequence that hold keys
   const int s0 = split * chunk;
   const int tid = threadIdx.x;
   const int h0 = hg * G;            // first query head of this workgroup
   if (s0 >= len) {
     // An empty split is never read by the merge.  A sequence without keys gets zeros, written by
     // its split-0 workgroup when no separate merge kernel will do it.
-    if (len == 0 && split == 0 && (a.n_splits == 1 || a.fused_merge)) {
+    if (len == 0 && split == 0 && (wk.n == 1 || a.fused_merge)) {
       for (int o = tid; o < G * D; o += kThreads)
         stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + h0) * D + o, 0.0f);
     }
@@ -349,7 +436,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
     // the first tile of cached keys is requested before q is prepared: those loads do not need it
     tile_load<T, D, U, true>(kb, vb, a.stride_s, s0, rg, kv_end, kr0, vr0);
     const int wave = tid >> 6, lane = tid & 63;
-    const int B = gridDim.z;
+    const int B = a.B;
     const bool writer = mine && (h0 % a.group == 0);
     for (int job = wave; job < G + (mine ? 2 : 0); job += kThreads / 64) {
       if (job < G) {
@@ -445,24 +532,24 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
       asum = __builtin_fmaf(s_acc[g][r][d], w, asum);
     }
     const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
-    if (a.n_splits == 1) {
+    if (n_valid == 1 && (wk.n == 1 || a.fused_merge)) {
+      // the only range of this sequence: normalise and write the result, nothing to merge
       stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
     } else {
-      st_agent(&a.part_acc[(bh * a.n_splits + split) * D + d], asum);
+      st_agent(&a.part_acc[(bh * a.split_stride + split) * D + d], asum);
       if (d == 0) {
-        st_agent(&a.part_ml[(bh * a.n_splits + split) * 2], mx);
-        st_agent(&a.part_ml[(bh * a.n_splits + split) * 2 + 1], lsum);
+        st_agent(&a.part_ml[(bh * a.split_stride + split) * 2], mx);
+        st_agent(&a.part_ml[(bh * a.split_stride + split) * 2 + 1], lsum);
       }
     }
   }
-  if (a.n_splits == 1 || !a.fused_merge) return;
+  if (n_valid == 1 || !a.fused_merge) return;
 
   // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
-  const int n_valid = (len + chunk - 1) / chunk;  // splits that run for this sequence
   __shared__ int s_last;
   __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
   if (tid == 0) {
-    unsigned int *ticket = &g_tickets[b * gridDim.y + hg];
+    unsigned int *ticket = &g_tickets[b * a.n_hg + hg];
     const unsigned int t = atomicAdd(ticket, 1u);
     s_last = (t == static_cast<unsigned int>(n_valid - 1));
     if (s_last) atomicExch(ticket, 0u);  // ready for the next launch
@@ -472,15 +559,35 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   for (int o = tid; o < G * D; o += kThreads) {
     const int g = o / D, d = o % D;
     const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
-    const float *ml = a.part_ml + bh * a.n_splits * 2;
-    const float *pa = a.part_acc + bh * a.n_splits * D + d;
-    float mx = kNegBig;
-    for (int s = 0; s < n_valid; ++s) mx = fmaxf(mx, ld_agent(ml + 2 * s));
-    float lsum = 0.0f, asum = 0.0f;
-    for (int s = 0; s < n_valid; ++s) {
-      const float w = __builtin_amdgcn_exp2f(ld_agent(ml + 2 * s) - mx);
-      lsum = __builtin_fmaf(ld_agent(ml + 2 * s + 1), w, lsum);
-      asum = __builtin_fmaf(ld_agent(pa + static_cast<int64_t>(s) * D), w, asum);
+    const float *ml = a.part_ml + bh * a.split_stride * 2;
+    const float *pa = a.part_acc + bh * a.split_stride * D + d;
+    // eight ranges at a time, every load of a batch in flight before the first is used (the loads
+    // go past the local caches: one at a time they would cost a memory round trip each)
+    float mx = kNegBig, lsum = 0.0f, asum = 0.0f;
+    for (int s0m = 0; s0m < n_valid; s0m += 8) {
+      float pm[8], pl[8], pv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int sidx = min(s0m + i, n_valid - 1);
+        pm[i] = ld_agent(ml + 2 * sidx);
+        pl[i] = ld_agent(ml + 2 * sidx + 1);
+        pv[i] = ld_agent(pa + static_cast<int64_t>(sidx) * D);
+      }
+      float bm = mx;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (s0m + i < n_valid) bm = fmaxf(bm, pm[i]);
+      const float keep = __builtin_amdgcn_exp2f(mx - bm);
+      lsum *= keep;
+      asum *= keep;
+      mx = bm;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (s0m + i >= n_valid) continue;
+        const float w = __builtin_amdgcn_exp2f(pm[i] - mx);
+        lsum = __builtin_fmaf(pl[i], w, lsum);
+        asum = __builtin_fmaf(pv[i], w, asum);
+      }
     }
     stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
   }
@@ -499,8 +606,8 @@ __global__ __launch_bounds__(D) void gqa_decode_merge_kernel(DecodeArgs a) {
     stf(out, 0.0f);
     return;
   }
-  const float *ml = a.part_ml + bh * a.n_splits * 2;
-  const float *pa = a.part_acc + bh * a.n_splits * D + d;
+  const float *ml = a.part_ml + bh * a.split_stride * 2;
+  const float *pa = a.part_acc + bh * a.split_stride * D + d;
   float mx = kNegBig;
   for (int s = 0; s < n_valid; ++s) mx = fmaxf(mx, ml[2 * s]);
   float lsum = 0.0f, asum = 0.0f;
@@ -515,7 +622,8 @@ __global__ __launch_bounds__(D) void gqa_decode_merge_kernel(DecodeArgs a) {
 template <typename T, int D, int G>
 int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   constexpr int U = (sizeof(T) == 2 ? 8 : 4) / (G >= 4 ? 2 : 1);
-  const dim3 grid(a.n_splits, a.Hq / G, B);
+  // static plan: (split, head group, sequence); length-dealt plan: one dimension, slot index slowest
+  const dim3 grid(a.dynamic ? a.active * (a.Hq / G) : a.n_splits, a.dynamic ? 1 : a.Hq / G, a.dynamic ? 1 : B);
   if (a.len_add)
     hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, true>), grid, dim3(kThreads), 0, st, a);
   else
@@ -564,13 +672,21 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
   a.max_len = max_len;
   a.chunk = plan.chunk;
   a.n_splits = plan.n_splits;
+  a.dynamic = plan.dynamic;
+  a.active = plan.active;
+  a.split_stride = plan.stride;
+  a.B = B;
+  a.n_hg = Hq / G;
   a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
   a.part_acc = nullptr;
   a.part_ml = nullptr;
-  a.fused_merge = (!g_tuning.separate_merge && static_cast<long>(B) * (Hq / G) <= kTicketSlots) ? 1 : 0;
-  if (plan.n_splits > 1) {
-    const size_t acc_elems = static_cast<size_t>(B) * Hq * plan.n_splits * D;
-    const size_t need = (acc_elems + static_cast<size_t>(B) * Hq * plan.n_splits * 2) * sizeof(float);
+  // the length-dealt plan always merges in the kernel (a second kernel could not be skipped when no
+  // sequence needs it); the static plan does unless the two-kernel form was asked for
+  a.fused_merge = ((plan.dynamic || !g_tuning.separate_merge) && static_cast<long>(B) * (Hq / G) <= kTicketSlots) ? 1 : 0;
+  if (plan.dynamic && !a.fused_merge) return AXHIP_INTERNAL_ERROR;  // B <= 64: the ticket slots always suffice
+  if (plan.stride > 1) {
+    const size_t acc_elems = static_cast<size_t>(B) * Hq * plan.stride * D;
+    const size_t need = (acc_elems + static_cast<size_t>(B) * Hq * plan.stride * 2) * sizeof(float);
     if (!workspace || workspace_bytes < need) return AXHIP_INVALID_ARGUMENT;
     a.part_acc = static_cast<float *>(workspace);
     a.part_ml = a.part_acc + acc_elems;
@@ -584,9 +700,8 @@ extern "C" {
 
 // Measurement hook: overrides the split heuristics (0 restores the default).
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits) {
-  // a negative target selects the single-launch form (the last workgroup merges); measured no
-  // faster than the second kernel (ticket + write-through latency at the tail), so not the default
-  g_tuning.separate_merge = target_workgroups < 0 ? 0 : 1;
+  // a negative target selects the two-kernel form for a forced split count (split kernel + merge kernel)
+  g_tuning.separate_merge = target_workgroups < 0 ? 1 : 0;
   g_tuning.target_workgroups = target_workgroups > 0 ? target_workgroups : Tuning().target_workgroups;
   g_tuning.force_splits = force_splits > 0 ? force_splits : 0;
 }

@@ -103,14 +103,15 @@ def main(argv=None):
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--gqa-single-launch", action="store_true",
-                    help="attention merges its splits in the last workgroup instead of a second kernel")
+    ap.add_argument("--gqa-two-kernels", type=int, default=0, metavar="SPLITS",
+                    help="attention with a fixed split count and a second merge kernel (the default deals "
+                         "workgroups by length and merges in the last workgroup)")
     ap.add_argument("--fused-tail", action="store_true",
                     help="each layer's post-attention part as one persistent launch (measured slower; off by default)")
     args = ap.parse_args(argv)
-    if args.gqa_single_launch:
+    if args.gqa_two_kernels:
         from .. import _lib
-        _lib.load().axhip_gqa_decode_tune(-1, 0)
+        _lib.load().axhip_gqa_decode_tune(-1, args.gqa_two_kernels)
     res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
               fused_tail=args.fused_tail)
     print(json.dumps(res), flush=True)

@@ -173,11 +173,14 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
                                int max_len, int64_t stride_b, int64_t stride_h, int64_t stride_s,
                                axhip_stream stream);
 
-/* The split plan the launcher uses for these sizes (it depends on host-side sizes only), and a
- * measurement hook that overrides the heuristics: target_workgroups = resident workgroups to aim
- * for (a negative value selects the single-launch form in which the last workgroup merges the
- * splits), force_splits > 0 fixes the split count; 0 restores a default.  No reference counterpart
- * (the reference hard-codes min(256, ceil(L/64)), gqa.cu:158-160). */
+/* The split plan the launcher uses for these sizes (it depends on host-side sizes only).  For batches of
+ * up to 64 sequences the launch holds a fixed number of workgroups which are dealt to the sequences on the
+ * device in proportion to their current lengths (n_splits = workgroup slots per sequence, chunk = keys per
+ * workgroup if every sequence had max_len keys), and the last workgroup of a sequence merges its ranges.
+ * Measurement hook: target_workgroups = workgroups to keep streaming (default 256, one per CU; a negative
+ * value selects a second merge kernel for a forced split count), force_splits > 0 cuts every sequence into
+ * that many ranges; 0 restores the defaults.  No reference counterpart (the reference hard-codes
+ * min(256, ceil(L/64)), gqa.cu:158-160). */
 AXHIP_API void axhip_gqa_decode_plan(int B, int Hq, int Hkv, int max_len, int *n_splits, int *chunk);
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
 

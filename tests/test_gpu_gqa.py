@@ -144,8 +144,10 @@ def test_error_codes():
 
 
 def test_two_kernel_merge_mode_matches_fused_merge():
-    """The merge done by the last workgroup and the merge done by a second kernel give the same
-    result (both against the oracle), also with empty and single-split sequences in the batch."""
+    """The default plan (workgroups dealt to the sequences by length, merge by the last workgroup of
+    a sequence), a fixed split count with the same in-kernel merge, and a fixed split count with a
+    second merge kernel give the same result (all against the oracle), also with empty, one-key and
+    single-range sequences in the batch."""
     rng = np.random.default_rng(15)
     B, Lmax = 6, 3000
     lens = np.array([3000, 0, 1, 257, 1500, 2999], np.int32)
@@ -153,16 +155,20 @@ def test_two_kernel_merge_mode_matches_fused_merge():
     k = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
     v = rng.standard_normal((B, 8, Lmax, 128)).astype(np.float32).astype(np.float16)
     want = port.gqa_decode_cache_native(q, k, v, lens)
-    two = gqa_decode(q, k, v, lens).astype(np.float32)       # default: split kernel + merge kernel
-    lib().axhip_gqa_decode_tune(-1, 0)                         # single launch, last workgroup merges
-    fused = gqa_decode(q, k, v, lens).astype(np.float32)
-    # repeated launches reuse the ticket counters: run the single-launch form several times
+    fused = gqa_decode(q, k, v, lens).astype(np.float32)      # default
+    # repeated launches reuse the ticket counters
     for _ in range(3):
         again = gqa_decode(q, k, v, lens).astype(np.float32)
         np.testing.assert_array_equal(again, fused)
+    lib().axhip_gqa_decode_tune(0, 5)                          # 5 ranges per sequence, in-kernel merge
+    fixed = gqa_decode(q, k, v, lens).astype(np.float32)
+    lib().axhip_gqa_decode_tune(-1, 5)                         # 5 ranges per sequence, split kernel + merge kernel
+    two = gqa_decode(q, k, v, lens).astype(np.float32)
     lib().axhip_gqa_decode_tune(0, 0)
-    assert np.abs(fused - want).max() <= TOL16 and np.abs(two - want).max() <= TOL16
-    assert np.all(fused[1] == 0) and np.all(two[1] == 0)
+    for o in (fused, fixed, two):
+        assert np.abs(o - want).max() <= TOL16
+        assert np.all(o[1] == 0)
+    np.testing.assert_array_equal(fixed, two)                  # same ranges, same merge arithmetic
     # a single split and an empty sequence (the split-0 workgroup writes the zeros)
     lib().axhip_gqa_decode_tune(0, 1)
     one = gqa_decode(q, k, v, lens).astype(np.float32)
@@ -275,3 +281,20 @@ def test_prefill_attention_matches_causal_oracle(Hq, Hkv, D, S, start):
     l = gu.lib()
     assert l.axhip_prefill_attention(dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F32, B, S, Hq, Hkv, D, rows, None) == 3
     assert l.axhip_prefill_attention(dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F16, B, S, Hq, Hkv, 256, rows, None) == 1
+
+
+def test_workgroups_are_dealt_by_length():
+    """Very uneven batches under the default plan: one long sequence among short ones, all equal,
+    and lengths that leave some of the launch's workgroup slots unused."""
+    rng = np.random.default_rng(33)
+    hq, hkv, d, Lmax = 4, 2, 128, 6000
+    for lens in ([6000, 17, 130, 1, 0, 900, 64, 3], [2048] * 5, [1] * 7, [6000] * 2, [0, 0, 5999]):
+        lens = np.asarray(lens, np.int32)
+        B = len(lens)
+        q = rng.standard_normal((B, hq, d)).astype(np.float32).astype(np.float16)
+        k = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
+        v = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
+        out = gqa_decode(q, k, v, lens).astype(np.float32)
+        want = port.gqa_decode_cache_native(q, k, v, lens)
+        assert np.abs(out - want).max() <= TOL16, lens
+        assert np.all(out[lens == 0] == 0)

@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the headline split kernel, from the rocprofv3 --pmc runs recorded in
 # profiles/gqa_decode_split_B32_L8192_f16.md (a measured constant, not computed in this process)
-MEASURED_TRAFFIC_BYTES = 1075559905
+MEASURED_TRAFFIC_BYTES = 1074176614
 
 F16 = 4
 
@@ -291,7 +291,7 @@ def main():
         # (FETCH_SIZE x 2.0000 + WRITE_SIZE x 1.0000, factors from a 1 GiB copy kernel), see profiles/
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "gqa_decode_split_kernel<__half,128,2,8> (+ gqa_decode_merge_kernel)",
+                     "kernel": "gqa_decode_split_kernel<__half,128,2,8> (one range per sequence at this shape: no merge)",
                      "avg_launch_us": round(ev_ms * 1e3, 2), "algorithmic_bytes": wl.bytes_per_step},
     }
     del wl

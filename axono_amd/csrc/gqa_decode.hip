@@ -223,17 +223,6 @@ __device__ __forceinline__ int clamped_len(const int32_t *seq_lens, int b, int m
   return len > max_len ? max_len : len;
 }
 
-// Which (sequence, split, head group) a workgroup works on, and how many splits that sequence has.
-// Static plan: straight from the grid.  Dynamic plan: workgroup id = slot * n_hg + head group; the
-// `active` slots of a head group are dealt by length - with c keys per workgroup, sequence b takes
-// max(1, ceil(len_b / c)) consecutive slots (the workgroup of an empty sequence writes zeros), and c
-// starts at ceil(sum of lengths / active) and grows until the slots suffice (a few rounds: the count
-// falls as c grows, and c = max_len needs B <= active slots).  Slots left over exit at once.  Every
-// wavefront builds the table in its registers: lane i holds sequence i (B <= 64), one vector load
-// for the lengths, wave sums, a wave prefix sum, one ballot.
-struct Work {
-  int b, k, n, hg;
-};
 __device__ __forceinline__ int dyn_splits_of(int len, int c, int stride) {
   const int n = len > 0 ? (len + c - 1) / c : 1;
   return n < stride ? n : stride;
@@ -243,41 +232,20 @@ __device__ __forceinline__ int wave_sum_i(int v) {
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
   return v;
 }
-__device__ __forceinline__ Work map_work(const DecodeArgs &a) {
-  if (!a.dynamic)
-    return Work{static_cast<int>(blockIdx.z), static_cast<int>(blockIdx.x), a.n_splits, static_cast<int>(blockIdx.y)};
-  const int lane = threadIdx.x & 63;
-  const int j = static_cast<int>(blockIdx.x) / a.n_hg, hg = static_cast<int>(blockIdx.x) % a.n_hg;
-  const bool live = lane < a.B;
-  const int len = live ? clamped_len(a.seq_lens, lane, a.max_len, a.len_add) : 0;
-  // sum of lengths in units of 64 keys (rounded up per sequence): fits an int for any supported size
-  const int total64 = wave_sum_i((len + 63) >> 6);
-  long long c64 = (static_cast<long long>(total64) * 64 + a.active - 1) / a.active;
-  int c = static_cast<int>(c64 < kMinDevChunk ? kMinDevChunk : (c64 > a.max_len ? a.max_len : c64));
-  int n = 0;
-#pragma unroll 1
-  for (int round = 0; round < 8; ++round) {
-    n = live ? dyn_splits_of(len, c, a.split_stride) : 0;
-    const int used = wave_sum_i(n);
-    if (used <= a.active) break;
-    // too many slots: grow c by the overshoot (at least one key), the last round takes one range each
-    const long long grown = (static_cast<long long>(c) * used + a.active - 1) / a.active;
-    c = round == 6 ? a.max_len : static_cast<int>(grown > a.max_len ? a.max_len : (grown > c ? grown : c + 1));
-  }
-  int incl = n;
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_prefix_i(int v, int lane) {  // inclusive prefix sum over the lanes
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
-    const int up = __shfl_up(incl, off, 64);
-    if (lane >= off) incl += up;
+    const int up = __shfl_up(v, off, 64);
+    if (lane >= off) v += up;
   }
-  const int first = incl - n;
-  const unsigned long long hit = __ballot(j >= first && j < first + n);
-  if (hit == 0ull) return Work{-1, 0, 0, hg};
-  const int b = __ffsll(hit) - 1;
-  // the same in every lane: say so, so that everything derived from it lives in scalar registers
-  return Work{__builtin_amdgcn_readfirstlane(b), __builtin_amdgcn_readfirstlane(j - __shfl(first, b, 64)),
-              __builtin_amdgcn_readfirstlane(__shfl(n, b, 64)), hg};
+  return v;
 }
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // One head row of the qkv projection -> RMSNorm over the head (weights optional) -> interleaved
 // M-RoPE at this sequence's (t, h, w) position, in the evaluation order of the single operators
@@ -387,29 +355,28 @@ __device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t st
   tile_update<T, D, G, U, CHECK>(kr, vr, base, rg, s1, scale_log2e, qf, m, l, acc);
 }
 
-template <typename T, int D, int G, int U, bool QKV>
-__global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArgs a) {
+// A sequence without keys: its output rows are zeros.
+template <typename T, int D, int G>
+__device__ __forceinline__ void write_zero_rows(const DecodeArgs &a, int b, int hg) {
+  for (int o = threadIdx.x; o < G * D; o += kThreads)
+    stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + hg * G) * D + o, 0.0f);
+}
+
+// Keys [s0, s1) of sequence b for the G query heads of head group hg: range number `split` of the
+// `n_valid` non-empty ranges this sequence is cut into in this launch.  The only range of a sequence
+// writes the result itself when `direct_ok`; otherwise the range leaves a partial state and (fused
+// merge) the workgroup that finishes last combines them.  A workgroup may call this several times:
+// the caller puts a barrier between two calls, because the LDS arrays are the same.
+template <typename T, int D, int G, int U, bool QKV, bool HOIST>
+__device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg, int split, int n_valid,
+                                              bool direct_ok, int s0, int s1) {
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
-  const Work wk = map_work(a);
-  if (wk.b < 0) return;  // a slot the lengths of this launch leave unused
-  const int split = wk.k, hg = wk.hg, b = wk.b;
-  const int len = clamped_len(a.seq_lens, b, a.max_len, a.len_add);
-  const int chunk = balanced_chunk(len, wk.n);
-  const int n_valid = (len + chunk - 1) / chunk;  // splits of this sequence that hold keys
-  const int s0 = split * chunk;
-  const int tid = threadIdx.x;
+  int tid = threadIdx.x;
+  // opaque inside a caller's loop over pieces, so that nothing derived from it is computed ahead of
+  // the loop and held in registers across the whole piece
+  if constexpr (!HOIST) asm volatile("" : "+v"(tid));
   const int h0 = hg * G;            // first query head of this workgroup
-  if (s0 >= len) {
-    // An empty split is never read by the merge.  A sequence without keys gets zeros, written by
-    // its split-0 workgroup when no separate merge kernel will do it.
-    if (len == 0 && split == 0 && (wk.n == 1 || a.fused_merge)) {
-      for (int o = tid; o < G * D; o += kThreads)
-        stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + h0) * D + o, 0.0f);
-    }
-    return;
-  }
-  const int s1 = min(s0 + chunk, len);
 
   const int rg = tid / LPR, dl = tid % LPR;
   const int hk = h0 / a.group;      // the kv head those G query heads share
@@ -427,14 +394,14 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   __shared__ __attribute__((aligned(16))) T s_kv[2][QKV ? D : 8];
   bool mine = false;
   int kv_end = s1;  // keys [s0, kv_end) come from the cache
-  Frag8<T> kr0[QKV ? U : 1], vr0[QKV ? U : 1];
+  Frag8<T> kr0[QKV && HOIST ? U : 1], vr0[QKV && HOIST ? U : 1];
   if constexpr (QKV) {
     int p_new = a.seq_lens[b];
     p_new = p_new < 0 ? 0 : p_new;
     mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
     if (mine) kv_end = p_new;
     // the first tile of cached keys is requested before q is prepared: those loads do not need it
-    tile_load<T, D, U, true>(kb, vb, a.stride_s, s0, rg, kv_end, kr0, vr0);
+    if constexpr (HOIST) tile_load<T, D, U, true>(kb, vb, a.stride_s, s0, rg, kv_end, kr0, vr0);
     const int wave = tid >> 6, lane = tid & 63;
     const int B = a.B;
     const bool writer = mine && (h0 % a.group == 0);
@@ -476,7 +443,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
   }
 
   int base = s0;
-  if constexpr (QKV) {
+  if constexpr (QKV && HOIST) {
     tile_update<T, D, G, U, true>(kr0, vr0, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
     base += U * RG;
   }
@@ -532,7 +499,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
       asum = __builtin_fmaf(s_acc[g][r][d], w, asum);
     }
     const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
-    if (n_valid == 1 && (wk.n == 1 || a.fused_merge)) {
+    if (n_valid == 1 && direct_ok) {
       // the only range of this sequence: normalise and write the result, nothing to merge
       stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
     } else {
@@ -591,6 +558,116 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
     }
     stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
   }
+}
+
+// Which keys a workgroup streams.
+//   Static plan: (range, head group, sequence) straight from the grid.
+//   Length-dealt plan: workgroup id = slot * n_hg + head group, and the `active` slots of a head group
+//   share the keys of the whole batch.  Every wavefront builds the table in its registers - lane i
+//   holds sequence i (B <= 64): one vector load for the lengths, wave sums, a prefix sum, a ballot.
+//   (1) Whole slots per sequence: with c keys per slot, sequence b takes max(1, ceil(len_b / c))
+//       consecutive slots and is cut into that many equal ranges; c starts at
+//       ceil(sum of lengths / active) and grows until the slots suffice (a few rounds: the count falls
+//       as c grows, and c = max_len needs B <= active slots).  Slots left over exit at once.  A batch
+//       of (nearly) equal lengths is cut exactly evenly this way, with one range per workgroup.
+//   (2) When whole slots leave the longest range more than an eighth (and 256 keys) above the
+//       average - a ragged batch, or fewer slots than it takes to follow the lengths - the sequences
+//       are laid end to end instead and slot j takes keys [j*c, (j+1)*c) of that line, whichever
+//       sequences they belong to: a workgroup then works through a piece of each sequence its range
+//       touches, and every slot streams the same number of keys.  A sequence without keys gets its
+//       zeros from the slot that holds its place on the line.
+template <typename T, int D, int G, int U, bool QKV>
+__global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArgs a) {
+  // the piece to work on: keys [s0, s1) of sequence b, range `split` of its n_valid ranges
+  int b, hg, split, n_valid, s0, s1;
+  bool direct_ok = true;
+  if (!a.dynamic) {
+    split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
+    const int len_b = clamped_len(a.seq_lens, b, a.max_len, a.len_add);
+    const int chunk = balanced_chunk(len_b, a.n_splits);
+    n_valid = (len_b + chunk - 1) / chunk;  // ranges of this sequence that hold keys
+    direct_ok = a.n_splits == 1 || a.fused_merge;
+    s0 = split * chunk;
+    s1 = min(s0 + chunk, len_b);
+    if (s0 >= len_b) {
+      // an empty range is never read by the merge; without a merge kernel the zeros of a sequence
+      // without keys come from its first workgroup
+      if (len_b == 0 && split == 0 && direct_ok) write_zero_rows<T, D, G>(a, b, hg);
+      return;
+    }
+  } else {
+    const int lane = threadIdx.x & 63;
+    const int j = static_cast<int>(blockIdx.x) / a.n_hg;
+    hg = static_cast<int>(blockIdx.x) % a.n_hg;
+    const bool live = lane < a.B;
+    const int len = live ? clamped_len(a.seq_lens, lane, a.max_len, a.len_add) : 0;
+    // sum of lengths in units of 64 keys (rounded up per sequence): fits an int for any supported size
+    const int total64 = wave_sum_i((len + 63) >> 6);
+    const long long c_even = (static_cast<long long>(total64) * 64 + a.active - 1) / a.active;
+    int c = static_cast<int>(c_even < kMinDevChunk ? kMinDevChunk : (c_even > a.max_len ? a.max_len : c_even));
+    int n = 0;
+#pragma unroll 1
+    for (int round = 0; round < 8; ++round) {
+      n = live ? dyn_splits_of(len, c, a.split_stride) : 0;
+      const int used = wave_sum_i(n);
+      if (used <= a.active) break;
+      // too many slots: grow c by the overshoot (at least one key), the last round takes one range each
+      const long long grown = (static_cast<long long>(c) * used + a.active - 1) / a.active;
+      c = round == 6 ? a.max_len : static_cast<int>(grown > a.max_len ? a.max_len : (grown > c ? grown : c + 1));
+    }
+    const int longest = wave_max_i(live && len > 0 ? balanced_chunk(len, n) : 0);
+    const long long slack = c_even / 8 > 256 ? c_even / 8 : 256;
+    // a slot can leave at most one piece per sequence, so `active` partial slots per sequence suffice
+    const bool end_to_end = a.active <= a.split_stride && total64 < (1 << 24) && longest - c_even > slack;
+    if (end_to_end) {
+      const int start = wave_prefix_i(len, lane) - len;  // where this lane's sequence begins on the line
+      const int total = uni(__shfl(start + len, 63, 64));
+      int cc = (total + a.active - 1) / a.active;
+      cc = cc < kMinDevChunk ? kMinDevChunk : cc;
+      cc = (cc + 15) & ~15;
+      const int g0 = j * cc, g1 = min(g0 + cc, total);
+      unsigned long long todo = __ballot(live && len > 0 && start < g1 && start + len > g0);
+      // the place of an empty sequence belongs to the slot of the key before it (slot 0 at the start)
+      unsigned long long empty = __ballot(live && len == 0 && (start > 0 ? (start - 1) / cc : 0) == j);
+      for (bool again = false; todo; again = true) {
+        b = uni(__ffsll(todo) - 1);
+        todo &= todo - 1;
+        // start and length of sequence b, from memory again: held in vector registers across the
+        // piece they would push the streaming loop over its register budget
+        const int lane2 = threadIdx.x & 63;
+        const int before = lane2 < b ? clamped_len(a.seq_lens, lane2, a.max_len, a.len_add) : 0;
+        const int start_b = uni(wave_sum_i(before));
+        const int len_b = clamped_len(a.seq_lens, b, a.max_len, a.len_add);
+        const int first_slot = start_b / cc, last_slot = (start_b + len_b - 1) / cc;
+        if (again) __syncthreads();  // the previous piece is done with the LDS arrays
+        process_range<T, D, G, U, QKV, false>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
+                                       max(g0 - start_b, 0), min(g1 - start_b, len_b));
+      }
+      while (empty) {
+        const int e = uni(__ffsll(empty) - 1);
+        empty &= empty - 1;
+        write_zero_rows<T, D, G>(a, e, hg);
+      }
+      return;
+    }
+    const int first = wave_prefix_i(n, lane) - n;
+    const unsigned long long hit = __ballot(j >= first && j < first + n);
+    if (hit == 0ull) return;  // a slot the lengths of this launch leave unused
+    // the same in every lane: say so, so that everything derived from it lives in scalar registers
+    b = uni(__ffsll(hit) - 1);
+    split = uni(j - __shfl(first, b, 64));
+    const int n_b = uni(__shfl(n, b, 64));
+    const int len_b = uni(__shfl(len, b, 64));
+    const int chunk = balanced_chunk(len_b, n_b);
+    n_valid = (len_b + chunk - 1) / chunk;
+    s0 = split * chunk;
+    s1 = min(s0 + chunk, len_b);
+    if (s0 >= len_b) {
+      if (len_b == 0 && split == 0) write_zero_rows<T, D, G>(a, b, hg);
+      return;
+    }
+  }
+  process_range<T, D, G, U, QKV, true>(a, b, hg, split, n_valid, direct_ok, s0, s1);
 }
 
 // Cross-split merge: one workgroup of D threads per (sequence, query head).

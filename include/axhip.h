@@ -176,7 +176,9 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
 /* The split plan the launcher uses for these sizes (it depends on host-side sizes only).  For batches of
  * up to 64 sequences the launch holds a fixed number of workgroups which are dealt to the sequences on the
  * device in proportion to their current lengths (n_splits = workgroup slots per sequence, chunk = keys per
- * workgroup if every sequence had max_len keys), and the last workgroup of a sequence merges its ranges.
+ * workgroup if every sequence had max_len keys): whole workgroups per sequence when that is within an eighth
+ * of the even share, otherwise equal runs of keys over the sequences laid end to end; the last workgroup of
+ * a sequence merges its ranges.
  * Measurement hook: target_workgroups = workgroups to keep streaming (default 256, one per CU; a negative
  * value selects a second merge kernel for a forced split count), force_splits > 0 cuts every sequence into
  * that many ranges; 0 restores the defaults.  No reference counterpart (the reference hard-codes

@@ -176,14 +176,9 @@ def test_two_kernel_merge_mode_matches_fused_merge():
     assert np.abs(one - want).max() <= TOL16 and np.all(one[1] == 0)
 
 
-@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (8, 1, 64), (3, 3, 256)])
-def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
-    """axhip_gqa_decode_qkv (q/k norm + M-RoPE + append + attention in the split kernel) against the
-    oracle's rms_norm -> rope_thd -> fp16 rounding -> append -> attention over len + 1 keys; sequences
-    that put the new row in the first split, in the last split, and alone in a split of its own."""
-    rng = np.random.default_rng(77)
-    rows, max_len = 1300, 1280
-    lens = np.array([0, 5, 255, 256, 700, 1279, 1280], np.int32)   # 1280: cache bound reached, nothing appended
+def _check_decode_step_form(Hq, Hkv, D, lens, rows, max_len, forced=(0, 5), seed=77):
+    rng = np.random.default_rng(seed)
+    lens = np.asarray(lens, np.int32)
     B = len(lens)
     width = (Hq + 2 * Hkv) * D
     qkv = rng.standard_normal((B, width)).astype(np.float32)
@@ -198,7 +193,7 @@ def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
     l = gu.lib()
     dq, dqw, dkw, dp, di, dl, dkc, dvc = (gu.dev(a) for a in (qkv, qw, kw, pos, inv, lens, kc, vc))
     out = gu.DeviceBuffer(B * Hq * D * 2)
-    for force_splits in (0, 5):
+    for force_splits in forced:
         l.axhip_gqa_decode_tune(0, force_splits)
         dkc.upload(kc.reshape(-1))
         dvc.upload(vc.reshape(-1))
@@ -232,12 +227,38 @@ def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
         got = out.download(np.float16, (B, Hq, D)).astype(np.float32)
         assert np.abs(got - want).max() <= 2e-3, (force_splits, np.abs(got - want).max())
     l.axhip_gqa_decode_tune(0, 0)
+    return dq, dp, di, dl, dkc, dvc, out, ws, wsb, width, hw
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (8, 1, 64), (3, 3, 256)])
+def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
+    """axhip_gqa_decode_qkv (q/k norm + M-RoPE + append + attention in the split kernel) against the
+    oracle's rms_norm -> rope_thd -> fp16 rounding -> append -> attention over len + 1 keys; sequences
+    that put the new row in the first split, in the last split, and alone in a split of its own."""
+    rows, max_len = 1300, 1280
+    lens = [0, 5, 255, 256, 700, 1279, 1280]   # 1280: cache bound reached, nothing appended
+    B = len(lens)
+    dq, dp, di, dl, dkc, dvc, out, ws, wsb, width, hw = _check_decode_step_form(Hq, Hkv, D, lens, rows, max_len)
+    l = gu.lib()
     # argument checks: seq_lens is required; max_len may not exceed the cache
     args = [dq.ptr, width, dq.ptr, width, dq.ptr, width, None, None, gu.F32, 1e-6, dp.ptr, di.ptr, hw, hw]
     assert l.axhip_gqa_decode_qkv(*args, None, dkc.ptr, dvc.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows,
                                   max_len, None) == 7
     assert l.axhip_gqa_decode_qkv(*args, dl.ptr, dkc.ptr, dvc.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows,
                                   rows + 1, None) == 1
+
+
+def test_decode_step_form_ragged_batch_with_one_workgroup_per_sequence_to_share():
+    """As many sequences as the launch has workgroups per head group, of very different lengths:
+    the workgroups then share the keys of the whole batch end to end, each working through pieces of
+    several sequences, and the new token's row may be a piece of its own."""
+    rng = np.random.default_rng(5)
+    max_len = 2400
+    lens = rng.integers(0, max_len, 32)
+    lens[[0, 7, 31]] = 0
+    lens[[1, 8]] = [max_len, max_len - 1]
+    lens[[2, 3]] = [1, 127]
+    _check_decode_step_form(16, 8, 128, lens, max_len + 8, max_len, forced=(0,), seed=6)
 
 
 @pytest.mark.parametrize("Hq,Hkv,D,S,start", [(4, 2, 128, 200, [0, 37]), (2, 2, 128, 64, [0, 0]), (8, 2, 64, 130, [5, 300]),
@@ -291,6 +312,22 @@ def test_workgroups_are_dealt_by_length():
     for lens in ([6000, 17, 130, 1, 0, 900, 64, 3], [2048] * 5, [1] * 7, [6000] * 2, [0, 0, 5999]):
         lens = np.asarray(lens, np.int32)
         B = len(lens)
+        q = rng.standard_normal((B, hq, d)).astype(np.float32).astype(np.float16)
+        k = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
+        v = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
+        out = gqa_decode(q, k, v, lens).astype(np.float32)
+        want = port.gqa_decode_cache_native(q, k, v, lens)
+        assert np.abs(out - want).max() <= TOL16, lens
+        assert np.all(out[lens == 0] == 0)
+    # 32 workgroups per head group for up to 32 sequences: uneven lengths make the workgroups share the
+    # keys of the batch end to end (a workgroup then works through pieces of several sequences); empty
+    # sequences at the start, in the middle and at the end of the batch, and single keys
+    hq, hkv, Lmax = 16, 8, 3000
+    for B in (32, 9):
+        lens = rng.integers(1, Lmax + 1, B).astype(np.int32)
+        lens[[0, 4, B - 1]] = 0
+        lens[[1, 5]] = 1
+        lens[2] = Lmax
         q = rng.standard_normal((B, hq, d)).astype(np.float32).astype(np.float16)
         k = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
         v = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)

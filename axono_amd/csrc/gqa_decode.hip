@@ -14,10 +14,10 @@
 // products with fp32 accumulation); the matrix cores would add nothing.
 //
 // Scores are kept in the log2 domain (q.k * scale * log2 e) so that the exponentials are single
-// v_exp_f32 instructions.  Per-split results (unnormalised output, running max, running sum) go to
-// a workspace and a second small kernel merges them; with one split the first kernel normalises
-// and writes the result itself.  (A single-launch form, in which the workgroup that takes the last
-// ticket of a (sequence, head group) merges, is kept behind the tuning hook: it measured no faster.)
+// v_exp_f32 instructions.  A sequence that is one key range is normalised and written by its
+// workgroup.  Otherwise the per-range results (unnormalised output, running max, running sum) go to
+// a workspace, and the workgroup that takes the last ticket of a (sequence, head group) merges them
+// in the same launch; a second small merge kernel is kept behind the tuning hook for comparison.
 #include "common.hpp"
 
 namespace axhip {

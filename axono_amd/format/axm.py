@@ -34,24 +34,37 @@ def _pad(n: int) -> int:
     return -n % _ALIGN
 
 
-def save_axm(state_dict: dict, path: str, meta: dict | None = None, dtype=None) -> None:
-    """Writes {name: ndarray} to `path`.  `dtype` (e.g. "float16") converts every tensor; None keeps
-    each array's dtype.  `meta` is stored verbatim in the index.  (Reference: axm.py:50-109.)"""
-    arrays, tensors, cursor = [], [], 0
-    for name, value in state_dict.items():
-        a = np.ascontiguousarray(value) if dtype is None else np.ascontiguousarray(value, dtype=dtype)
-        tensors.append({"name": name, "dtype": str(a.dtype), "shape": [int(d) for d in a.shape], "offset": cursor,
-                        "size": int(a.nbytes)})
-        arrays.append(a)
-        cursor += a.nbytes + _pad(a.nbytes)
+def write_axm(specs, path: str, meta: dict | None = None) -> None:
+    """Writes an AXM1 file from `specs`, an iterable of (name, numpy dtype, shape, produce) where
+    produce() returns the array: the index is laid out from dtype and shape alone, and the arrays are
+    produced and written one at a time, so a converter never holds more than one tensor."""
+    specs = list(specs)
+    tensors, cursor = [], 0
+    for name, dt, shape, _ in specs:
+        nbytes = int(np.dtype(dt).itemsize * int(np.prod(shape, dtype=np.int64)))
+        tensors.append({"name": name, "dtype": str(np.dtype(dt)), "shape": [int(d) for d in shape], "offset": cursor,
+                        "size": nbytes})
+        cursor += nbytes + _pad(nbytes)
     index = json.dumps({"tensors": tensors, "meta": meta or {}}).encode("utf-8")
     with open(path, "wb") as f:
         f.write(_HEAD.pack(MAGIC, VERSION, 0, len(index)))
         f.write(index)
         f.write(bytes(_pad(_HEAD.size + len(index))))
-        for a in arrays:
+        for (name, dt, shape, produce), t in zip(specs, tensors):
+            a = np.ascontiguousarray(produce(), dtype=dt)
+            if a.nbytes != t["size"] or tuple(a.shape) != tuple(shape):
+                raise ValueError(f"tensor {name}: produced {a.shape} {a.dtype}, announced {tuple(shape)} {np.dtype(dt)}")
             f.write(memoryview(a).cast("B") if a.nbytes else b"")
             f.write(bytes(_pad(a.nbytes)))
+
+
+def save_axm(state_dict: dict, path: str, meta: dict | None = None, dtype=None) -> None:
+    """Writes {name: ndarray} to `path`.  `dtype` (e.g. "float16") converts every tensor; None keeps
+    each array's dtype.  `meta` is stored verbatim in the index.  (Reference: axm.py:50-109.)"""
+    def spec(name, value):
+        a = np.asarray(value)
+        return name, (a.dtype if dtype is None else np.dtype(dtype)), a.shape, lambda: a
+    write_axm((spec(n, v) for n, v in state_dict.items()), path, meta)
 
 
 def read_axm_index(path: str):

@@ -128,3 +128,87 @@ def test_text_model_weights_roundtrip_in_reference_naming(tmp_path):
     for k in w:
         assert back[k].dtype == w[k].dtype, k
         np.testing.assert_array_equal(back[k], w[k])
+
+
+# ---- safetensors -> AXM1 (reference: examples/vlm/qwen3vl/convert.py:32-64) ------------------------
+
+def _write_checkpoint(dirname, tensors, filename="model.safetensors"):
+    from safetensors.torch import save_file
+
+    os.makedirs(dirname, exist_ok=True)
+    save_file(tensors, os.path.join(dirname, filename), metadata={"format": "pt"})
+
+
+def _fake_checkpoint():
+    import torch
+
+    g = torch.Generator().manual_seed(11)
+    return {
+        "model.language_model.embed_tokens.weight": torch.randn(50, 16, generator=g).to(torch.bfloat16),
+        "model.language_model.layers.0.self_attn.q_proj.weight": torch.randn(32, 16, generator=g).to(torch.bfloat16),
+        "model.language_model.norm.weight": torch.ones(16, dtype=torch.float16),
+        "model.visual.patch_embed.proj.weight": torch.randn(8, 3, 2, 4, 4, generator=g),
+        "model.visual.patch_embed.proj.bias": torch.randn(8, generator=g),
+        "model.visual.blocks.0.attn.qkv.weight": torch.tensor([[1e-40, -0.0, 65504.0, 3.3895314e38]]).to(torch.bfloat16),
+        "model.language_model.empty": torch.zeros(0, 4),
+    }
+
+
+def test_convert_safetensors_checkpoint(tmp_path):
+    from axono_amd.format.convert import convert, main
+
+    src = _fake_checkpoint()
+    d = str(tmp_path / "qwen3vl-2b")
+    _write_checkpoint(d, src)
+    out = os.path.join(d, "model.axm")
+    st = convert(d, out, None)
+    assert st["n_tensors"] == len(src) and st["size_gb"] > 0
+    got = load_axm(out)
+    assert set(got) == set(src)
+    for k, v in src.items():
+        want = v.float().numpy()
+        if k.endswith("patch_embed.proj.weight"):
+            want = want.reshape(want.shape[0], -1)       # (out, 3*t*p*p), as the model's Linear wants it
+        assert got[k].dtype == np.float32 and got[k].shape == want.shape, k
+        np.testing.assert_array_equal(got[k].view(np.uint32), want.view(np.uint32), err_msg=k)  # bf16 widening is exact
+    index, _ = read_axm_index(out)
+    assert index["meta"]["source"] == "hf-safetensors" and index["meta"]["model_dir"] == "qwen3vl-2b"
+    assert index["meta"]["dtype"] == "keep" and "converted_at" in index["meta"]
+    # --dtype float16 halves the file; default output path; command line
+    with np.errstate(over="ignore"):  # the largest bf16 value of the fixture is inf in fp16
+        assert main(["--model", d, "--dtype", "float16", "--out", str(tmp_path / "h.axm")]) == 0
+    half = load_axm(str(tmp_path / "h.axm"))
+    k = "model.language_model.layers.0.self_attn.q_proj.weight"
+    np.testing.assert_array_equal(half[k], src[k].float().numpy().astype(np.float16))
+    assert read_axm_index(str(tmp_path / "h.axm"))[0]["meta"]["dtype"] == "float16"
+    os.remove(out)
+    assert main(["--model", d]) == 0 and os.path.exists(out)
+
+
+def test_convert_sharded_checkpoint_and_errors(tmp_path):
+    import json
+
+    from axono_amd.format.convert import convert, read_safetensors_index
+
+    src = _fake_checkpoint()
+    names = sorted(src)
+    d = str(tmp_path / "sharded")
+    parts = {"model-00001-of-00002.safetensors": names[:3], "model-00002-of-00002.safetensors": names[3:]}
+    for fn, ks in parts.items():
+        _write_checkpoint(d, {k: src[k] for k in ks}, fn)
+    with open(os.path.join(d, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": {k: fn for fn, ks in parts.items() for k in ks}}, f)
+    out = str(tmp_path / "s.axm")
+    assert convert(d, out, None)["n_tensors"] == len(src)
+    got = load_axm(out)
+    for k, v in src.items():
+        np.testing.assert_array_equal(got[k].reshape(-1), v.float().numpy().reshape(-1))
+    with pytest.raises(FileNotFoundError):
+        convert(str(tmp_path / "nothing"), out, None)
+    bad = tmp_path / "bad.safetensors"
+    bad.write_bytes(b"\xff" * 16)
+    with pytest.raises(ValueError):
+        read_safetensors_index(str(bad))
+    bad.write_bytes(b"\x01\x02")
+    with pytest.raises(ValueError):
+        read_safetensors_index(str(bad))

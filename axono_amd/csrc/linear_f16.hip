@@ -34,6 +34,7 @@ LinearTuning g_lin;
 
 struct SkinnyPlan {
   int nt, mt, waves, k_per_wave;
+  int half;  // packed weights: a workgroup takes 8 of the 16 rows of its tile (twice the workgroups)
 };
 
 // A workgroup owns NT*16 rows of W and all of K; its wavefronts split K and add their fragments
@@ -60,6 +61,8 @@ SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
   if (p.nt == 4 && waves > 4) waves = 4;   // LDS: the reduction buffer grows with NT * waves
   if (p.nt * p.mt >= 2 && waves > 8) waves = 8;
   p.waves = waves;
+  // with one row tile per workgroup and at most 128 tiles half the CUs would idle: 8 rows per workgroup
+  p.half = (p.nt == 1 && ntiles * ((M + p.mt * 16 - 1) / (p.mt * 16)) <= 128) ? 1 : 0;
   int64_t kpw = (K + waves - 1) / waves;
   p.k_per_wave = static_cast<int>((kpw + 127) / 128 * 128);
   return p;
@@ -375,8 +378,9 @@ struct PackedArgs {
 // converting fp32 to fp16 on the way, and reads the fragments from LDS.  The strip has no padding;
 // the 16-byte unit index is XOR-ed with the row so that the 16 rows of a fragment read fall into
 // 16 different bank groups.
-template <int NT, int MT, int WAVES, int U, typename XT>
+template <int NT, int MT, int WAVES, int U, bool HALF, typename XT>
 __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(PackedArgs a) {
+  static_assert(!HALF || NT == 1, "half tiles come one per workgroup");
   constexpr int ROWS = MT * 16;
   constexpr int UNITS = U * 4;                 // 16-byte units per strip row
   constexpr int STRIP_HALVES = ROWS * U * 32;  // per wavefront
@@ -385,7 +389,12 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
   __shared__ __attribute__((aligned(16))) unsigned char smem[STRIP_BYTES > RED_BYTES ? STRIP_BYTES : RED_BYTES];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
-  const int tile0 = blockIdx.x * NT;
+  // HALF: two workgroups per row tile.  Both run the full 16-row product, with the 8 rows of their half
+  // loaded into both halves of the fragment (lane r and lane r ^ 8 read the same 16 bytes: no extra
+  // memory traffic), and each stores the rows of its half only.
+  const int tile0 = HALF ? blockIdx.x >> 1 : blockIdx.x * NT;
+  const int half = blockIdx.x & 1;
+  const int src_lane = HALF ? ((lane & ~8) | (half << 3)) : lane;
   const int n_tiles = (a.N + 15) / 16;
   const int m_base = blockIdx.y * ROWS;
   const int c_begin = wave * a.chunks_per_wave;
@@ -404,7 +413,7 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     wok[t] = tile0 + t < n_tiles;
-    wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + lane * 8;
+    wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + src_lane * 8;
   }
 
   for (int c = c_begin; c < c_end; c += U) {
@@ -459,6 +468,7 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
   }
   __syncthreads();
   if (wave != 0) return;
+  if (HALF && (g >> 1) != half) return;  // output rows 4g .. 4g+3 of the tile belong to the other workgroup
   LinearArgs o;  // only the fields store_out4 reads
   o.bias = a.bias;
   o.out = a.out;
@@ -511,38 +521,46 @@ constexpr int packed_unroll() {
 }
 
 template <int NT, int MT, int WAVES, typename XT>
-void launch_packed(const PackedArgs &a, hipStream_t st) {
+void launch_packed(const PackedArgs &a, bool half, hipStream_t st) {
   constexpr int U = packed_unroll<NT, MT, WAVES>();
   const int n_tiles = (a.N + 15) / 16;
   const dim3 grid((n_tiles + NT - 1) / NT, (a.M + MT * 16 - 1) / (MT * 16));
-  hipLaunchKernelGGL((linear_skinny_packed_kernel<NT, MT, WAVES, U, XT>), grid, dim3(WAVES * 64), 0, st, a);
+  if constexpr (NT == 1) {
+    if (half && !a.glu) {
+      hipLaunchKernelGGL((linear_skinny_packed_kernel<NT, MT, WAVES, U, true, XT>), dim3(grid.x * 2, grid.y),
+                         dim3(WAVES * 64), 0, st, a);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((linear_skinny_packed_kernel<NT, MT, WAVES, U, false, XT>), grid, dim3(WAVES * 64), 0, st, a);
 }
 
 template <int NT, int MT, typename XT>
-void dispatch_packed_waves(const PackedArgs &a, int waves, hipStream_t st) {
+void dispatch_packed_waves(const PackedArgs &a, int waves, bool half, hipStream_t st) {
   if constexpr (NT * MT == 1) {
-    if (waves >= 16) return launch_packed<NT, MT, 16, XT>(a, st);
+    if (waves >= 16) return launch_packed<NT, MT, 16, XT>(a, half, st);
   }
   if constexpr (NT < 4) {
-    if (waves >= 8) return launch_packed<NT, MT, 8, XT>(a, st);
+    if (waves >= 8) return launch_packed<NT, MT, 8, XT>(a, half, st);
   }
-  launch_packed<NT, MT, 4, XT>(a, st);
+  launch_packed<NT, MT, 4, XT>(a, half, st);
 }
 
 template <typename XT>
 void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
+  const bool half = p.half != 0;
   if (p.mt == 1) {
     if (p.nt == 4)
-      dispatch_packed_waves<4, 1, XT>(a, p.waves, st);
+      dispatch_packed_waves<4, 1, XT>(a, p.waves, half, st);
     else if (p.nt == 2)
-      dispatch_packed_waves<2, 1, XT>(a, p.waves, st);
+      dispatch_packed_waves<2, 1, XT>(a, p.waves, half, st);
     else
-      dispatch_packed_waves<1, 1, XT>(a, p.waves, st);
+      dispatch_packed_waves<1, 1, XT>(a, p.waves, half, st);
   } else {
     if (p.nt == 2)
-      dispatch_packed_waves<2, 2, XT>(a, p.waves, st);
+      dispatch_packed_waves<2, 2, XT>(a, p.waves, half, st);
     else
-      dispatch_packed_waves<1, 2, XT>(a, p.waves, st);
+      dispatch_packed_waves<1, 2, XT>(a, p.waves, half, st);
   }
 }
 

@@ -512,21 +512,55 @@ __device__ __forceinline__ bool better(float ov, int64_t oi, float v, int64_t i)
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restrict__ x,
-                                                              int64_t *__restrict__ out, int64_t cols) {
+                                                              int64_t *__restrict__ out, int64_t cols, int vec_ok) {
   __shared__ float s_val[kBlock / 64];
   __shared__ int64_t s_idx[kBlock / 64];
   __shared__ int s_last;
   const int row = blockIdx.y, part = blockIdx.x;
   const T *xr = x + static_cast<int64_t>(row) * cols;
-  const int64_t per = (cols + kArgmaxParts - 1) / kArgmaxParts;
-  const int64_t c0 = part * per, c1 = c0 + per < cols ? c0 + per : cols;
+  // parts start on multiples of 8 elements, so that a row whose length is a multiple of 8 can be read
+  // with 16-byte loads; the first maximum wins inside a thread as it does across threads
+  const int64_t per = ((cols + kArgmaxParts - 1) / kArgmaxParts + 7) & ~static_cast<int64_t>(7);
+  const int64_t c0 = part * per < cols ? part * per : cols, c1 = c0 + per < cols ? c0 + per : cols;
   float best = -INFINITY;
   int64_t bi = INT64_MAX;
-  for (int64_t c = c0 + threadIdx.x; c < c1; c += kBlock) {
-    const float v = ldf(xr + c);
-    if (v > best || bi == INT64_MAX) {
-      best = v;
-      bi = c;
+  if (vec_ok) {
+    // whole 8-element groups, four per thread in flight
+    const int64_t groups = (c1 - c0) / 8;
+    for (int64_t g0 = 0; g0 < groups; g0 += 4 * kBlock) {
+      float v[4][8];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t g = g0 + u * kBlock + threadIdx.x;
+        Row8<T>::load(xr + c0 + (g < groups ? g : groups - 1) * 8, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t g = g0 + u * kBlock + threadIdx.x;
+        if (g < groups) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (v[u][j] > best || bi == INT64_MAX) {
+              best = v[u][j];
+              bi = c0 + g * 8 + j;
+            }
+        }
+      }
+    }
+    for (int64_t c = c0 + groups * 8 + threadIdx.x; c < c1; c += kBlock) {
+      const float v = ldf(xr + c);
+      if (better(v, c, best, bi)) {
+        best = v;
+        bi = c;
+      }
+    }
+  } else {
+    for (int64_t c = c0 + threadIdx.x; c < c1; c += kBlock) {
+      const float v = ldf(xr + c);
+      if (v > best || bi == INT64_MAX) {
+        best = v;
+        bi = c;
+      }
     }
   }
   for (int off = 32; off > 0; off >>= 1) {
@@ -762,12 +796,13 @@ AXHIP_API int axhip_argmax(const void *x, int64_t *out, int dtype, int64_t rows,
   hipStream_t st = as_stream(stream);
   if (cols >= 16384 && rows <= kArgmaxMaxRows) {
     const dim3 pgrid(kArgmaxParts, static_cast<unsigned>(rows));
+    const int vec_ok = (cols % 8 == 0 && aligned16(x)) ? 1 : 0;  // every part of every row then starts 16-byte aligned
     if (dtype == AXHIP_FLOAT16)
       hipLaunchKernelGGL((argmax_parts_kernel<__half>), pgrid, dim3(kBlock), 0, st,
-                         static_cast<const __half *>(x), out, cols);
+                         static_cast<const __half *>(x), out, cols, vec_ok);
     else
       hipLaunchKernelGGL((argmax_parts_kernel<float>), pgrid, dim3(kBlock), 0, st,
-                         static_cast<const float *>(x), out, cols);
+                         static_cast<const float *>(x), out, cols, vec_ok);
     return launch_status();
   }
   const dim3 grid(static_cast<unsigned>(rows));

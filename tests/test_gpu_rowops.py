@@ -203,6 +203,16 @@ def test_cast_add_embedding_argmax():
     np.testing.assert_array_equal(gu.argmax(lg), port.argmax(lg))
     assert gu.argmax(lg)[3] == 777
     np.testing.assert_array_equal(gu.argmax(h16(lg)), port.argmax(h16(lg).astype(np.float32)))
+    # many ties (values from a small set): the first index wins inside a 16-byte group, inside a thread, across
+    # threads and across the 64 parts of a row; row lengths that are and are not a multiple of 8
+    for cols in (151936, 20000, 16387, 100003):
+        t = rng.integers(0, 5, (5, cols)).astype(np.float32)
+        t[1, -1] = 9.0            # the maximum in the last element
+        t[2, cols // 2 + 3] = 9.0
+        t[2, cols - 2] = 9.0
+        t[3, :] = -np.inf         # nothing compares greater: index 0
+        np.testing.assert_array_equal(gu.argmax(t), port.argmax(t))
+        np.testing.assert_array_equal(gu.argmax(h16(t)), port.argmax(t))
 
 
 def test_sdpa_prefill_and_small_heads():

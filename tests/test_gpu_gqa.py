@@ -135,6 +135,51 @@ def test_invariants_full_size_headline():
     assert np.abs(out[:1] - want0).max() <= TOL16
 
 
+def test_largest_config_periodic_cache():
+    """B=64, L=32768 fp16 (8.6 GB of cache, the largest configuration): every (sequence, kv head) row of
+    the cache repeats a block of 1024 random keys and values, built on the device by doubling copies.
+    Attention over r whole repetitions equals attention over one block (every copy of a key gets the same
+    weight), so the oracle on the 1024-key block checks the full-size launch - with all sequences full
+    (whole workgroups per sequence) and with ragged multiples of the block (the end-to-end cut)."""
+    B, Hq, Hkv, D, L, P = 64, 16, 8, 128, 32768, 1024
+    rng = np.random.default_rng(64)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16)
+    kp = rng.standard_normal((B, Hkv, P, D)).astype(np.float32).astype(np.float16)
+    vp = rng.standard_normal((B, Hkv, P, D)).astype(np.float32).astype(np.float16)
+    l = lib()
+    row_bytes, blk = L * D * 2, P * D * 2
+    bufs = []
+    for host in (kp, vp):
+        big = gu.DeviceBuffer(B * Hkv * row_bytes)
+        for r in range(B * Hkv):
+            base = big.ptr + r * row_bytes
+            gu.check(l.axhip_memcpy_h2d(base, host.reshape(B * Hkv, -1)[r].ctypes.data, blk), "h2d")
+            have = blk
+            while have < row_bytes:
+                gu.check(l.axhip_memcpy_d2d(base + have, base, have), "d2d")
+                have *= 2
+        bufs.append(big)
+    dk, dv = bufs
+    dq = gu.dev(q)
+    out = gu.DeviceBuffer(q.nbytes)
+    wsb = l.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
+    ws = gu.DeviceBuffer(max(wsb, 256))
+    want = port.gqa_decode_cache_native(q, kp, vp, np.full(B, P, np.int32))
+    ragged = (P * rng.integers(1, L // P + 1, B)).astype(np.int32)
+    ragged[:3] = [L, P, 0]
+    for lens in (np.full(B, L, np.int32), ragged):
+        dl = gu.dev(lens)
+        gu.check(l.axhip_gqa_decode(dq.ptr, dk.ptr, dv.ptr, dl.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, L,
+                                    Hkv * L * D, L * D, D, None), "gqa_decode")
+        gu.synchronize()
+        got = out.download(np.float16, q.shape).astype(np.float32)
+        live = lens > 0
+        assert np.abs(got[live] - want[live]).max() <= TOL16, lens
+        assert np.all(got[~live] == 0)
+    for b in (dk, dv):
+        b.release()
+
+
 def test_error_codes():
     l = lib()
     assert l.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 8, 128, 16, 0, 0, 0, None) == 7

@@ -566,15 +566,17 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
 
 // ------------------------------------------------------------------------------------------------
 // GEMM over packed weights (M > 32).  Workgroup tile: 256 rows of W (16 packed row tiles, 4 per
-// wavefront) x 128 rows of x; K advances 128 per step.  The W fragments come straight from the
+// wavefront; 2 or 1 per wavefront when the problem is too small to fill the chip with that) x 64 or
+// 128 rows of x; K advances 128 per step.  The W fragments come straight from the
 // packed buffer (1 KiB contiguous per load, no LDS); the x tile of a step (128 x 128 halves) is
 // staged once per workgroup into LDS (XOR-swizzled, double-buffered) with coalesced loads and read
 // back as MFMA "B" fragments by all four wavefronts.  Loads of step i+1 are issued before the 128
 // MFMAs of step i.  Workgroup ids are mapped so that the m-blocks sharing a block of W rows run on
 // the same XCD back to back: that XCD's L2 then serves W to all of them after one HBM read.
 // ------------------------------------------------------------------------------------------------
-constexpr int kGN = 256, kGK = 128;  // workgroup tile: kGN weight rows x GM rows of x, K in steps of kGK
+constexpr int kGK = 128;  // workgroup tile: 64 TW weight rows (TW row tiles per wavefront) x GM rows of x, K in steps of kGK
 int g_gemm_rows = 0;                 // measurement hook: 64 or 128 rows of x per workgroup (0 = default)
+int g_gemm_tiles = 0;                // measurement hook: 1, 2 or 4 row tiles of W per wavefront (0 = by size)
 constexpr int kXcds = 8;
 
 // FULL: K is a multiple of the 128-column step, so no load needs a predicate (rows and tiles past
@@ -583,7 +585,7 @@ constexpr int kXcds = 8;
 // GM: rows of x per workgroup.  128 gives the larger tile (one workgroup per CU, 87 flop per byte
 // moved from L2); 64 halves the registers so that two workgroups share a CU and one's loads hide
 // behind the other's MFMAs.
-template <typename XT, bool FULL, int GM>
+template <typename XT, bool FULL, int GM, int TW>
 __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kernel(PackedArgs a, int n_blocks, int m_blocks) {
   constexpr int MT = GM / 16;        // x row tiles per wavefront
   constexpr int XV = GM * 16 / 256;  // 16-byte x vectors staged per thread and step
@@ -596,15 +598,15 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
   const int nb = (slot / m_blocks) * kXcds + xcd, mb = slot % m_blocks;
   if (nb >= n_blocks) return;
   const int n_tiles = (a.N + 15) / 16;
-  const int tile0 = nb * (kGN / 16) + wave * 4;  // first of this wavefront's 4 row tiles
+  const int tile0 = (nb * 4 + wave) * TW;  // first of this wavefront's TW row tiles
   const int m0 = mb * GM;
   const XT *x = static_cast<const XT *>(a.x);
   const int steps = (a.KC + 3) / 4;  // 4 chunks of 32 K per step
 
-  const __half *wt[4];
-  bool wok[4];
+  const __half *wt[TW];
+  bool wok[TW];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < TW; ++t) {
     wok[t] = tile0 + t < n_tiles;
     wt[t] = a.wp + (static_cast<int64_t>(wok[t] ? tile0 + t : 0) * a.KC) * 512 + lane * 8;
   }
@@ -634,18 +636,18 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
     }
   };
 
-  float4_t acc[4][MT];
+  float4_t acc[TW][MT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < TW; ++t)
 #pragma unroll
     for (int u = 0; u < MT; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  half8_t wf[4][4];  // [row tile][chunk within the step]
+  half8_t wf[TW][4];  // [row tile][chunk within the step]
   half8_t xv[XV];
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) wf[t][j] = load_w(t, j);
+    for (int t = 0; t < TW; ++t) wf[t][j] = load_w(t, j);
   load_x(0, xv);
   store_x(0, xv);
   __syncthreads();
@@ -669,14 +671,14 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
         bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
       }
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < TW; ++t)
 #pragma unroll
         for (int u = 0; u < MT; ++u)
           acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[t][j], bf[u], acc[t][u], 0, 0, 0);
       // the fragments of chunk j are consumed: fetch chunk j of the next step into the same registers
       if (more) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) wf[t][j] = load_w(t, nxt * 4 + j);
+        for (int t = 0; t < TW; ++t) wf[t][j] = load_w(t, nxt * 4 + j);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -693,9 +695,9 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
 #pragma unroll
   for (int u = 0; u < MT; ++u) {
     const int m = m0 + u * 16 + r;
-    if (a.glu) {
+    if (TW % 2 == 0 && a.glu) {
 #pragma unroll
-      for (int t = 0; t < 4; t += 2) {
+      for (int t = 0; t + 1 < TW; t += 2) {
         float v[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -706,7 +708,7 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
       }
     } else {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
+      for (int t = 0; t < TW; ++t) {
         const float v[4] = {acc[t][u][0], acc[t][u][1], acc[t][u][2], acc[t][u][3]};
         store_out4(o, m, (tile0 + t) * 16 + 4 * g, v);
       }
@@ -714,21 +716,42 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
   }
 }
 
-template <typename XT>
-void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
-  const int gm = g_gemm_rows > 0 ? g_gemm_rows : 64;
-  const int n_blocks = (a.N + kGN - 1) / kGN, m_blocks = (a.M + gm - 1) / gm;
+// Weight rows per workgroup: 256 (four row tiles per wavefront), or 128 / 64 when 256 would leave CUs
+// without a workgroup (M = 512, N = 2048: 64 workgroups of 256 x 64, 256 of 64 x 64).
+int gemm_tiles_per_wave(const PackedArgs &a, int gm) {
+  if (g_gemm_tiles == 1 || g_gemm_tiles == 2 || g_gemm_tiles == 4) return g_gemm_tiles;
+  const int64_t m_blocks = (a.M + gm - 1) / gm;
+  int tw = 4;
+  while (tw > 1 && ((a.N + 64 * tw - 1) / (64 * tw)) * m_blocks < 256) tw /= 2;
+  if (a.glu && tw < 2) tw = 2;  // the gated epilogue needs a gate tile and its up tile in one wavefront
+  return tw;
+}
+
+template <typename XT, int TW>
+void launch_gemm_packed_tw(const PackedArgs &a, int gm, hipStream_t st) {
+  const int gn = 64 * TW;
+  const int n_blocks = (a.N + gn - 1) / gn, m_blocks = (a.M + gm - 1) / gm;
   const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;  // whole rounds over the XCDs
   const dim3 grid(static_cast<unsigned>(nb_pad) * m_blocks);
   const bool full = a.K % kGK == 0;
 #define AXHIP_GEMM_LAUNCH(F, G) \
-  hipLaunchKernelGGL((linear_gemm_packed_kernel<XT, F, G>), grid, dim3(256), 0, st, a, n_blocks, m_blocks)
+  hipLaunchKernelGGL((linear_gemm_packed_kernel<XT, F, G, TW>), grid, dim3(256), 0, st, a, n_blocks, m_blocks)
   if (gm == 128) {
     if (full) AXHIP_GEMM_LAUNCH(true, 128); else AXHIP_GEMM_LAUNCH(false, 128);
   } else {
     if (full) AXHIP_GEMM_LAUNCH(true, 64); else AXHIP_GEMM_LAUNCH(false, 64);
   }
 #undef AXHIP_GEMM_LAUNCH
+}
+
+template <typename XT>
+void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
+  const int gm = g_gemm_rows > 0 ? g_gemm_rows : 64;
+  switch (gemm_tiles_per_wave(a, gm)) {
+    case 1: return launch_gemm_packed_tw<XT, 1>(a, gm, st);
+    case 2: return launch_gemm_packed_tw<XT, 2>(a, gm, st);
+    default: return launch_gemm_packed_tw<XT, 4>(a, gm, st);
+  }
 }
 
 }  // namespace
@@ -740,6 +763,9 @@ extern "C" {
 
 // Measurement hook for sweeps (0 restores a default).
 AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows) {
+  // gemm_rows: 64 or 128 rows of x per GEMM workgroup, plus 1000 t to force t = 1, 2, 4 row tiles of W per wavefront
+  g_gemm_tiles = gemm_rows >= 1000 ? gemm_rows / 1000 : 0;
+  gemm_rows %= 1000;
   g_gemm_rows = (gemm_rows == 64 || gemm_rows == 128) ? gemm_rows : 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
@@ -841,7 +867,7 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
     ga.chunks_per_wave = 0;
     ga.out_f16 = out_dtype == AXHIP_FLOAT16;
     ga.glu = glu ? 1 : 0;
-    const int64_t wgs = ((N + kGN - 1) / kGN + kXcds - 1) / kXcds * kXcds * ((M + 63) / 64);
+    const int64_t wgs = ((N + 63) / 64 + kXcds - 1) / kXcds * kXcds * ((M + 63) / 64);  // the smallest tile
     if (wgs > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
     if (x_dtype == AXHIP_FLOAT16)
       launch_gemm_packed<__half>(ga, as_stream(stream));

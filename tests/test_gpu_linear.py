@@ -183,3 +183,31 @@ def test_packed_gemm_glu_large_M():
     np.testing.assert_allclose(gu.linear_f16_packed(x, w, glu=True), want, rtol=0, atol=2e-5)
     got16 = gu.linear_f16_packed(x, w, out_dtype=np.float16, glu=True)
     assert np.abs(got16.astype(np.float32) - want).max() <= 2e-3
+
+
+@pytest.mark.parametrize("tiles", [1, 2, 4])
+def test_packed_gemm_row_tiles_per_wavefront(tiles):
+    """The GEMM's weight-row tile (64, 128 or 256 rows per workgroup; chosen by problem size) forced to each
+    height on one ragged shape: same bits from all three (K is summed in the same order), bias, and the
+    gate/up layout where a wavefront holds a gate tile and its up tile."""
+    rng = np.random.default_rng(5)
+    M, K, N = 300, 264, 600
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.05 * rng.standard_normal((N, K)))
+    b = h16(0.05 * rng.standard_normal(N))
+    l = gu.lib()
+    base = gu.linear_f16_packed(x, w, b)
+    l.axhip_linear_f16_tune(0, 0, 0, 1000 * tiles + 64)
+    try:
+        out = gu.linear_f16_packed(x, w, b)
+        glu = gu.linear_f16_packed(x, w[:576], glu=True) if tiles >= 2 else None
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
+    np.testing.assert_array_equal(out, base)
+    want = port.linear(x.astype(np.float32), w.astype(np.float32), b.astype(np.float32))
+    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
+    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag + 1e-3 * 2.0 ** -11)
+    if glu is not None:
+        gu_ = port.linear(x.astype(np.float32), w[:576].astype(np.float32))
+        wantg = port.silu_mul(np.ascontiguousarray(gu_[:, :288]), np.ascontiguousarray(gu_[:, 288:]))
+        np.testing.assert_allclose(glu, wantg, rtol=0, atol=2e-5)

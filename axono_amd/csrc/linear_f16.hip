@@ -662,19 +662,27 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
     // keep the prefetches where they are written: left alone, the scheduler sinks them to the end of
     // the step (shorter live ranges) and the step then waits out a full memory latency
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      half8_t bf[MT];
+    // x fragments are read from LDS one chunk ahead of their products: four reads per 4 TW products
+    // keep the LDS half busy, and a wavefront that waits for its reads before every chunk leaves the
+    // matrix pipe idle for as long
+    half8_t bf[2][MT];
+    auto load_bf = [&](int j, half8_t (&f)[MT]) {
 #pragma unroll
       for (int u = 0; u < MT; ++u) {
         const int row = u * 16 + r, unit = j * 4 + g;
-        bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
+        f[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
       }
+    };
+    load_bf(0, bf[0]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (j + 1 < 4) load_bf(j + 1, bf[(j + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < TW; ++t)
 #pragma unroll
         for (int u = 0; u < MT; ++u)
-          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[t][j], bf[u], acc[t][u], 0, 0, 0);
+          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[t][j], bf[j & 1][u], acc[t][u], 0, 0, 0);
       // the fragments of chunk j are consumed: fetch chunk j of the next step into the same registers
       if (more) {
 #pragma unroll

@@ -724,6 +724,131 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kern
   }
 }
 
+// 256 weight rows x 128 rows of x with two workgroups per CU.  Against the 256 x 64 tile this halves
+// the W bytes that pass through the CU's vector memory path per product (that path, 64 bytes per
+// clock, is what bounds the smaller tile), but its 128 accumulators leave room for little else in the
+// 256 registers of a wavefront at this occupancy: the W fragments are held for two chunks of 32 K only
+// (chunk j+2 is requested when chunk j has been used), and the x fragments of a chunk are read from
+// LDS when they are needed.  K % 128 == 0, N in whole row tiles handled by clamping.
+template <typename XT>
+__global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedArgs a, int n_blocks, int m_blocks) {
+  constexpr int GM = 128, MT = 8, TW = 4;
+  constexpr int XV = GM * 16 / 256;
+  __shared__ __attribute__((aligned(16))) _Float16 xs[2][GM * kGK];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int id = blockIdx.x;
+  const int xcd = id % kXcds, slot = id / kXcds;
+  const int nb = (slot / m_blocks) * kXcds + xcd, mb = slot % m_blocks;
+  if (nb >= n_blocks) return;
+  const int n_tiles = (a.N + 15) / 16;
+  const int tile0 = (nb * 4 + wave) * TW;
+  const int m0 = mb * GM;
+  const XT *x = static_cast<const XT *>(a.x);
+  const int chunks = a.K / 32, steps = chunks / 4;
+
+  const __half *wt[TW];
+#pragma unroll
+  for (int t = 0; t < TW; ++t)
+    wt[t] = a.wp + (static_cast<int64_t>(min(tile0 + t, n_tiles - 1)) * a.KC) * 512 + lane * 8;
+  auto load_w = [&](int chunk, half8_t (&f)[TW]) {
+    const int64_t off = static_cast<int64_t>(min(chunk, chunks - 1)) * 512;  // past the end: the last chunk again
+#pragma unroll
+    for (int t = 0; t < TW; ++t) f[t] = load_h8(wt[t] + off);
+  };
+  // x staging: 128 rows x 16 units of 16 bytes per step, 8 per thread; 32-bit element offsets
+  unsigned xo[XV];
+#pragma unroll
+  for (int p = 0; p < XV; ++p) {
+    const int v = p * 256 + tid;
+    xo[p] = static_cast<unsigned>(min(m0 + (v >> 4), a.M - 1)) * static_cast<unsigned>(a.K) + (v & 15) * 8;
+  }
+  auto load_x = [&](int step, half8_t (&xv)[XV]) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) xv[p] = load_h8(x + (static_cast<size_t>(xo[p]) + step * kGK));
+  };
+  auto store_x = [&](int buf, const half8_t (&xv)[XV]) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) {
+      const int v = p * 256 + tid;
+      const int row = v >> 4, unit = v & 15;
+      *reinterpret_cast<half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]) = xv[p];
+    }
+  };
+
+  float4_t acc[TW][MT];
+#pragma unroll
+  for (int t = 0; t < TW; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  half8_t wf[2][TW];  // chunk c waits in wf[c & 1]
+  half8_t xv[XV];
+  load_w(0, wf[0]);
+  load_w(1, wf[1]);
+  load_x(0, xv);
+  store_x(0, xv);
+  __syncthreads();
+
+  for (int i = 0; i < steps; ++i) {
+    const int buf = i & 1;
+    load_x(min(i + 1, steps - 1), xv);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int uh = 0; uh < MT; uh += 4) {  // x fragments four at a time: registers
+        half8_t bf[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int row = (uh + u) * 16 + r, unit = j * 4 + g;
+          bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
+        }
+#pragma unroll
+        for (int t = 0; t < TW; ++t)
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            acc[t][uh + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j & 1][t], bf[u], acc[t][uh + u], 0, 0, 0);
+      }
+      load_w(i * 4 + j + 2, wf[j & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    store_x(buf ^ 1, xv);
+    __syncthreads();
+  }
+
+  LinearArgs o;
+  o.bias = a.bias;
+  o.out = a.out;
+  o.M = a.M;
+  o.N = a.glu ? a.N / 2 : a.N;
+  o.out_f16 = a.out_f16;
+  if (a.glu) {
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+#pragma unroll
+      for (int t = 0; t < TW; t += 2) {
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float gt = acc[t][u][q];
+          v[q] = gt / (1.0f + expf(-gt)) * acc[t + 1][u][q];
+        }
+        store_out4(o, m0 + u * 16 + r, ((tile0 + t) / 2) * 16 + 4 * g, v);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+#pragma unroll
+      for (int t = 0; t < TW; ++t) {
+        const float v[4] = {acc[t][u][0], acc[t][u][1], acc[t][u][2], acc[t][u][3]};
+        store_out4(o, m0 + u * 16 + r, (tile0 + t) * 16 + 4 * g, v);
+      }
+    }
+  }
+}
+
 // Weight rows per workgroup: 256 (four row tiles per wavefront), or 128 / 64 when 256 would leave CUs
 // without a workgroup (M = 512, N = 2048: 64 workgroups of 256 x 64, 256 of 64 x 64).
 int gemm_tiles_per_wave(const PackedArgs &a, int gm) {
@@ -754,7 +879,19 @@ void launch_gemm_packed_tw(const PackedArgs &a, int gm, hipStream_t st) {
 
 template <typename XT>
 void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
-  const int gm = g_gemm_rows > 0 ? g_gemm_rows : 64;
+  if constexpr (sizeof(XT) == 2) {  // fp32 x waits for its conversion in twice the registers: it keeps the 64-row tile
+    // by default wherever it gives every CU a workgroup
+    const bool fits = a.K % kGK == 0 && static_cast<int64_t>(a.M) * a.K < (1ll << 32);
+    const int64_t tiles128 = static_cast<int64_t>((a.N + 255) / 256) * ((a.M + 127) / 128);
+    if (fits && (g_gemm_rows == 256 || (g_gemm_rows == 0 && g_gemm_tiles == 0 && tiles128 >= 256))) {
+      const int n_blocks = (a.N + 255) / 256, m_blocks = (a.M + 127) / 128;
+      const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
+      hipLaunchKernelGGL((linear_gemm_packed_128_kernel<XT>), dim3(static_cast<unsigned>(nb_pad) * m_blocks), dim3(256), 0,
+                         st, a, n_blocks, m_blocks);
+      return;
+    }
+  }
+  const int gm = (g_gemm_rows == 64 || g_gemm_rows == 128) ? g_gemm_rows : 64;
   switch (gemm_tiles_per_wave(a, gm)) {
     case 1: return launch_gemm_packed_tw<XT, 1>(a, gm, st);
     case 2: return launch_gemm_packed_tw<XT, 2>(a, gm, st);
@@ -774,7 +911,7 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
   // gemm_rows: 64 or 128 rows of x per GEMM workgroup, plus 1000 t to force t = 1, 2, 4 row tiles of W per wavefront
   g_gemm_tiles = gemm_rows >= 1000 ? gemm_rows / 1000 : 0;
   gemm_rows %= 1000;
-  g_gemm_rows = (gemm_rows == 64 || gemm_rows == 128) ? gemm_rows : 0;
+  g_gemm_rows = (gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256) ? gemm_rows : 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;

@@ -296,7 +296,8 @@ AXHIP_API int axhip_rope_with_cos_sin(const void *x, const float *cos_t, const f
 AXHIP_API size_t axhip_linear_f16_workspace_bytes(int64_t M, int64_t K, int64_t N);
 /* Measurement hook for the skinny-M kernel's plan (0 restores a default): wavefronts to aim for,
  * 16-row groups of W per wavefront (1, 2 or 4), wavefronts (K slices) per workgroup (4, 8, 16);
- * for the M > 32 GEMM, rows of x per workgroup (64 or 128), plus 1000 t to force t = 1, 2 or 4 row
+ * for the M > 32 GEMM, the tile: 64 or 128 rows of x per workgroup (128: one workgroup per CU), 256 = the
+ * 256 x 128 tile at two workgroups per CU (the default for large problems), plus 1000 t to force t = 1, 2 or 4 row
  * tiles of W per wavefront (64, 128 or 256 weight rows per workgroup; by default the largest that still
  * gives every CU a workgroup).  No reference counterpart (the reference leaves the choice to cuBLAS). */
 AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows);

@@ -211,3 +211,32 @@ def test_packed_gemm_row_tiles_per_wavefront(tiles):
         gu_ = port.linear(x.astype(np.float32), w[:576].astype(np.float32))
         wantg = port.silu_mul(np.ascontiguousarray(gu_[:, :288]), np.ascontiguousarray(gu_[:, 288:]))
         np.testing.assert_allclose(glu, wantg, rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 128, 256), (700, 384, 520), (1000, 2048, 768)])
+def test_packed_gemm_256x128_tile(M, K, N):
+    """The 256 x 128 tile (two workgroups per CU, W fragments held two chunks ahead), forced on small shapes:
+    M and N that are not multiples of the tile, bias, fp16 output, the gate/up layout; same bits as the
+    64-row tile (K is summed in the same order)."""
+    rng = np.random.default_rng(M + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    b = h16(0.05 * rng.standard_normal(N))
+    l = gu.lib()
+    base = gu.linear_f16_packed(x, w, b)
+    l.axhip_linear_f16_tune(0, 0, 0, 256)
+    try:
+        out = gu.linear_f16_packed(x, w, b)
+        out16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16)
+        n2 = N // 32 * 32
+        glu = gu.linear_f16_packed(x, w[:n2], glu=True)
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
+    np.testing.assert_array_equal(out, base)
+    want = port.linear(x.astype(np.float32), w.astype(np.float32), b.astype(np.float32))
+    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
+    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag + 1e-3 * 2.0 ** -11)
+    assert np.abs(out16.astype(np.float32) - want).max() <= 2e-3
+    gu_ = port.linear(x.astype(np.float32), w[:n2].astype(np.float32))
+    wantg = port.silu_mul(np.ascontiguousarray(gu_[:, : n2 // 2]), np.ascontiguousarray(gu_[:, n2 // 2:]))
+    np.testing.assert_allclose(glu, wantg, rtol=0, atol=2e-5)

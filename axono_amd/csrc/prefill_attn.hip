@@ -179,19 +179,25 @@ __global__ __launch_bounds__(kPThreads) void prefill_attn_kernel(PrefillArgs a) 
           mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
           mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
           const float mn = fmaxf(m[t], mx);
-          const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
-          m[t] = mn;
           float ps = 0.f;
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             float p = __builtin_amdgcn_exp2f(x[j] - mn);
-            if (x[j] <= kMasked) p = 0.f;  // a fully masked row keeps m == kMasked: exp2(0) would count
+            // a fully masked row keeps m == kMasked: exp2(0) would count (masks occur in diagonal blocks only)
+            if (diag && x[j] <= kMasked) p = 0.f;
             ps += p;
             pf[t][j] = static_cast<_Float16>(p);
           }
-          lsum[t] = lsum[t] * corr + ps;
+          // once the running maxima have settled, most blocks change none of them: the rescale of the
+          // 4 DT output registers is skipped when no query of the wavefront needs it
+          if (__any(mn != m[t])) {
+            const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
+            lsum[t] *= corr;
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
+            for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
+          }
+          m[t] = mn;
+          lsum[t] += ps;
         }
         // ---- O^T += V^T . P^T ----
         const _Float16 *vst_l = &vs[buf][sub * 32 * D];

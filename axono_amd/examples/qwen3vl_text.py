@@ -277,7 +277,7 @@ class Qwen3VLTextDecoder(nn.Module):
             xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
             for i in range(cfg.num_hidden_layers):
                 p = f"layers.{i}."
-                qkv = L.linear_nobias(xn, self._w(p + "self_attn.qkv_proj.weight"))  # [S, width] fp32
+                qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")  # [S, width] fp32
                 kc, vc = self._cache.get(i)
                 seq_off = b * nkv * lmax * D * esz
                 q = Tensor(DataType.FLOAT16, [S, nq, D], dev, _zero=False)
@@ -300,7 +300,7 @@ class Qwen3VLTextDecoder(nn.Module):
                     check(lib.axhip_gqa_decode(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, vis.data_ptr,
                                                attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq,
                                                nkv, D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
-                attn_out = L.linear_nobias(attn, self._w(p + "self_attn.o_proj.weight"))
+                attn_out = self._linear(attn, p + "self_attn.o_proj.weight")
                 h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                     DataType.FLOAT16)
                 mlp_out = self._mlp(xn2, p)

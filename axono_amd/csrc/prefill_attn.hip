@@ -57,8 +57,13 @@ __device__ __forceinline__ half4_t lds_v_tr(const _Float16 *stage, int key0, int
   return __builtin_bit_cast(half4_t, r);
 }
 
+// Up to two query heads per workgroup the kernel is held to 256 registers, so that two workgroups share
+// a CU (their 64 KB of LDS each fit): a wavefront's products wait on its own softmax arithmetic, and a
+// second wavefront per SIMD fills those gaps (B=1, S=4096: 372 -> 219 us).  Left to itself the
+// compiler takes 296 registers.  Sharing every K/V fragment among two tiles of 16 positions per
+// wavefront instead (half the LDS reads per product, one workgroup per CU) measured slower.
 template <int D, int G>
-__global__ __launch_bounds__(kPThreads) void prefill_attn_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel(PrefillArgs a) {
   constexpr int KK = D / 32;   // MFMA steps over d for S^T
   constexpr int DT = D / 16;   // d tiles of O^T
   constexpr int UPR = D / 8;   // 16-byte units per K/V row

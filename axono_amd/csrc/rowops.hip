@@ -283,18 +283,20 @@ struct RopeArgs {
   int heads, dim, h_lim, w_lim;
 };
 
+// One thread rotates 8 pairs (i, i + dim/2) of `hpt` consecutive heads of one row: the angles depend on
+// (row, i) only, so the accurate sincosf - most of this kernel's arithmetic - is paid once per hpt heads.
 template <typename T, int MODE>
-__global__ __launch_bounds__(kBlock) void rope_kernel(RopeArgs a, FreqTable ft) {
+__global__ __launch_bounds__(kBlock) void rope_kernel(RopeArgs a, FreqTable ft, int hpt) {
   const int half = a.dim / 2;
   const int chunks = (half + 7) / 8;  // 8-pair chunks per (row, head)
-  const int64_t total = a.rows * a.heads * chunks;
+  const int hgroups = a.heads / hpt;
+  const int64_t total = a.rows * hgroups * chunks;
   const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   if (t >= total) return;
   const int ch = static_cast<int>(t % chunks);
-  const int64_t rh = t / chunks;
-  const int64_t row = rh / a.heads;
-  const T *src = static_cast<const T *>(a.x) + rh * a.dim;
-  T *dst = static_cast<T *>(a.out) + rh * a.dim;
+  const int64_t rg = t / chunks;
+  const int64_t row = rg / hgroups;
+  const int64_t rh0 = row * a.heads + (rg % hgroups) * hpt;  // first (row, head) of this thread
   float pt = 0.f, ph = 0.f, pw = 0.f;
   if (MODE == kRopeTheta) pt = static_cast<float>(a.pos[row]);
   if (MODE == kRopeThd) {
@@ -304,29 +306,17 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(RopeArgs a, FreqTable ft) 
   }
   const int i0 = ch * 8;
   const bool full = (i0 + 8 <= half) && (half % 8 == 0) && (sizeof(T) * a.dim % 16 == 0);
-  float lo[8], hi[8];
-  if (full) {
-    Row8<T>::load(src + i0, lo);
-    Row8<T>::load(src + i0 + half, hi);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      lo[j] = (i0 + j < half) ? ldf(src + i0 + j) : 0.f;
-      hi[j] = (i0 + j < half) ? ldf(src + i0 + j + half) : 0.f;
-    }
-  }
-  float olo[8], ohi[8];
+  float c_lo[8], s_lo[8], c_hi[8], s_hi[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int i = i0 + j;
-    float c_lo, s_lo, c_hi, s_hi;
     if (MODE == kRopeTable) {
       const bool in = i < half;
       const float *cr = a.cos_t + row * a.dim, *sr = a.sin_t + row * a.dim;
-      c_lo = in ? cr[i] : 1.f;
-      s_lo = in ? sr[i] : 0.f;
-      c_hi = in ? cr[i + half] : 1.f;
-      s_hi = in ? sr[i + half] : 0.f;
+      c_lo[j] = in ? cr[i] : 1.f;
+      s_lo[j] = in ? sr[i] : 0.f;
+      c_hi[j] = in ? cr[i + half] : 1.f;
+      s_hi[j] = in ? sr[i + half] : 0.f;
     } else {
       float f, ang;
       if (MODE == kRopeTheta) {
@@ -340,22 +330,41 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(RopeArgs a, FreqTable ft) 
         else if (i % 3 == 2 && i < a.w_lim)
           ang = pw * f;
       }
-      sincosf(ang, &s_lo, &c_lo);
-      c_hi = c_lo;
-      s_hi = s_lo;
+      sincosf(ang, &s_lo[j], &c_lo[j]);
+      c_hi[j] = c_lo[j];
+      s_hi[j] = s_lo[j];
     }
-    olo[j] = lo[j] * c_lo - hi[j] * s_lo;
-    ohi[j] = hi[j] * c_hi + lo[j] * s_hi;
   }
-  if (full) {
-    Row8<T>::store(dst + i0, olo);
-    Row8<T>::store(dst + i0 + half, ohi);
-  } else {
+  for (int hh = 0; hh < hpt; ++hh) {
+    const T *src = static_cast<const T *>(a.x) + (rh0 + hh) * a.dim;
+    T *dst = static_cast<T *>(a.out) + (rh0 + hh) * a.dim;
+    float lo[8], hi[8];
+    if (full) {
+      Row8<T>::load(src + i0, lo);
+      Row8<T>::load(src + i0 + half, hi);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        lo[j] = (i0 + j < half) ? ldf(src + i0 + j) : 0.f;
+        hi[j] = (i0 + j < half) ? ldf(src + i0 + j + half) : 0.f;
+      }
+    }
+    float olo[8], ohi[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      if (i0 + j < half) {
-        stf(dst + i0 + j, olo[j]);
-        stf(dst + i0 + j + half, ohi[j]);
+      olo[j] = lo[j] * c_lo[j] - hi[j] * s_lo[j];
+      ohi[j] = hi[j] * c_hi[j] + lo[j] * s_hi[j];
+    }
+    if (full) {
+      Row8<T>::store(dst + i0, olo);
+      Row8<T>::store(dst + i0 + half, ohi);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (i0 + j < half) {
+          stf(dst + i0 + j, olo[j]);
+          stf(dst + i0 + j + half, ohi[j]);
+        }
       }
     }
   }
@@ -369,11 +378,14 @@ int launch_rope(const RopeArgs &a, const FreqTable &ft, int dtype, hipStream_t s
   if (!a.x || !a.out) return AXHIP_INVALID_PTR;
   if (!aligned16(a.x) || !aligned16(a.out)) return AXHIP_INVALID_ARGUMENT;
   const int chunks = (a.dim / 2 + 7) / 8;
-  const unsigned grid = blocks_for(a.rows * a.heads * chunks, kBlock);
+  // heads per thread: as many as still leave about a thousand workgroups
+  int hpt = 1;
+  while (hpt < 8 && a.heads % (hpt * 2) == 0 && a.rows * (a.heads / (hpt * 2)) * chunks >= (1 << 18)) hpt *= 2;
+  const unsigned grid = blocks_for(a.rows * (a.heads / hpt) * chunks, kBlock);
   if (dtype == AXHIP_FLOAT16)
-    hipLaunchKernelGGL((rope_kernel<__half, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft);
+    hipLaunchKernelGGL((rope_kernel<__half, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft, hpt);
   else
-    hipLaunchKernelGGL((rope_kernel<float, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft);
+    hipLaunchKernelGGL((rope_kernel<float, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft, hpt);
   return launch_status();
 }
 

@@ -137,6 +137,28 @@ def test_mrope_family():
     np.testing.assert_allclose(gu.rope(xs, np.arange(4), 1e4), port.rope(xs, np.arange(4), 1e4), rtol=0, atol=TOL32)
 
 
+def test_rope_many_rows_shares_angles_across_heads():
+    """Prefill-sized inputs, where one thread rotates several heads of a row with one set of angles
+    (2, 4 or 8 heads per thread depending on the row count): all three rope forms, fp16 and fp32,
+    a head count that is not a power of two, and bit-equality with the one-head-per-thread result."""
+    rng = np.random.default_rng(29)
+    inv = port.rope_inv_freq(1e6, 128)
+    for rows, heads in ((4096, 16), (16384, 16), (8192, 12), (16384, 8)):
+        pos = rng.integers(0, 32768, rows).astype(np.int64)
+        x = h16(rng.standard_normal((rows, heads, 128)))
+        got = gu.rope(x, pos, 1e6)
+        assert_fp16_close(got, port.rope(x, pos, 1e6))
+        # the same rows in slices small enough for one head per thread
+        part = np.concatenate([gu.rope(x[i:i + 256], pos[i:i + 256], 1e6) for i in range(0, 1024, 256)])
+        np.testing.assert_array_equal(got[:1024].view(np.uint16), part.view(np.uint16))
+    rows, heads = 8192, 16
+    pos3 = rng.integers(0, 8192, (3, rows)).astype(np.int64)
+    x = rng.standard_normal((rows, heads, 128)).astype(np.float32)
+    np.testing.assert_allclose(gu.rope_thd(x, pos3, inv, [24, 20, 20]), port.rope_thd(x, pos3, inv, [24, 20, 20]), rtol=0, atol=TOL32)
+    wc, ws = port.mrope_cos_sin(pos3, inv, 20, 20)
+    np.testing.assert_allclose(gu.rope_with_cos_sin(x, wc, ws), port.rope_with_cos_sin(x, wc, ws), rtol=0, atol=TOL32)
+
+
 def test_kv_append_bit_exact_config2():
     rng = np.random.default_rng(24)
     B, Hkv, Lmax, D = 32, 8, 8192, 128

@@ -89,6 +89,8 @@ PROTOTYPES = {
                                          c_i, c_i, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_silu_mul_fused": (c_i, [c_vp, c_vp, c_i, c_i, c_i64, c_i64, c_vp]),
     "axhip_index_add": (c_i, [c_vp, c_i, c_i64, c_i64, c_vp]),
+    "axhip_embedding_rms_norm": (c_i, [c_vp, c_i, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "axhip_decode_advance": (c_i, [c_vp, c_vp, c_vp, c_i, c_vp, c_vp, c_i64, c_vp, c_i, c_vp]),
 }
 
 _lib = None

@@ -104,6 +104,67 @@ __global__ __launch_bounds__(kBlock) void qkv_norm_rope_append_kernel(QkvArgs a)
   }
 }
 
+// First operators of a decode step in one launch: h[i, :] = float(table[ids[i], :]) (the embedding row
+// widened to the fp32 residual stream) and xn[i, :] = fp16((h * rms) * w), the first RMSNorm.  Same
+// arithmetic, in the same order, as axhip_embedding -> axhip_cast -> axhip_rms_norm_ex: 8 elements per
+// thread and pass, per-thread fused multiply-add sum of squares, block sum, 1 / sqrt(mean + eps).
+constexpr int kEmbedChunks = 4;  // 8-element chunks a thread keeps: dim <= 256 * 8 * 4
+template <typename I, typename WT>
+__global__ __launch_bounds__(kBlock) void embed_norm_kernel(const I *__restrict__ ids, const __half *__restrict__ table,
+                                                            const WT *__restrict__ w, float eps, float *__restrict__ h,
+                                                            __half *__restrict__ xn, int64_t vocab, int dim) {
+  __shared__ float red[kBlock / 64];
+  const int64_t row = blockIdx.x;
+  const int64_t id = static_cast<int64_t>(ids[row]);
+  const bool valid = id >= 0 && id < vocab;  // out-of-range ids give a zero row, as the gather alone does
+  const __half *src = table + (valid ? id : 0) * dim;
+  const int nvec = dim / 8;
+  float keep[kEmbedChunks][8];
+  float ss = 0.f;
+  int c = 0;
+  for (int i = threadIdx.x; i < nvec; i += kBlock, ++c) {
+    float a[8];
+    Row8<__half>::load(src + i * 8, a);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      a[j] = valid ? a[j] : 0.f;
+      ss = __builtin_fmaf(a[j], a[j], ss);
+      keep[c][j] = a[j];
+    }
+    Row8<float>::store(h + row * dim + i * 8, a);
+  }
+  ss = block_sum<kBlock / 64>(ss, red);
+  const float rms = 1.0f / sqrtf(ss / static_cast<float>(dim) + eps);
+  c = 0;
+  for (int i = threadIdx.x; i < nvec; i += kBlock, ++c) {
+    float wv[8], o[8];
+    Row8<WT>::load(w + i * 8, wv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = keep[c][j] * rms * wv[j];
+    Row8<__half>::store(xn + row * dim + i * 8, o);
+  }
+}
+
+// Last operators of a greedy decode step in one launch (one workgroup): the chosen tokens become the
+// next step's input ids, positions and sequence lengths advance by one, and the tokens are appended
+// to a device-side log at the row a device-side counter names.
+__global__ __launch_bounds__(kBlock) void decode_advance_kernel(const int64_t *__restrict__ next_ids,
+                                                                int64_t *__restrict__ ids, int64_t *__restrict__ pos,
+                                                                int pos_rows, int32_t *__restrict__ seq_lens,
+                                                                int64_t *__restrict__ log, int64_t log_rows,
+                                                                unsigned long long *__restrict__ counter, int B) {
+  const unsigned long long step = counter ? *counter : 0ull;
+  for (int t = threadIdx.x; t < B; t += kBlock) {
+    const int64_t id = next_ids[t];
+    if (ids) ids[t] = id;
+    for (int r = 0; r < pos_rows; ++r) pos[static_cast<int64_t>(r) * B + t] += 1;
+    if (seq_lens) seq_lens[t] += 1;
+    if (log && step < static_cast<unsigned long long>(log_rows)) log[step * B + t] = id;
+  }
+  __syncthreads();  // every thread has read the counter
+  if (threadIdx.x == 0 && counter) *counter = step + 1;
+}
+
 template <typename T, typename OT>
 __global__ __launch_bounds__(kBlock) void silu_mul_fused_kernel(const T *__restrict__ gu,
                                                                 OT *__restrict__ y, int64_t rows,
@@ -198,6 +259,43 @@ AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int 
     hipLaunchKernelGGL((silu_mul_fused_kernel<float, float>), dim3(grid), dim3(kBlock), 0, st,
                        static_cast<const float *>(gate_up), static_cast<float *>(y), rows,
                        static_cast<int>(cols));
+  return launch_status();
+}
+
+AXHIP_API int axhip_embedding_rms_norm(const void *ids, int ids_dtype, const void *table, const void *weight,
+                                       int w_dtype, float eps, void *h, void *xn, int64_t n_ids, int64_t vocab,
+                                       int64_t dim, axhip_stream stream) {
+  if (ids_dtype != AXHIP_INT32 && ids_dtype != AXHIP_INT64) return AXHIP_UNSUPPORTED_TYPE;
+  if (w_dtype != AXHIP_FLOAT32 && w_dtype != AXHIP_FLOAT16) return AXHIP_UNSUPPORTED_TYPE;
+  if (n_ids < 0 || vocab <= 0 || dim <= 0 || dim % 8 != 0 || dim > kBlock * 8 * kEmbedChunks) return AXHIP_INVALID_ARGUMENT;
+  if (n_ids == 0) return AXHIP_OK;
+  if (!ids || !table || !weight || !h || !xn) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(table) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(h) |
+       reinterpret_cast<uintptr_t>(xn)) & 15)
+    return AXHIP_INVALID_ARGUMENT;
+  const dim3 grid(static_cast<unsigned>(n_ids));
+  hipStream_t st = as_stream(stream);
+#define AXHIP_EMBED_LAUNCH(I, WT)                                                                      \
+  hipLaunchKernelGGL((embed_norm_kernel<I, WT>), grid, dim3(kBlock), 0, st, static_cast<const I *>(ids), \
+                     static_cast<const __half *>(table), static_cast<const WT *>(weight), eps,          \
+                     static_cast<float *>(h), static_cast<__half *>(xn), vocab, static_cast<int>(dim))
+  if (ids_dtype == AXHIP_INT64) {
+    if (w_dtype == AXHIP_FLOAT16) AXHIP_EMBED_LAUNCH(int64_t, __half); else AXHIP_EMBED_LAUNCH(int64_t, float);
+  } else {
+    if (w_dtype == AXHIP_FLOAT16) AXHIP_EMBED_LAUNCH(int32_t, __half); else AXHIP_EMBED_LAUNCH(int32_t, float);
+  }
+#undef AXHIP_EMBED_LAUNCH
+  return launch_status();
+}
+
+AXHIP_API int axhip_decode_advance(const int64_t *next_ids, int64_t *ids, int64_t *pos, int pos_rows,
+                                   int32_t *seq_lens, int64_t *log, int64_t log_rows, uint64_t *counter, int B,
+                                   axhip_stream stream) {
+  if (B < 0 || pos_rows < 0 || log_rows < 0) return AXHIP_INVALID_ARGUMENT;
+  if (B == 0) return AXHIP_OK;
+  if (!next_ids || (pos_rows > 0 && !pos)) return AXHIP_INVALID_PTR;
+  hipLaunchKernelGGL(decode_advance_kernel, dim3(1), dim3(kBlock), 0, as_stream(stream), next_ids, ids, pos, pos_rows,
+                     seq_lens, log, log_rows, reinterpret_cast<unsigned long long *>(counter), B);
   return launch_status();
 }
 

@@ -198,8 +198,9 @@ class Qwen3VLTextDecoder(nn.Module):
         B = self._batch
         cache = self._cache
         max_len = attn_max_len or cache.max_len
-        h = L.embedding(ids, self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)  # [B,H]
-        xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
+        # embedding row widened to the fp32 residual stream + the first RMSNorm: one launch
+        h, xn = L.embedding_rms_norm(ids, self._w("embed_tokens.weight"), self._w("layers.0.input_layernorm.weight"),
+                                     cfg.rms_norm_eps)  # [B,H] each
         nl = cfg.num_hidden_layers
         nqd = cfg.num_attention_heads * cfg.head_dim
         if self.fused_tail and L.decode_layer_tail_supported(B, cfg.hidden_size, nqd, cfg.intermediate_size, 16):
@@ -320,13 +321,14 @@ class Qwen3VLTextDecoder(nn.Module):
         self._ids.copy_from_numpy(np.ascontiguousarray(first_ids, dtype=np.int64).reshape(B))
         self._pos.copy_from_numpy(np.ascontiguousarray(first_pos, dtype=np.int64).reshape(3, B))
         bound = min(self._cache.max_len, len(self._cache) + max_new_tokens + 1)
+        # the tokens of every step are gathered on the device, at the row a device-side counter names
+        self._log = Tensor(DataType.INT64, [max(max_new_tokens, 1), B], self._device)
+        self._counter = Tensor(DataType.INT64, [1], self._device)
 
         def step():
             logits, nxt = self.decode_forward(self._ids, self._pos, bound)
-            # feed the device-side state of the next step
-            check(self._lib.axhip_memcpy_d2d(self._ids.data_ptr, nxt.data_ptr, 8 * B), "copy")
-            L.index_add(self._pos, 1)
-            L.index_add(self._cache.seq_lens, 1)
+            # the device-side state of the next step, and the token log: one launch
+            L.decode_advance(nxt, self._ids, self._pos, self._cache.seq_lens, self._log, self._counter)
             return logits, nxt
 
         self._step_fn = step
@@ -343,23 +345,22 @@ class Qwen3VLTextDecoder(nn.Module):
         self._ids.copy_from_numpy(ids0)
         self._pos.copy_from_numpy(pos0)
         self._cache.seq_lens.copy_from_numpy(lens0)
+        self._counter.copy_from_numpy(np.zeros(1, np.int64))
         self._graph = g
         self._graph_out = g.outputs
         return g
 
     def generate(self, max_new_tokens: int, use_graph: bool = True):
         """Greedy decode loop.  Returns int64 [steps, B] of generated ids.  The tokens of every step
-        are gathered on the device and read back once at the end."""
-        B = self._batch
-        tokens = Tensor(DataType.INT64, [max_new_tokens, B], self._device)
-        lib = self._lib
-        for s in range(max_new_tokens):
+        are gathered on the device (by the step itself) and read back once at the end."""
+        if max_new_tokens > self._log.shape[0]:
+            raise ValueError("generate(): more steps than start_decode() was told to expect")
+        self._counter.copy_from_numpy(np.zeros(1, np.int64))
+        for _ in range(max_new_tokens):
             if use_graph:
                 self._graph.launch()
-                nxt = self._graph_out[1]
             else:
-                _, nxt = self._step_fn()
-            check(lib.axhip_memcpy_d2d(tokens.data_ptr + s * 8 * B, nxt.data_ptr, 8 * B), "copy")
+                self._step_fn()
         L.synchronize()
         self._cache._host_len += max_new_tokens
-        return tokens.numpy()
+        return self._log.numpy()[:max_new_tokens].copy()

@@ -468,6 +468,46 @@ def index_add(x: Tensor, delta: int) -> Tensor:
     return x
 
 
+def embedding_rms_norm(ids: Tensor, table: Tensor, weight: Tensor, eps: float):
+    """The opening of a decode step in one launch: (h, xn) with h = embedding(ids, table) widened to FLOAT32 and
+    xn = rms_norm(h, weight, eps) stored as FLOAT16 - bit for bit what the three operators give."""
+    op = "embedding_rms_norm"
+    _need_hip(op, ids, table, weight)
+    if ids.ndim < 1 or table.ndim != 2 or weight.ndim != 1 or weight.shape[0] != table.shape[1]:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if table.dtype != DataType.FLOAT16 or weight.dtype not in _FLOATS or ids.dtype not in (DataType.INT32, DataType.INT64):
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    vocab, hidden = table.shape
+    h = _new(DataType.FLOAT32, ids.shape + [hidden], table)
+    xn = _new(DataType.FLOAT16, ids.shape + [hidden], table)
+    check(_lib_().axhip_embedding_rms_norm(ids.data_ptr, int(ids.dtype), table.data_ptr, weight.data_ptr, int(weight.dtype),
+                                           float(eps), h.data_ptr, xn.data_ptr, ids.num_elements, vocab, hidden,
+                                           current_stream()), op)
+    return h, xn
+
+
+def decode_advance(next_ids: Tensor, ids: Tensor | None = None, pos: Tensor | None = None, seq_lens: Tensor | None = None,
+                   log: Tensor | None = None, counter: Tensor | None = None) -> None:
+    """The closing of a greedy decode step in one launch: ids = next_ids, pos += 1 (INT64 [rows, B]),
+    seq_lens += 1 (INT32 [B]), log[counter] = next_ids (INT64 [steps, B]), counter += 1 (INT64 [1])."""
+    op = "decode_advance"
+    _need_hip(op, next_ids)
+    B = next_ids.num_elements
+    if next_ids.dtype != DataType.INT64 or (ids is not None and ids.dtype != DataType.INT64) or \
+            (pos is not None and pos.dtype != DataType.INT64) or (seq_lens is not None and seq_lens.dtype != DataType.INT32) or \
+            (log is not None and log.dtype != DataType.INT64) or (counter is not None and counter.dtype != DataType.INT64):
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    for t in (ids, seq_lens):
+        if t is not None and t.num_elements != B:
+            raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if (pos is not None and pos.num_elements % B) or (log is not None and log.num_elements % B):
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    ptr = lambda t: t.data_ptr if t is not None else None
+    check(_lib_().axhip_decode_advance(next_ids.data_ptr, ptr(ids), ptr(pos), pos.num_elements // B if pos is not None else 0,
+                                       ptr(seq_lens), ptr(log), log.num_elements // B if log is not None else 0, ptr(counter),
+                                       B, current_stream()), op)
+
+
 def silu_mul_fused(gate_up: Tensor, out_dtype: DataType | None = None) -> Tensor:
     """[rows, 2*cols] = [gate | up] -> silu(gate) * up, [rows, cols]; out_dtype FLOAT16 for a FLOAT32
     input stores the result rounded once (for a result that only feeds an fp16 Linear)."""

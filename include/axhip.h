@@ -417,6 +417,24 @@ AXHIP_API void axhip_decode_layer_tail_tune(int workgroups, int skip_phases);
 AXHIP_API int axhip_silu_mul_fused(const void *gate_up, void *y, int dtype, int out_dtype, int64_t rows,
                                    int64_t cols, axhip_stream stream);
 
+/* First launch of a decode step: h[i, :] = float(table[ids[i], :]) (FLOAT16 table, FLOAT32 h: the
+ * residual stream) and xn[i, :] = FLOAT16 of rms_norm(h[i, :]) * weight - the arithmetic of
+ * axhip_embedding, axhip_cast and axhip_rms_norm_ex in that order, bit for bit.  dim % 8 == 0,
+ * dim <= 8192.  Replaces the sequence Embedding -> CastTo -> RmsNorm that opens
+ * Qwen3VLTextModel.forward, examples/vlm/qwen3vl/model.py:470-476. */
+AXHIP_API int axhip_embedding_rms_norm(const void *ids, int ids_dtype, const void *table, const void *weight,
+                                       int w_dtype, float eps, void *h, void *xn, int64_t n_ids, int64_t vocab,
+                                       int64_t dim, axhip_stream stream);
+
+/* Last launch of a greedy decode step: ids[b] = next_ids[b]; pos[r, b] += 1 for r < pos_rows;
+ * seq_lens[b] += 1; log[*counter, b] = next_ids[b] while *counter < log_rows; *counter += 1.  Any of
+ * ids, pos (with pos_rows 0), seq_lens, log and counter may be NULL.  The reference does all of this
+ * on the host between steps (examples/vlm/qwen3vl/model.py:739-748, 846-858); inside a captured step
+ * it has to happen on the device. */
+AXHIP_API int axhip_decode_advance(const int64_t *next_ids, int64_t *ids, int64_t *pos, int pos_rows,
+                                   int32_t *seq_lens, int64_t *log, int64_t log_rows, uint64_t *counter, int B,
+                                   axhip_stream stream);
+
 /* x[i] += delta in place for INT32 / INT64 device arrays (sequence lengths and positions that a
  * captured decode step advances on the device; the reference rebuilds them on the host each step,
  * examples/vlm/qwen3vl/model.py:739-748). */

@@ -332,3 +332,74 @@ def test_index_add():
     gu.synchronize()
     np.testing.assert_array_equal(d32.download(np.int32, (3,)), a32 + 1)
     np.testing.assert_array_equal(d64.download(np.int64, (3, 2)), a64 + 7)
+
+
+def test_embedding_rms_norm_equals_the_three_operators():
+    """One launch for embedding -> cast to fp32 -> rms_norm (fp16 out): same bits as the three operators."""
+    rng = np.random.default_rng(41)
+    vocab, dim, n = 1000, 2048, 16
+    table = h16(rng.standard_normal((vocab, dim)))
+    ids = rng.integers(0, vocab, n).astype(np.int64)
+    ids[3] = vocab + 5      # out of range: a zero row, as the gather alone gives
+    l = gu.lib()
+    for wdt in (np.float32, np.float16):
+        w = (1 + 0.1 * rng.standard_normal(dim)).astype(wdt)
+        di, dtb, dw = gu.dev(ids), gu.dev(table), gu.dev(w)
+        dh, dxn = gu.DeviceBuffer(n * dim * 4), gu.DeviceBuffer(n * dim * 2)
+        gu._run("axhip_embedding_rms_norm", di.ptr, gu.I64, dtb.ptr, dw.ptr, gu.dt(w), 1e-6, dh.ptr, dxn.ptr, n, vocab, dim, None)
+        gu.synchronize()
+        h, xn = dh.download(np.float32, (n, dim)), dxn.download(np.float16, (n, dim))
+        rows = table[np.clip(ids, 0, vocab - 1)].astype(np.float32)
+        rows[3] = 0
+        np.testing.assert_array_equal(h, rows)
+        # the separate operators on the device
+        e = gu.embedding(ids.reshape(n, 1), table).reshape(n, dim)
+        dh2, dxn2 = gu.dev(gu.cast(e, np.float32)), gu.DeviceBuffer(n * dim * 2)
+        gu._run("axhip_rms_norm_ex", dh2.ptr, dw.ptr, 1e-6, dxn2.ptr, gu.F32, gu.dt(w), gu.F16, n, dim, None)
+        gu.synchronize()
+        np.testing.assert_array_equal(xn.view(np.uint16), dxn2.download(np.float16, (n, dim)).view(np.uint16))
+        # and the oracle
+        want = port.rms_norm(rows, w.astype(np.float32), 1e-6)
+        assert_fp16_close(xn, want)
+    # int32 ids; argument checks
+    di32 = gu.dev(ids.astype(np.int32))
+    gu._run("axhip_embedding_rms_norm", di32.ptr, gu.I32, dtb.ptr, dw.ptr, gu.dt(w), 1e-6, dh.ptr, dxn.ptr, n, vocab, dim, None)
+    gu.synchronize()
+    np.testing.assert_array_equal(dh.download(np.float32, (n, dim)), rows)
+    assert l.axhip_embedding_rms_norm(di.ptr, gu.I64, dtb.ptr, dw.ptr, gu.dt(w), 1e-6, dh.ptr, dxn.ptr, n, vocab, 2044, None) == 1
+    assert l.axhip_embedding_rms_norm(di.ptr, gu.F32, dtb.ptr, dw.ptr, gu.dt(w), 1e-6, dh.ptr, dxn.ptr, n, vocab, dim, None) == 3
+    assert l.axhip_embedding_rms_norm(di.ptr, gu.I64, None, dw.ptr, gu.dt(w), 1e-6, dh.ptr, dxn.ptr, n, vocab, dim, None) == 7
+
+
+def test_decode_advance():
+    """ids <- next ids, positions and lengths + 1, token log at the device-side counter; several steps,
+    a log shorter than the number of steps, optional outputs left out."""
+    rng = np.random.default_rng(42)
+    l = gu.lib()
+    for B in (1, 16, 700):
+        ids = rng.integers(0, 1000, B).astype(np.int64)
+        pos = rng.integers(0, 8192, (3, B)).astype(np.int64)
+        lens = rng.integers(0, 4096, B).astype(np.int32)
+        log_rows = 3
+        d_ids, d_pos, d_lens = gu.dev(ids), gu.dev(pos), gu.dev(lens)
+        d_log, d_cnt = gu.dev(np.full((log_rows, B), -1, np.int64)), gu.dev(np.zeros(1, np.int64))
+        want_log = np.full((log_rows, B), -1, np.int64)
+        for step in range(5):
+            nxt = rng.integers(0, 1000, B).astype(np.int64)
+            d_nxt = gu.dev(nxt)
+            gu._run("axhip_decode_advance", d_nxt.ptr, d_ids.ptr, d_pos.ptr, 3, d_lens.ptr, d_log.ptr, log_rows, d_cnt.ptr, B, None)
+            gu.synchronize()
+            if step < log_rows:
+                want_log[step] = nxt
+            np.testing.assert_array_equal(d_ids.download(np.int64, (B,)), nxt)
+            np.testing.assert_array_equal(d_pos.download(np.int64, (3, B)), pos + step + 1)
+            np.testing.assert_array_equal(d_lens.download(np.int32, (B,)), lens + step + 1)
+            np.testing.assert_array_equal(d_log.download(np.int64, (log_rows, B)), want_log)
+            assert d_cnt.download(np.int64, (1,))[0] == step + 1
+        # only the ids
+        gu._run("axhip_decode_advance", d_nxt.ptr, d_ids.ptr, None, 0, None, None, 0, None, B, None)
+        gu.synchronize()
+        np.testing.assert_array_equal(d_lens.download(np.int32, (B,)), lens + 5)
+    assert l.axhip_decode_advance(None, d_ids.ptr, None, 0, None, None, 0, None, 4, None) == 7
+    assert l.axhip_decode_advance(d_nxt.ptr, d_ids.ptr, None, 3, None, None, 0, None, 4, None) == 7
+    assert l.axhip_decode_advance(d_nxt.ptr, d_ids.ptr, None, 0, None, None, 0, None, -1, None) == 1

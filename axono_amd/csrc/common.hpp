@@ -190,4 +190,19 @@ __device__ __forceinline__ float block_sum(float x, float *smem) {
   return t;
 }
 
+// ---- LDS reads of MFMA operands (attention kernels) ------------------------------------------------
+__device__ __forceinline__ half8_t lds_h8(const _Float16 *p) { return *reinterpret_cast<const half8_t *>(p); }
+
+// 4 keys x 16 d of row-major V, delivered transposed: this lane gets V[key0 .. key0+3][d0 + lane%16].
+// `row_base` points at V[key0][0] of the stage in LDS for this lane's group; rows are 2*D bytes.
+template <int D>
+__device__ __forceinline__ half4_t lds_v_tr(const _Float16 *stage, int key0, int d0, int c) {
+  const int key = key0 + (c >> 2);           // the row this lane addresses
+  const int unit = (d0 >> 3) + ((c & 3) >> 1);  // 16-byte unit within the row
+  const _Float16 *p = stage + key * D + ((unit ^ (key & (D / 8 - 1))) << 3) + ((c & 1) << 2);
+  typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+  const fp16x4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p));
+  return __builtin_bit_cast(half4_t, r);
+}
+
 }  // namespace axhip

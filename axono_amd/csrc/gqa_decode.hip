@@ -34,6 +34,7 @@ struct Tuning {
                                 // streaming loads (measured: 256 workgroups 153 us, 1024 163 us at
                                 // B=32 L=8192), and nothing has to be merged when a sequence is one
   int force_splits = 0;         // > 0: fixed split count for every sequence (measurement sweeps)
+  int mfma_groups = 1;          // 0: head groups of four and more stay on the vector path (measurement sweeps)
   int separate_merge = 0;       // 1: merge in a second kernel; 0: the last workgroup of a sequence merges
 };
 Tuning g_tuning;
@@ -176,6 +177,7 @@ struct DecodeArgs {
   float *part_ml;   // [B, Hq, n_splits, 2]  (running max in log2 units, running sum)
   int Hq, group, max_len, chunk, n_splits;
   int dynamic, active, split_stride, B, n_hg;  // see SplitPlan; split_stride = partial slots per (sequence, head)
+  int wg_heads;  // query heads per workgroup (the template parameter G on the vector path)
   int64_t stride_b, stride_h, stride_s;
   float scale_log2e;
   int fused_merge;  // the last workgroup of a (sequence, head group) merges the splits
@@ -356,8 +358,13 @@ __device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t st
 }
 
 // A sequence without keys: its output rows are zeros.
-template <typename T, int D, int G>
+template <typename T, int D, int G, bool MFMA = false>
 __device__ __forceinline__ void write_zero_rows(const DecodeArgs &a, int b, int hg) {
+  if constexpr (MFMA) {
+    for (int o = threadIdx.x; o < a.wg_heads * D; o += kThreads)
+      stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + hg * a.wg_heads) * D + o, 0.0f);
+    return;
+  }
   for (int o = threadIdx.x; o < G * D; o += kThreads)
     stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + hg * G) * D + o, 0.0f);
 }
@@ -560,6 +567,257 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   }
 }
 
+// The end of a range on the matrix-core path (the same steps as the tail of process_range, with the
+// head count at run time): the workgroup's NS partial states (running
+// maximum s_m[head][NS], sum s_l[head][NS], unnormalised output s_acc[head][NS][D], in LDS, complete
+// and visible) are combined; the only range of a sequence writes the result when `direct_ok`, otherwise
+// the range leaves its state in the workspace and (fused merge) the workgroup that takes the last
+// ticket of the (sequence, head group) combines all ranges.
+// The states are named through LDS pointers: as generic pointers they cost 64-bit addresses and flat loads.
+typedef const float __attribute__((address_space(3))) *lds_cfloat_ptr;
+typedef int __attribute__((address_space(3))) *lds_int_ptr;
+template <typename T, int D, int NS>
+__device__ __forceinline__ void finish_range(const DecodeArgs &a, int b, int hg, int h0, int heads, int split,
+                                             int n_valid, bool direct_ok, lds_cfloat_ptr s_m, lds_cfloat_ptr s_l,
+                                             lds_cfloat_ptr s_acc, lds_int_ptr s_last) {
+  const int tid = threadIdx.x;
+  for (int o = tid; o < heads * D; o += kThreads) {
+    const int g = o / D, d = o % D;
+    float mx = kNegBig;
+#pragma unroll
+    for (int r = 0; r < NS; ++r) mx = fmaxf(mx, s_m[g * NS + r]);
+    float lsum = 0.0f, asum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < NS; ++r) {
+      const float w = __builtin_amdgcn_exp2f(s_m[g * NS + r] - mx);
+      lsum = __builtin_fmaf(s_l[g * NS + r], w, lsum);
+      asum = __builtin_fmaf(s_acc[(g * NS + r) * D + d], w, asum);
+    }
+    const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
+    if (n_valid == 1 && direct_ok) {
+      // the only range of this sequence: normalise and write the result, nothing to merge
+      stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
+    } else {
+      st_agent(&a.part_acc[(bh * a.split_stride + split) * D + d], asum);
+      if (d == 0) {
+        st_agent(&a.part_ml[(bh * a.split_stride + split) * 2], mx);
+        st_agent(&a.part_ml[(bh * a.split_stride + split) * 2 + 1], lsum);
+      }
+    }
+  }
+  if (n_valid == 1 || !a.fused_merge) return;
+
+  // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
+  __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
+  if (tid == 0) {
+    unsigned int *ticket = &g_tickets[b * a.n_hg + hg];
+    const unsigned int t = atomicAdd(ticket, 1u);
+    *s_last = (t == static_cast<unsigned int>(n_valid - 1));
+    if (*s_last) atomicExch(ticket, 0u);  // ready for the next launch
+  }
+  __syncthreads();
+  if (!*s_last) return;
+  for (int o = tid; o < heads * D; o += kThreads) {
+    const int g = o / D, d = o % D;
+    const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
+    const float *ml = a.part_ml + bh * a.split_stride * 2;
+    const float *pa = a.part_acc + bh * a.split_stride * D + d;
+    // eight ranges at a time, every load of a batch in flight before the first is used (the loads
+    // go past the local caches: one at a time they would cost a memory round trip each)
+    float mx = kNegBig, lsum = 0.0f, asum = 0.0f;
+    for (int s0m = 0; s0m < n_valid; s0m += 8) {
+      float pm[8], pl[8], pv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int sidx = min(s0m + i, n_valid - 1);
+        pm[i] = ld_agent(ml + 2 * sidx);
+        pl[i] = ld_agent(ml + 2 * sidx + 1);
+        pv[i] = ld_agent(pa + static_cast<int64_t>(sidx) * D);
+      }
+      float bm = mx;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (s0m + i < n_valid) bm = fmaxf(bm, pm[i]);
+      const float keep = __builtin_amdgcn_exp2f(mx - bm);
+      lsum *= keep;
+      asum *= keep;
+      mx = bm;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (s0m + i >= n_valid) continue;
+        const float w = __builtin_amdgcn_exp2f(pm[i] - mx);
+        lsum = __builtin_fmaf(pl[i], w, lsum);
+        asum = __builtin_fmaf(pv[i], w, asum);
+      }
+    }
+    stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
+  }
+}
+
+// ---- large head groups: the matrix-core path ---------------------------------------------------------
+// With four or more query heads per kv head the per-key arithmetic of the loop above (one dot product
+// and one axpy of D elements per head and key on the vector ALUs) takes longer than the key's bytes take
+// to arrive (Hq=32, Hkv=8: 65 % of HBM peak; Hq=64: 38 %).  Here the heads of a kv head - up to 16 - are
+// the columns of one MFMA tile instead, exactly as the positions are in the prefill kernel:
+//   S^T = K . Q^T (16 keys x 16 heads per tile), O^T += V^T . P^T,
+// so a key costs the same whatever the group size, and K and V are read once per kv head.  One workgroup
+// per (sequence, kv head, key range); a stage of 128 keys of K and V travels through LDS (coalesced
+// streaming loads into registers one stage ahead, XOR-swizzled rows, V^T fragments by the transposing
+// LDS read), each of the 4 wavefronts takes 32 of the 128 keys and keeps its own online-softmax state for
+// the 16 columns; the four states are merged at the end like the row groups of the vector path.
+constexpr int kMfmaStage = 128;  // keys per LDS stage (32 per wavefront)
+constexpr int kMfmaHeads = 16;   // columns of the MFMA tile: heads per workgroup at most
+
+template <int D>
+__device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, int hg, int split, int n_valid,
+                                                   bool direct_ok, int s0, int s1) {
+  constexpr int KK = D / 32;   // MFMA steps over d for S^T
+  constexpr int DT = D / 16;   // d tiles of O^T
+  constexpr int UPR = D / 8;   // 16-byte units per K/V row
+  constexpr int VEC = kMfmaStage * UPR / kThreads;  // staging vectors per thread and tensor
+  // one stage of K and of V; once the keys are done, the four per-wavefront states live in the same memory
+  constexpr int kStateFloats = kMfmaHeads * 4 * (D + 2) + 1;  // + the merge flag
+  constexpr int kStageHalves = kMfmaStage * D;
+  constexpr int kLdsBytes = 2 * kStageHalves * 2 > kStateFloats * 4 ? 2 * kStageHalves * 2 : kStateFloats * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[kLdsBytes];
+  _Float16 *ks = reinterpret_cast<_Float16 *>(smem), *vs = ks + kStageHalves;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const int heads = a.wg_heads;     // query heads of this workgroup: columns 0 .. heads-1
+  const int h0 = hg * heads;
+  const int hk = h0 / a.group;
+
+  // Q as the B operand: column c is head h0 + c (columns past the last head are zero and never stored)
+  half8_t qf[KK];
+  {
+    const __half *qrow = static_cast<const __half *>(a.q) + (static_cast<int64_t>(b) * a.Hq + h0 + min(c, heads - 1)) * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qf[kk] = *reinterpret_cast<const half8_t *>(qrow + kk * 32 + g * 8);
+      if (c >= heads) qf[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+
+  const __half *kbase = static_cast<const __half *>(a.k) + b * a.stride_b + hk * a.stride_h;
+  const __half *vbase = static_cast<const __half *>(a.v) + b * a.stride_b + hk * a.stride_h;
+  // one stage waits in registers while the previous one is used from LDS.  (Two stages in registers
+  // measured no faster: at 255 registers the compiler parks loaded data in accumulator registers, which
+  // makes it wait for the loads early.  Per stage the kernel takes about 0.35 us more than its bytes do.)
+  half8_t kst[1][VEC], vst[1][VEC];
+  auto load_stage = [&](int key0, half8_t (&kr)[VEC], half8_t (&vr)[VEC]) {
+#pragma unroll
+    for (int p = 0; p < VEC; ++p) {
+      const int vi = p * kThreads + tid;
+      const int row = vi / UPR, unit = vi % UPR;
+      const int64_t off = static_cast<int64_t>(min(key0 + row, s1 - 1)) * a.stride_s + unit * 8;  // rows past the range: its last key again
+      kr[p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(kbase + off));
+      vr[p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(vbase + off));
+    }
+  };
+  // V rows past the range are stored as zeros: their probabilities are zero, and 0 * finite stays 0
+  auto store_stage = [&](int key0, const half8_t (&kr)[VEC], const half8_t (&vr)[VEC]) {
+#pragma unroll
+    for (int p = 0; p < VEC; ++p) {
+      const int vi = p * kThreads + tid;
+      const int row = vi / UPR, unit = vi % UPR;
+      const int o = row * D + ((unit ^ (row & (UPR - 1))) << 3);
+      *reinterpret_cast<half8_t *>(&ks[o]) = kr[p];
+      half8_t vv = vr[p];
+      if (key0 + row >= s1) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      *reinterpret_cast<half8_t *>(&vs[o]) = vv;
+    }
+  };
+
+  float4_t o[DT];
+  float m = kNegBig, lsum = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int n_stages = (s1 - s0 + kMfmaStage - 1) / kMfmaStage;
+  auto do_stage = [&](int st, half8_t (&kr)[VEC], half8_t (&vr)[VEC]) __attribute__((always_inline)) {
+    const int key0 = s0 + st * kMfmaStage;
+    store_stage(key0, kr, vr);
+    __syncthreads();
+    // the next stage into the registers just emptied; the last stage fetches itself again: no branch
+    load_stage(s0 + min(st + 1, n_stages - 1) * kMfmaStage, kr, vr);
+    __builtin_amdgcn_sched_barrier(0);
+    const int kb = key0 + wave * 32;  // first of this wavefront's 32 keys
+    if (kb < s1) {
+      const _Float16 *k_l = ks + wave * 32 * D;
+      float4_t sc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const int row = tk * 16 + c, unit = kk * 4 + g;
+          const half8_t kf = lds_h8(k_l + row * D + ((unit ^ (row & (UPR - 1))) << 3));
+          sc[tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[kk], sc[tk], 0, 0, 0);
+        }
+      // this lane: head c, keys kb + 16 tk + 4 g + e
+      const bool tail = kb + 32 > s1;
+      float x[8];
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = sc[tk][e] * a.scale_log2e;
+          if (tail && kb + tk * 16 + 4 * g + e >= s1) v = kNegBig;
+          x[tk * 4 + e] = v;
+        }
+      float mx = x[0];
+#pragma unroll
+      for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m, mx);
+      half8_t pf;
+      float ps = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float pr = __builtin_amdgcn_exp2f(x[j] - mn);
+        if (tail && x[j] <= kNegBig) pr = 0.f;
+        ps += pr;
+        pf[j] = static_cast<_Float16>(pr);
+      }
+      if (__any(mn != m)) {
+        const float corr = __builtin_amdgcn_exp2f(m - mn);
+        lsum *= corr;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
+      }
+      m = mn;
+      lsum += ps;
+      const _Float16 *v_l = vs + wave * 32 * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const half4_t lo = lds_v_tr<D>(v_l, 4 * g, dt * 16, c);
+        const half4_t hi = lds_v_tr<D>(v_l, 16 + 4 * g, dt * 16, c);
+        const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
+      }
+    }
+    __syncthreads();  // every wavefront is done with the stage before the next one overwrites it
+  };
+  load_stage(s0, kst[0], vst[0]);
+  for (int st = 0; st < n_stages; ++st) do_stage(st, kst[0], vst[0]);
+
+  // the four per-wavefront states, [head][wavefront]: maximum, sum, output
+  float *s_m = reinterpret_cast<float *>(smem), *s_l = s_m + kMfmaHeads * 4, *s_acc = s_l + kMfmaHeads * 4;
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  if (g == 0) {
+    s_m[c * 4 + wave] = m;
+    s_l[c * 4 + wave] = lsum;
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    *reinterpret_cast<float4_t *>(&s_acc[(c * 4 + wave) * D + dt * 16 + 4 * g]) = o[dt];
+  __syncthreads();
+  finish_range<__half, D, 4>(a, b, hg, h0, heads, split, n_valid, direct_ok, (lds_cfloat_ptr)s_m, (lds_cfloat_ptr)s_l,
+                             (lds_cfloat_ptr)s_acc, (lds_int_ptr)(s_acc + kMfmaHeads * 4 * D));
+}
+
 // Which keys a workgroup streams.
 //   Static plan: (range, head group, sequence) straight from the grid.
 //   Length-dealt plan: workgroup id = slot * n_hg + head group, and the `active` slots of a head group
@@ -576,8 +834,8 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
 //       sequences they belong to: a workgroup then works through a piece of each sequence its range
 //       touches, and every slot streams the same number of keys.  A sequence without keys gets its
 //       zeros from the slot that holds its place on the line.
-template <typename T, int D, int G, int U, bool QKV>
-__global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArgs a) {
+template <typename T, int D, int G, int U, bool QKV, bool MFMA = false>
+__global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kernel(DecodeArgs a) {
   // the piece to work on: keys [s0, s1) of sequence b, range `split` of its n_valid ranges
   int b, hg, split, n_valid, s0, s1;
   bool direct_ok = true;
@@ -592,7 +850,7 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
     if (s0 >= len_b) {
       // an empty range is never read by the merge; without a merge kernel the zeros of a sequence
       // without keys come from its first workgroup
-      if (len_b == 0 && split == 0 && direct_ok) write_zero_rows<T, D, G>(a, b, hg);
+      if (len_b == 0 && split == 0 && direct_ok) write_zero_rows<T, D, G, MFMA>(a, b, hg);
       return;
     }
   } else {
@@ -640,13 +898,17 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
         const int len_b = clamped_len(a.seq_lens, b, a.max_len, a.len_add);
         const int first_slot = start_b / cc, last_slot = (start_b + len_b - 1) / cc;
         if (again) __syncthreads();  // the previous piece is done with the LDS arrays
-        process_range<T, D, G, U, QKV, false>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
-                                       max(g0 - start_b, 0), min(g1 - start_b, len_b));
+        if constexpr (MFMA)
+          process_range_mfma<D>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true, max(g0 - start_b, 0),
+                                min(g1 - start_b, len_b));
+        else
+          process_range<T, D, G, U, QKV, false>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
+                                                max(g0 - start_b, 0), min(g1 - start_b, len_b));
       }
       while (empty) {
         const int e = uni(__ffsll(empty) - 1);
         empty &= empty - 1;
-        write_zero_rows<T, D, G>(a, e, hg);
+        write_zero_rows<T, D, G, MFMA>(a, e, hg);
       }
       return;
     }
@@ -663,11 +925,14 @@ __global__ __launch_bounds__(kThreads, 4) void gqa_decode_split_kernel(DecodeArg
     s0 = split * chunk;
     s1 = min(s0 + chunk, len_b);
     if (s0 >= len_b) {
-      if (len_b == 0 && split == 0) write_zero_rows<T, D, G>(a, b, hg);
+      if (len_b == 0 && split == 0) write_zero_rows<T, D, G, MFMA>(a, b, hg);
       return;
     }
   }
-  process_range<T, D, G, U, QKV, true>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+  if constexpr (MFMA)
+    process_range_mfma<D>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+  else
+    process_range<T, D, G, U, QKV, true>(a, b, hg, split, n_valid, direct_ok, s0, s1);
 }
 
 // Cross-split merge: one workgroup of D threads per (sequence, query head).
@@ -710,6 +975,16 @@ int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   return launch_status();
 }
 
+template <int D>
+int launch_decode_mfma(const DecodeArgs &a, int B, hipStream_t st) {
+  const int n_hg = a.n_hg;
+  const dim3 grid(a.dynamic ? a.active * n_hg : a.n_splits, a.dynamic ? 1 : n_hg, a.dynamic ? 1 : B);
+  hipLaunchKernelGGL((gqa_decode_split_kernel<__half, D, 1, 8, false, true>), grid, dim3(kThreads), 0, st, a);
+  if (a.n_splits > 1 && !a.fused_merge)
+    hipLaunchKernelGGL((gqa_decode_merge_kernel<__half, D>), dim3(a.Hq, B), dim3(D), 0, st, a);
+  return launch_status();
+}
+
 template <typename T, int D>
 int dispatch_group(const DecodeArgs &a, int G, int B, hipStream_t st) {
   switch (G) {
@@ -731,6 +1006,13 @@ int dispatch_dim(const DecodeArgs &a, int D, int G, int B, hipStream_t st) {
 
 // Query heads served per workgroup: the largest of 4, 2, 1 that divides the group size.
 int heads_per_workgroup(int group) { return group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1); }
+// Matrix-core path: all heads of a kv head in one workgroup when there are at most 16 (the columns of a
+// tile), otherwise the largest divisor of the group size that fits.
+int mfma_heads_per_workgroup(int group) {
+  int h = group < kMfmaHeads ? group : kMfmaHeads;
+  while (group % h != 0) --h;
+  return h;
+}
 
 }  // namespace
 }  // namespace axhip
@@ -742,7 +1024,11 @@ namespace {
 int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int dtype, int B, int Hq, int Hkv,
                     int D, int max_len, axhip_stream stream) {
   const int group = Hq / Hkv;
-  const int G = heads_per_workgroup(group);
+  // four or more heads per kv head, fp16, plain form: the heads of a kv head become the columns of an MFMA tile
+  const bool mfma = g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) && !a.len_add &&
+                    a.stride_s % 8 == 0 && a.stride_h % 8 == 0 && a.stride_b % 8 == 0;
+  const int G = mfma ? mfma_heads_per_workgroup(group) : heads_per_workgroup(group);
+  a.wg_heads = G;
   const SplitPlan plan = plan_splits(B, Hq / G, max_len);
   a.Hq = Hq;
   a.group = group;
@@ -769,6 +1055,7 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
     a.part_ml = a.part_acc + acc_elems;
   }
   hipStream_t st = as_stream(stream);
+  if (mfma) return D == 128 ? launch_decode_mfma<128>(a, B, st) : launch_decode_mfma<64>(a, B, st);
   return dtype == AXHIP_FLOAT16 ? dispatch_dim<__half>(a, D, G, B, st) : dispatch_dim<float>(a, D, G, B, st);
 }
 }  // namespace
@@ -780,13 +1067,18 @@ AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits) {
   // a negative target selects the two-kernel form for a forced split count (split kernel + merge kernel)
   g_tuning.separate_merge = target_workgroups < 0 ? 1 : 0;
   g_tuning.target_workgroups = target_workgroups > 0 ? target_workgroups : Tuning().target_workgroups;
+  // force_splits >= 1000: keep large head groups on the vector path (for comparison), splits = force_splits - 1000
+  g_tuning.mfma_groups = force_splits >= 1000 ? 0 : 1;
+  if (force_splits >= 1000) force_splits -= 1000;
   g_tuning.force_splits = force_splits > 0 ? force_splits : 0;
 }
 
 // Reports the plan the launcher will use (tests and benchmarks print it).
 AXHIP_API void axhip_gqa_decode_plan(int B, int Hq, int Hkv, int max_len, int *n_splits, int *chunk) {
   const int group = (Hkv > 0 && Hq % Hkv == 0) ? Hq / Hkv : 1;
-  const SplitPlan p = plan_splits(B, Hq / heads_per_workgroup(group), max_len);
+  // (as for fp16 and D <= 128; other launches of groups >= 4 use heads_per_workgroup)
+  const int G = (g_tuning.mfma_groups && group >= 4) ? mfma_heads_per_workgroup(group) : heads_per_workgroup(group);
+  const SplitPlan p = plan_splits(B, Hq / G, max_len);
   if (n_splits) *n_splits = p.n_splits;
   if (chunk) *chunk = p.chunk;
 }

@@ -181,7 +181,8 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
  * a sequence merges its ranges.
  * Measurement hook: target_workgroups = workgroups to keep streaming (default 256, one per CU; a negative
  * value selects a second merge kernel for a forced split count), force_splits > 0 cuts every sequence into
- * that many ranges; 0 restores the defaults.  No reference counterpart (the reference hard-codes
+ * that many ranges (+ 1000: head groups of four and more stay on the vector ALUs instead of the matrix cores,
+ * for comparison); 0 restores the defaults.  No reference counterpart (the reference hard-codes
  * min(256, ceil(L/64)), gqa.cu:158-160). */
 AXHIP_API void axhip_gqa_decode_plan(int B, int Hq, int Hkv, int max_len, int *n_splits, int *chunk);
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);

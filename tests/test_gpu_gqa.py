@@ -104,6 +104,44 @@ def test_head_shapes(hq, hkv, d):
         assert np.abs(out - want).max() <= tol
 
 
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (32, 4, 128), (64, 8, 128), (28, 4, 128), (40, 2, 64), (16, 4, 64)])
+def test_large_head_groups_on_the_matrix_cores(hq, hkv, d):
+    """Four and more query heads per kv head (fp16): the heads are the columns of an MFMA tile.  Group
+    sizes 4, 8, 7 (not a power of two), 20 (two workgroups of 10 heads per kv head); lengths that are
+    not multiples of the 32 keys of a wavefront or the 128 of a stage, a single key, an empty sequence;
+    the reference's (L, Hkv, D) layout; cut into ranges in one launch and in two; and against the vector
+    path on the same inputs."""
+    rng = np.random.default_rng(hq * 7 + hkv + d)
+    Lmax = 1500
+    lens = np.array([1500, 0, 1, 33, 127, 129, 1279, 640], np.int32)
+    B = len(lens)
+    q = rng.standard_normal((B, hq, d)).astype(np.float32).astype(np.float16)
+    k = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
+    v = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(np.float16)
+    want = port.gqa_decode_cache_native(q, k, v, lens)
+    l = lib()
+    outs = {}
+    try:
+        for name, tune in (("default", (0, 0)), ("3 ranges", (0, 3)), ("3 ranges, merge kernel", (-1, 3)),
+                           ("vector path", (0, 1000))):
+            l.axhip_gqa_decode_tune(*tune)
+            outs[name] = gqa_decode(q, k, v, lens).astype(np.float32)
+    finally:
+        l.axhip_gqa_decode_tune(0, 0)
+    for name, out in outs.items():
+        assert np.abs(out - want).max() <= TOL16, name
+        assert np.all(out[1] == 0), name
+    # the matrix-core path rounds the probabilities to fp16 before the second product; the vector path does not
+    assert np.abs(outs["default"] - outs["vector path"]).max() <= TOL16
+    # the reference's call: one sequence, k/v (L, Hkv, D)
+    L = 700
+    q1 = rng.standard_normal((1, hq, d)).astype(np.float32).astype(np.float16)
+    k1 = rng.standard_normal((L, hkv, d)).astype(np.float32).astype(np.float16)
+    v1 = rng.standard_normal((L, hkv, d)).astype(np.float32).astype(np.float16)
+    np.testing.assert_allclose(gqa_decode(q1, k1, v1, layout="ref").astype(np.float32), port.gqa_decode(q1, k1, v1),
+                               rtol=0, atol=TOL16)
+
+
 def test_result_independent_of_split_count():
     rng = np.random.default_rng(5)
     q, k, v = _qkv_ref(rng, 5000)

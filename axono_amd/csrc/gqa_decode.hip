@@ -668,19 +668,30 @@ __device__ __forceinline__ void finish_range(const DecodeArgs &a, int b, int hg,
 constexpr int kMfmaStage = 128;  // keys per LDS stage (32 per wavefront)
 constexpr int kMfmaHeads = 16;   // columns of the MFMA tile: heads per workgroup at most
 
+// Decode-step form (QKV): the query heads are prepared (RMSNorm, M-RoPE) into LDS by the wavefronts
+// before the first stage is stored there; the workgroup whose range ends with the token being decoded
+// prepares its key and value as well, keeps them in two rows of LDS behind the stage, attends to them in
+// one more step after the cached keys, and writes the cache row.
+extern __shared__ __attribute__((aligned(16))) unsigned char mfma_smem[];
+
 template <int D>
+constexpr int mfma_lds_bytes() {
+  // one stage of K and of V (the per-wavefront states reuse it), two rows for a new token, the merge flag
+  return 2 * kMfmaStage * D * 2 + 2 * D * 2 + 16;
+}
+
+template <int D, bool QKV>
 __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, int hg, int split, int n_valid,
                                                    bool direct_ok, int s0, int s1) {
   constexpr int KK = D / 32;   // MFMA steps over d for S^T
   constexpr int DT = D / 16;   // d tiles of O^T
   constexpr int UPR = D / 8;   // 16-byte units per K/V row
   constexpr int VEC = kMfmaStage * UPR / kThreads;  // staging vectors per thread and tensor
-  // one stage of K and of V; once the keys are done, the four per-wavefront states live in the same memory
-  constexpr int kStateFloats = kMfmaHeads * 4 * (D + 2) + 1;  // + the merge flag
   constexpr int kStageHalves = kMfmaStage * D;
-  constexpr int kLdsBytes = 2 * kStageHalves * 2 > kStateFloats * 4 ? 2 * kStageHalves * 2 : kStateFloats * 4;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[kLdsBytes];
+  static_assert(kMfmaHeads * 4 * (D + 2) * 4 <= 2 * kStageHalves * 2, "the merge states fit the stage memory");
+  unsigned char *smem = mfma_smem;
   _Float16 *ks = reinterpret_cast<_Float16 *>(smem), *vs = ks + kStageHalves;
+  _Float16 *s_new = vs + kStageHalves;  // [2][D]: key and value of the token being decoded
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int c = lane & 15, g = lane >> 4;
@@ -688,17 +699,15 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
   const int h0 = hg * heads;
   const int hk = h0 / a.group;
 
-  // Q as the B operand: column c is head h0 + c (columns past the last head are zero and never stored)
-  half8_t qf[KK];
-  {
-    const __half *qrow = static_cast<const __half *>(a.q) + (static_cast<int64_t>(b) * a.Hq + h0 + min(c, heads - 1)) * D;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      qf[kk] = *reinterpret_cast<const half8_t *>(qrow + kk * 32 + g * 8);
-      if (c >= heads) qf[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    }
+  bool mine = false;
+  int kv_end = s1;  // keys [s0, kv_end) come from the cache
+  int p_new = 0;
+  if constexpr (QKV) {
+    p_new = a.seq_lens[b];
+    p_new = p_new < 0 ? 0 : p_new;
+    mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
+    if (mine) kv_end = p_new;
   }
-
   const __half *kbase = static_cast<const __half *>(a.k) + b * a.stride_b + hk * a.stride_h;
   const __half *vbase = static_cast<const __half *>(a.v) + b * a.stride_b + hk * a.stride_h;
   // one stage waits in registers while the previous one is used from LDS.  (Two stages in registers
@@ -710,7 +719,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
     for (int p = 0; p < VEC; ++p) {
       const int vi = p * kThreads + tid;
       const int row = vi / UPR, unit = vi % UPR;
-      const int64_t off = static_cast<int64_t>(min(key0 + row, s1 - 1)) * a.stride_s + unit * 8;  // rows past the range: its last key again
+      const int64_t off = static_cast<int64_t>(min(key0 + row, kv_end - 1)) * a.stride_s + unit * 8;  // rows past the range: its last key again
       kr[p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(kbase + off));
       vr[p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(vbase + off));
     }
@@ -724,7 +733,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
       const int o = row * D + ((unit ^ (row & (UPR - 1))) << 3);
       *reinterpret_cast<half8_t *>(&ks[o]) = kr[p];
       half8_t vv = vr[p];
-      if (key0 + row >= s1) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (key0 + row >= kv_end) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
       *reinterpret_cast<half8_t *>(&vs[o]) = vv;
     }
   };
@@ -734,76 +743,135 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int n_stages = (s1 - s0 + kMfmaStage - 1) / kMfmaStage;
-  auto do_stage = [&](int st, half8_t (&kr)[VEC], half8_t (&vr)[VEC]) __attribute__((always_inline)) {
-    const int key0 = s0 + st * kMfmaStage;
-    store_stage(key0, kr, vr);
-    __syncthreads();
-    // the next stage into the registers just emptied; the last stage fetches itself again: no branch
-    load_stage(s0 + min(st + 1, n_stages - 1) * kMfmaStage, kr, vr);
-    __builtin_amdgcn_sched_barrier(0);
-    const int kb = key0 + wave * 32;  // first of this wavefront's 32 keys
-    if (kb < s1) {
-      const _Float16 *k_l = ks + wave * 32 * D;
-      float4_t sc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk)
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-          const int row = tk * 16 + c, unit = kk * 4 + g;
-          const half8_t kf = lds_h8(k_l + row * D + ((unit ^ (row & (UPR - 1))) << 3));
-          sc[tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[kk], sc[tk], 0, 0, 0);
+  const int n_stages = (kv_end - s0 + kMfmaStage - 1) / kMfmaStage;
+  // the first stage is requested before the queries are prepared: those loads do not need them
+  if (n_stages > 0) load_stage(s0, kst[0], vst[0]);
+
+  // Q as the B operand: column c is head h0 + c (columns past the last head are zero and never stored)
+  half8_t qf[KK];
+  if constexpr (QKV) {
+    _Float16 *s_q = ks;  // [heads][D], gone once the first stage is stored
+    const bool writer = mine && (h0 % a.group == 0);
+    for (int job = wave; job < heads + (mine ? 2 : 0); job += kThreads / 64) {
+      if (job < heads) {
+        norm_rope_row<__half, D>(a, a.pq + b * a.pq_stride + static_cast<int64_t>(h0 + job) * D, a.qw, b, a.B, lane,
+                                 reinterpret_cast<__half *>(s_q + job * D), static_cast<__half *>(nullptr));
+      } else {
+        __half *crow = const_cast<__half *>(static_cast<const __half *>(job == heads ? a.k : a.v)) + b * a.stride_b +
+                       hk * a.stride_h + static_cast<int64_t>(p_new) * a.stride_s;
+        if (job == heads) {
+          norm_rope_row<__half, D>(a, a.pk + b * a.pk_stride + static_cast<int64_t>(hk) * D, a.kw, b, a.B, lane,
+                                   reinterpret_cast<__half *>(s_new), writer ? crow : static_cast<__half *>(nullptr));
+        } else {
+          const float *src = a.pv + b * a.pv_stride + static_cast<int64_t>(hk) * D;
+          for (int i = lane; i < D; i += 64) {
+            stf(reinterpret_cast<__half *>(s_new + D) + i, src[i]);
+            if (writer) stf(crow + i, src[i]);
+          }
         }
-      // this lane: head c, keys kb + 16 tk + 4 g + e
-      const bool tail = kb + 32 > s1;
-      float x[8];
-#pragma unroll
-      for (int tk = 0; tk < 2; ++tk)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float v = sc[tk][e] * a.scale_log2e;
-          if (tail && kb + tk * 16 + 4 * g + e >= s1) v = kNegBig;
-          x[tk * 4 + e] = v;
-        }
-      float mx = x[0];
-#pragma unroll
-      for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float mn = fmaxf(m, mx);
-      half8_t pf;
-      float ps = 0.f;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float pr = __builtin_amdgcn_exp2f(x[j] - mn);
-        if (tail && x[j] <= kNegBig) pr = 0.f;
-        ps += pr;
-        pf[j] = static_cast<_Float16>(pr);
-      }
-      if (__any(mn != m)) {
-        const float corr = __builtin_amdgcn_exp2f(m - mn);
-        lsum *= corr;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
-      }
-      m = mn;
-      lsum += ps;
-      const _Float16 *v_l = vs + wave * 32 * D;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const half4_t lo = lds_v_tr<D>(v_l, 4 * g, dt * 16, c);
-        const half4_t hi = lds_v_tr<D>(v_l, 16 + 4 * g, dt * 16, c);
-        const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
       }
     }
-    __syncthreads();  // every wavefront is done with the stage before the next one overwrites it
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qf[kk] = lds_h8(s_q + min(c, heads - 1) * D + kk * 32 + g * 8);
+      if (c >= heads) qf[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    __syncthreads();  // everyone has its fragments before the first stage overwrites the rows
+  } else {
+    const __half *qrow = static_cast<const __half *>(a.q) + (static_cast<int64_t>(b) * a.Hq + h0 + min(c, heads - 1)) * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qf[kk] = *reinterpret_cast<const half8_t *>(qrow + kk * 32 + g * 8);
+      if (c >= heads) qf[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+
+  // one wavefront's 32 keys kb .. kb + 31 (those below `limit` count), rows k_l / v_l of the stage in LDS
+  auto attend = [&](int kb, int limit, const _Float16 *k_l, const _Float16 *v_l) __attribute__((always_inline)) {
+    float4_t sc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const int row = tk * 16 + c, unit = kk * 4 + g;
+        const half8_t kf = lds_h8(k_l + row * D + ((unit ^ (row & (UPR - 1))) << 3));
+        sc[tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[kk], sc[tk], 0, 0, 0);
+      }
+    // this lane: head c, keys kb + 16 tk + 4 g + e
+    const bool tail = kb + 32 > limit;
+    float x[8];
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = sc[tk][e] * a.scale_log2e;
+        if (tail && kb + tk * 16 + 4 * g + e >= limit) v = kNegBig;
+        x[tk * 4 + e] = v;
+      }
+    float mx = x[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    half8_t pf;
+    float ps = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float pr = __builtin_amdgcn_exp2f(x[j] - mn);
+      if (tail && x[j] <= kNegBig) pr = 0.f;
+      ps += pr;
+      pf[j] = static_cast<_Float16>(pr);
+    }
+    if (__any(mn != m)) {
+      const float corr = __builtin_amdgcn_exp2f(m - mn);
+      lsum *= corr;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
+    }
+    m = mn;
+    lsum += ps;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const half4_t lo = lds_v_tr<D>(v_l, 4 * g, dt * 16, c);
+      const half4_t hi = lds_v_tr<D>(v_l, 16 + 4 * g, dt * 16, c);
+      const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
+    }
   };
-  load_stage(s0, kst[0], vst[0]);
-  for (int st = 0; st < n_stages; ++st) do_stage(st, kst[0], vst[0]);
+  for (int st = 0; st < n_stages; ++st) {
+    const int key0 = s0 + st * kMfmaStage;
+    store_stage(key0, kst[0], vst[0]);
+    __syncthreads();
+    // the next stage into the registers just emptied; the last stage fetches itself again: no branch
+    load_stage(s0 + min(st + 1, n_stages - 1) * kMfmaStage, kst[0], vst[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    const int kb = key0 + wave * 32;  // first of this wavefront's 32 keys
+    if (kb < kv_end) attend(kb, kv_end, ks + wave * 32 * D, vs + wave * 32 * D);
+    __syncthreads();  // every wavefront is done with the stage before the next one overwrites it
+  }
+  if constexpr (QKV) {
+    if (mine) {
+      // the token being decoded: its key and value become row 0 of a stage of their own (row 0 is not
+      // swizzled; the other rows hold finite leftovers that the mask keeps out)
+      if (n_stages == 0) {
+        for (int i = tid; i < 2 * kStageHalves / 8; i += kThreads)
+          *reinterpret_cast<half8_t *>(ks + i * 8) = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        __syncthreads();
+      }
+      if (tid < UPR) *reinterpret_cast<half8_t *>(ks + tid * 8) = *reinterpret_cast<const half8_t *>(s_new + tid * 8);
+      else if (tid < 2 * UPR)
+        *reinterpret_cast<half8_t *>(vs + (tid - UPR) * 8) = *reinterpret_cast<const half8_t *>(s_new + D + (tid - UPR) * 8);
+      __syncthreads();
+      if (wave == 0) attend(p_new, p_new + 1, ks, vs);
+      __syncthreads();
+    }
+  }
 
   // the four per-wavefront states, [head][wavefront]: maximum, sum, output
   float *s_m = reinterpret_cast<float *>(smem), *s_l = s_m + kMfmaHeads * 4, *s_acc = s_l + kMfmaHeads * 4;
+  int *s_flag = reinterpret_cast<int *>(smem + 2 * kStageHalves * 2 + 2 * D * 2);
   lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
   if (g == 0) {
@@ -815,7 +883,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
     *reinterpret_cast<float4_t *>(&s_acc[(c * 4 + wave) * D + dt * 16 + 4 * g]) = o[dt];
   __syncthreads();
   finish_range<__half, D, 4>(a, b, hg, h0, heads, split, n_valid, direct_ok, (lds_cfloat_ptr)s_m, (lds_cfloat_ptr)s_l,
-                             (lds_cfloat_ptr)s_acc, (lds_int_ptr)(s_acc + kMfmaHeads * 4 * D));
+                             (lds_cfloat_ptr)s_acc, (lds_int_ptr)s_flag);
 }
 
 // Which keys a workgroup streams.
@@ -899,7 +967,7 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
         const int first_slot = start_b / cc, last_slot = (start_b + len_b - 1) / cc;
         if (again) __syncthreads();  // the previous piece is done with the LDS arrays
         if constexpr (MFMA)
-          process_range_mfma<D>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true, max(g0 - start_b, 0),
+          process_range_mfma<D, QKV>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true, max(g0 - start_b, 0),
                                 min(g1 - start_b, len_b));
         else
           process_range<T, D, G, U, QKV, false>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
@@ -930,7 +998,7 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
     }
   }
   if constexpr (MFMA)
-    process_range_mfma<D>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+    process_range_mfma<D, QKV>(a, b, hg, split, n_valid, direct_ok, s0, s1);
   else
     process_range<T, D, G, U, QKV, true>(a, b, hg, split, n_valid, direct_ok, s0, s1);
 }
@@ -975,14 +1043,30 @@ int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   return launch_status();
 }
 
-template <int D>
-int launch_decode_mfma(const DecodeArgs &a, int B, hipStream_t st) {
+template <int D, bool QKV>
+int launch_decode_mfma_form(const DecodeArgs &a, int B, hipStream_t st) {
   const int n_hg = a.n_hg;
   const dim3 grid(a.dynamic ? a.active * n_hg : a.n_splits, a.dynamic ? 1 : n_hg, a.dynamic ? 1 : B);
-  hipLaunchKernelGGL((gqa_decode_split_kernel<__half, D, 1, 8, false, true>), grid, dim3(kThreads), 0, st, a);
+  auto kernel = gqa_decode_split_kernel<__half, D, 1, 8, QKV, true>;
+  constexpr int lds = mfma_lds_bytes<D>();
+  if (lds > 64 * 1024) {  // more dynamic LDS than the default limit: raised once per process and kernel
+    static bool lds_set = false;
+    if (!lds_set) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
+          hipSuccess)
+        return AXHIP_INTERNAL_ERROR;
+      lds_set = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, a);
   if (a.n_splits > 1 && !a.fused_merge)
     hipLaunchKernelGGL((gqa_decode_merge_kernel<__half, D>), dim3(a.Hq, B), dim3(D), 0, st, a);
   return launch_status();
+}
+
+template <int D>
+int launch_decode_mfma(const DecodeArgs &a, int B, hipStream_t st) {
+  return a.len_add ? launch_decode_mfma_form<D, true>(a, B, st) : launch_decode_mfma_form<D, false>(a, B, st);
 }
 
 template <typename T, int D>
@@ -1024,8 +1108,8 @@ namespace {
 int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int dtype, int B, int Hq, int Hkv,
                     int D, int max_len, axhip_stream stream) {
   const int group = Hq / Hkv;
-  // four or more heads per kv head, fp16, plain form: the heads of a kv head become the columns of an MFMA tile
-  const bool mfma = g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) && !a.len_add &&
+  // four or more heads per kv head, fp16: the heads of a kv head become the columns of an MFMA tile
+  const bool mfma = g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) &&
                     a.stride_s % 8 == 0 && a.stride_h % 8 == 0 && a.stride_b % 8 == 0;
   const int G = mfma ? mfma_heads_per_workgroup(group) : heads_per_workgroup(group);
   a.wg_heads = G;

@@ -15,7 +15,12 @@ CFG = TextConfig(num_hidden_layers=3, hidden_size=256, num_attention_heads=4, nu
                  intermediate_size=512, vocab_size=1000)
 
 
-def _setup(B=3, S=21, max_len=64, seed=0):
+# four query heads per kv head: decode attention (and its decode-step form) on the matrix cores
+CFG4 = TextConfig(num_hidden_layers=2, hidden_size=256, num_attention_heads=8, num_key_value_heads=2, head_dim=128,
+                  intermediate_size=512, vocab_size=1000)
+
+
+def _setup(B=3, S=21, max_len=64, seed=0, CFG=CFG):
     w = random_weights(CFG, seed)
     # non-trivial norm weights so a dropped weight would show
     rng = np.random.default_rng(seed + 1)
@@ -141,3 +146,29 @@ def test_persistent_layer_tail_path_matches_oracle_and_replays():
     t_logits, _ = gpu.decode_forward(gpu._ids, gpu._pos)
     err_paths = float(np.abs(t_logits.to_numpy() - d_logits).max())
     assert err_paths <= 2e-3 + 1e-3 * float(np.abs(d_logits).max()), err_paths
+
+
+def test_decode_steps_match_oracle_with_four_heads_per_kv_head():
+    """The captured step of a model whose attention runs on the matrix-core decode path (group size 4)."""
+    gpu, cpu, ids = _setup(seed=11, CFG=CFG4)
+    B, S = ids.shape
+    g_logits, g_next = gpu.prefill(ids)
+    c_logits, _ = cpu.prefill(ids)
+    assert np.abs(g_logits.to_numpy() - c_logits).max() <= 2e-3
+    first = g_next.to_numpy()
+    pos = np.full((3, B), S, np.int64)
+    n_steps = 5
+    gpu.start_decode(first, pos, n_steps)
+    gpu.capture()
+    toks = gpu.generate(n_steps, use_graph=True)
+    cur = first
+    for s in range(n_steps):
+        logits, _ = cpu.decode_step(cur, pos + s)
+        chosen = logits[np.arange(B), toks[s]]
+        assert np.all(chosen >= logits.max(-1) - 4e-3), (s, chosen, logits.max(-1))
+        cur = toks[s]
+    for i in range(CFG4.num_hidden_layers):
+        kc, vc = gpu.cache.get(i)
+        n = S + n_steps
+        assert np.abs(kc.numpy()[:, :, :n].astype(np.float32) - cpu.k[i][:, :, :n].astype(np.float32)).max() <= 4e-3
+        assert np.abs(vc.numpy()[:, :, :n].astype(np.float32) - cpu.v[i][:, :, :n].astype(np.float32)).max() <= 4e-3

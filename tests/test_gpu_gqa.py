@@ -313,7 +313,7 @@ def _check_decode_step_form(Hq, Hkv, D, lens, rows, max_len, forced=(0, 5), seed
     return dq, dp, di, dl, dkc, dvc, out, ws, wsb, width, hw
 
 
-@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (8, 1, 64), (3, 3, 256)])
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (8, 1, 64), (3, 3, 256), (8, 2, 128), (20, 1, 128), (32, 4, 64)])
 def test_decode_step_form_equals_append_then_attention(Hq, Hkv, D):
     """axhip_gqa_decode_qkv (q/k norm + M-RoPE + append + attention in the split kernel) against the
     oracle's rms_norm -> rope_thd -> fp16 rounding -> append -> attention over len + 1 keys; sequences
@@ -342,6 +342,8 @@ def test_decode_step_form_ragged_batch_with_one_workgroup_per_sequence_to_share(
     lens[[1, 8]] = [max_len, max_len - 1]
     lens[[2, 3]] = [1, 127]
     _check_decode_step_form(16, 8, 128, lens, max_len + 8, max_len, forced=(0,), seed=6)
+    # the same with four heads per kv head (the matrix-core path)
+    _check_decode_step_form(16, 4, 128, lens, max_len + 8, max_len, forced=(0,), seed=7)
 
 
 @pytest.mark.parametrize("Hq,Hkv,D,S,start", [(4, 2, 128, 200, [0, 37]), (2, 2, 128, 64, [0, 0]), (8, 2, 64, 130, [5, 300]),

@@ -247,7 +247,8 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "copy", "rowops", "linear", "linear-packed", "prefill-attn", "tail"])
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "copy", "rowops", "linear", "linear-packed", "prefill-attn",
+                                     "tail"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -278,6 +279,11 @@ def main(argv=None):
         bench_gqa(lib, 32, 32768, 20, lens, tag="gqa_ragged_512_32768")
     elif args.what == "tail":
         bench_tail(lib, args.steps)
+    elif args.what == "gqa-shapes":
+        # other head shapes: group sizes 1, 4 and 8 (four and more run on the matrix cores), D = 64 and 256
+        for Hq, Hkv, D in ((8, 8, 128), (32, 8, 128), (64, 8, 128), (32, 4, 128), (32, 8, 64), (16, 8, 64), (16, 8, 256)):
+            for B, L in ((32, 8192), (16, 4160), (4, 8192), (1, 32768)):
+                bench_gqa(lib, B, L, min(args.steps, 50), Hq=Hq, Hkv=Hkv, D=D, tag=f"gqa_Hq{Hq}_Hkv{Hkv}_D{D}")
     elif args.what == "prefill-attn":
         for S in (1024, 4096, 16384):
             bench_prefill_attn(lib, max(1, min(args.B, 65536 // S)), S, max(5, min(args.steps, 20)))

@@ -30,77 +30,93 @@ __device__ __forceinline__ float wload(const void *w, int f16, int i) {
   return f16 ? __half2float(static_cast<const __half *>(w)[i]) : static_cast<const float *>(w)[i];
 }
 
-// One wavefront per (sequence, head) row; heads [0,Hq) are q, [Hq,Hq+Hkv) are k, the rest v.
+// One wavefront per token and group of `hpw` consecutive heads; heads [0,Hq) are q, [Hq,Hq+Hkv) are k,
+// the rest v.  The rotation angles depend on the token and the pair only, so a wavefront computes its
+// sincosf values once and applies them to every q / k head of its group (with many tokens hpw grows,
+// up to 8: the accurate sincosf is most of this kernel's arithmetic).
 // PAIRS = ceil(D/2/64): rotate-half pairs (i, i + D/2) owned by each lane.
 template <typename CT, int PAIRS>
-__global__ __launch_bounds__(kBlock) void qkv_norm_rope_append_kernel(QkvArgs a) {
+__global__ __launch_bounds__(kBlock) void qkv_norm_rope_append_kernel(QkvArgs a, int hpw) {
   const int lane = threadIdx.x & 63;
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
+  const int64_t unit = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
   const int heads = a.Hq + 2 * a.Hkv;
+  const int groups = (heads + hpw - 1) / hpw;
   const int64_t tokens = static_cast<int64_t>(a.B) * a.S;
-  if (row >= tokens * heads) return;  // whole wavefront leaves together
-  const int64_t r = row / heads;      // token
-  const int h = static_cast<int>(row % heads);
+  if (unit >= tokens * groups) return;  // whole wavefront leaves together
+  const int64_t r = unit / groups;      // token
+  const int h_begin = static_cast<int>(unit % groups) * hpw, h_end = min(h_begin + hpw, heads);
   const int b = static_cast<int>(r / a.S);
   const int half = a.D / 2;
   const int64_t len = (a.seq_lens ? a.seq_lens[b] : 0) + r % a.S;  // append position of this token
   const bool can_append = len >= 0 && len < a.Lmax;
 
-  if (h >= a.Hq + a.Hkv) {  // v: convert and append
-    if (!can_append) return;
-    const int hv = h - a.Hq - a.Hkv;
-    const float *src = a.v + r * a.v_stride + static_cast<int64_t>(hv) * a.D;
-    CT *dst = static_cast<CT *>(a.v_cache) + ((static_cast<int64_t>(b) * a.Hkv + hv) * a.Lmax + len) * a.D;
-    for (int i = lane; i < a.D; i += 64) stf(dst + i, src[i]);
-    return;
-  }
-  const bool is_q = h < a.Hq;
-  const int hh = is_q ? h : h - a.Hq;
-  const float *src = is_q ? a.q + r * a.q_stride + static_cast<int64_t>(hh) * a.D
-                          : a.k + r * a.k_stride + static_cast<int64_t>(hh) * a.D;
-  const void *w = is_q ? a.qw : a.kw;
-  float lo[PAIRS], hi[PAIRS];
-  float ss = 0.f;
+  float cs[PAIRS], sn[PAIRS];
+  if (h_begin < a.Hq + a.Hkv) {  // some head of this group is rotated
+    const float pt = static_cast<float>(a.pos[r]);
+    const float ph = static_cast<float>(a.pos[tokens + r]);
+    const float pw = static_cast<float>(a.pos[2 * tokens + r]);
 #pragma unroll
-  for (int p = 0; p < PAIRS; ++p) {
-    const int i = lane + p * 64;
-    lo[p] = i < half ? src[i] : 0.f;
-    hi[p] = i < half ? src[i + half] : 0.f;
-    ss = __builtin_fmaf(lo[p], lo[p], ss);
-    ss = __builtin_fmaf(hi[p], hi[p], ss);
-  }
-  ss = group_sum<64>(ss);
-  const float inv = 1.0f / sqrtf(ss / static_cast<float>(a.D) + a.eps);
-  const float pt = static_cast<float>(a.pos[r]);
-  const float ph = static_cast<float>(a.pos[tokens + r]);
-  const float pw = static_cast<float>(a.pos[2 * tokens + r]);
-  CT *dst;
-  if (is_q) {
-    dst = static_cast<CT *>(a.q_out) + (r * a.Hq + hh) * a.D;
-  } else {
-    if (!can_append) return;
-    dst = static_cast<CT *>(a.k_cache) + ((static_cast<int64_t>(b) * a.Hkv + hh) * a.Lmax + len) * a.D;
-  }
-#pragma unroll
-  for (int p = 0; p < PAIRS; ++p) {
-    const int i = lane + p * 64;
-    if (i >= half) continue;
-    // same evaluation order as rms_norm then rope_thd: (x * inv) * w, then the rotation
-    float x0 = lo[p] * inv, x1 = hi[p] * inv;
-    if (w) {
-      x0 *= wload(w, a.w_f16, i);
-      x1 *= wload(w, a.w_f16, i + half);
+    for (int p = 0; p < PAIRS; ++p) {
+      const int i = lane + p * 64;
+      cs[p] = 1.f;
+      sn[p] = 0.f;
+      if (i >= half) continue;
+      const float f = a.inv_freq[i];
+      float ang = pt * f;
+      if (i % 3 == 1 && i < a.h_lim)
+        ang = ph * f;
+      else if (i % 3 == 2 && i < a.w_lim)
+        ang = pw * f;
+      sincosf(ang, &sn[p], &cs[p]);
     }
-    const float f = a.inv_freq[i];
-    float ang = pt * f;
-    if (i % 3 == 1 && i < a.h_lim)
-      ang = ph * f;
-    else if (i % 3 == 2 && i < a.w_lim)
-      ang = pw * f;
-    float s, c;
-    sincosf(ang, &s, &c);
-    stf(dst + i, x0 * c - x1 * s);
-    stf(dst + i + half, x1 * c + x0 * s);
+  }
+
+  for (int h = h_begin; h < h_end; ++h) {
+    if (h >= a.Hq + a.Hkv) {  // v: convert and append
+      if (!can_append) continue;
+      const int hv = h - a.Hq - a.Hkv;
+      const float *src = a.v + r * a.v_stride + static_cast<int64_t>(hv) * a.D;
+      CT *dst = static_cast<CT *>(a.v_cache) + ((static_cast<int64_t>(b) * a.Hkv + hv) * a.Lmax + len) * a.D;
+      for (int i = lane; i < a.D; i += 64) stf(dst + i, src[i]);
+      continue;
+    }
+    const bool is_q = h < a.Hq;
+    const int hh = is_q ? h : h - a.Hq;
+    const float *src = is_q ? a.q + r * a.q_stride + static_cast<int64_t>(hh) * a.D
+                            : a.k + r * a.k_stride + static_cast<int64_t>(hh) * a.D;
+    const void *w = is_q ? a.qw : a.kw;
+    float lo[PAIRS], hi[PAIRS];
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+      const int i = lane + p * 64;
+      lo[p] = i < half ? src[i] : 0.f;
+      hi[p] = i < half ? src[i + half] : 0.f;
+      ss = __builtin_fmaf(lo[p], lo[p], ss);
+      ss = __builtin_fmaf(hi[p], hi[p], ss);
+    }
+    ss = group_sum<64>(ss);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(a.D) + a.eps);
+    CT *dst;
+    if (is_q) {
+      dst = static_cast<CT *>(a.q_out) + (r * a.Hq + hh) * a.D;
+    } else {
+      if (!can_append) continue;
+      dst = static_cast<CT *>(a.k_cache) + ((static_cast<int64_t>(b) * a.Hkv + hh) * a.Lmax + len) * a.D;
+    }
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+      const int i = lane + p * 64;
+      if (i >= half) continue;
+      // same evaluation order as rms_norm then rope_thd: (x * inv) * w, then the rotation
+      float x0 = lo[p] * inv, x1 = hi[p] * inv;
+      if (w) {
+        x0 *= wload(w, a.w_f16, i);
+        x1 *= wload(w, a.w_f16, i + half);
+      }
+      stf(dst + i, x0 * cs[p] - x1 * sn[p]);
+      stf(dst + i + half, x1 * cs[p] + x0 * sn[p]);
+    }
   }
 }
 
@@ -214,7 +230,11 @@ AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const
     return AXHIP_INVALID_PTR;
   QkvArgs a{q, k, v, q_stride, k_stride, v_stride, q_weight, k_weight, w_dtype == AXHIP_FLOAT16, eps,
             pos, inv_freq, h_sec * 3, w_sec * 3, seq_lens, q_out, k_cache, v_cache, B, Hq, Hkv, D, Lmax, S};
-  const int64_t rows = static_cast<int64_t>(B) * S * (Hq + 2 * Hkv);
+  // heads per wavefront: as many (up to 8) as still leave 16384 wavefronts
+  const int heads = Hq + 2 * Hkv;
+  int hpw = 1;
+  while (hpw < 8 && static_cast<int64_t>(B) * S * ((heads + 2 * hpw - 1) / (2 * hpw)) >= 16384) hpw *= 2;
+  const int64_t rows = static_cast<int64_t>(B) * S * ((heads + hpw - 1) / hpw);
   const dim3 grid(static_cast<unsigned>((rows + kBlock / 64 - 1) / (kBlock / 64)));
   hipStream_t st = as_stream(stream);
   const int pairs = (D / 2 + 63) / 64;
@@ -222,9 +242,9 @@ AXHIP_API int axhip_qkv_norm_rope_append(const float *q, int64_t q_stride, const
 #define AXHIP_QKV_LAUNCH(P)                                                                          \
   do {                                                                                               \
     if (f16)                                                                                         \
-      hipLaunchKernelGGL((qkv_norm_rope_append_kernel<__half, P>), grid, dim3(kBlock), 0, st, a);    \
+      hipLaunchKernelGGL((qkv_norm_rope_append_kernel<__half, P>), grid, dim3(kBlock), 0, st, a, hpw); \
     else                                                                                             \
-      hipLaunchKernelGGL((qkv_norm_rope_append_kernel<float, P>), grid, dim3(kBlock), 0, st, a);     \
+      hipLaunchKernelGGL((qkv_norm_rope_append_kernel<float, P>), grid, dim3(kBlock), 0, st, a, hpw);  \
   } while (0)
   switch (pairs) {
     case 1: AXHIP_QKV_LAUNCH(1); break;

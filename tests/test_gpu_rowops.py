@@ -284,10 +284,14 @@ def test_fp16_output_variants_round_once():
     assert gu.lib().axhip_silu_mul_fused(dg.ptr, o_f32.ptr, gu.F16, gu.F32, 16, 6144, None) == 3  # fp16 in, fp32 out: refused
 
 
-def test_qkv_norm_rope_append_equals_op_composition():
-    """The fused decode glue against rms_norm -> rope_thd -> round to fp16 -> append of the oracle."""
+@pytest.mark.parametrize("B,S,nq,nkv,lmax,lens", [(3, 2, 4, 2, 16, [5, 0, 13]),
+                                                   (1, 4096, 4, 2, 4100, [3]),      # two heads per wavefront
+                                                   (2, 8192, 5, 1, 8200, [0, 8])])  # q, k and v heads in one wavefront
+def test_qkv_norm_rope_append_equals_op_composition(B, S, nq, nkv, lmax, lens):
+    """The fused glue against rms_norm -> rope_thd -> round to fp16 -> append of the oracle; with many
+    tokens a wavefront takes several heads of a token with one set of rotation angles."""
     rng = np.random.default_rng(31)
-    B, S, nq, nkv, D, lmax = 3, 2, 4, 2, 128, 16
+    D = 128
     T = B * S
     width = (nq + 2 * nkv) * D
     qkv = rng.standard_normal((T, width)).astype(np.float32)
@@ -295,7 +299,7 @@ def test_qkv_norm_rope_append_equals_op_composition():
     kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
     pos = rng.integers(0, 8192, (3, T)).astype(np.int64)
     inv = port.rope_inv_freq(1e6, D)
-    lens = np.array([5, 0, 13], np.int32)
+    lens = np.array(lens, np.int32)
     kc = rng.standard_normal((B, nkv, lmax, D)).astype(np.float16)
     vc = rng.standard_normal((B, nkv, lmax, D)).astype(np.float16)
     dq, dqw, dkw, dp, di, dl, dkc, dvc = (gu.dev(a) for a in (qkv, qw, kw, pos, inv, lens, kc, vc))

@@ -111,6 +111,22 @@ def bench_prefill_attn(lib, B, S, steps, Hq=16, Hkv=8, D=128):
            "TFLOPs": round(fl / us / 1e6, 1), "pct_mfma_f16_peak": round(100 * fl / us / 1e6 / MFMA_F16_PEAK, 2)})
 
 
+def bench_sdpa(lib, S, steps, causal, Hq=16, Hkv=8, D=128):
+    """The general attention entry on token-major q [S,Hq,D] and k/v [S,Hkv,D]."""
+    q, out = DeviceBuffer(S * Hq * D * 2), DeviceBuffer(S * Hq * D * 2)
+    k, v = DeviceBuffer(S * Hkv * D * 2), DeviceBuffer(S * Hkv * D * 2)
+    for i, buf in enumerate((q, k, v)):
+        _rand_fill(buf, buf.nbytes, 200 + i)
+
+    def step():
+        check(lib.axhip_sdpa(q.ptr, k.ptr, v.ptr, out.ptr, F16, S, Hq, Hkv, D, S, int(causal), None), "sdpa")
+
+    us = _time(lib, step, steps)
+    fl = 4.0 * D * Hq * (S * (S + 1) / 2 if causal else S * S)
+    _emit({"op": "sdpa", "S": S, "Hq": Hq, "Hkv": Hkv, "D": D, "causal": bool(causal), "us": round(us, 1),
+           "TFLOPs": round(fl / us / 1e6, 1), "pct_mfma_f16_peak": round(100 * fl / us / 1e6 / MFMA_F16_PEAK, 2)})
+
+
 def bench_tail(lib, steps, M=16, H=2048, K1=2048, I=6144, N_next=4096, rot=8):
     """The persistent layer-tail launch, weights rotated through `rot` copies; with phases skipped one
     by one (timing only) to see where the time goes."""
@@ -287,6 +303,9 @@ def main(argv=None):
     elif args.what == "prefill-attn":
         for S in (1024, 4096, 16384):
             bench_prefill_attn(lib, max(1, min(args.B, 65536 // S)), S, max(5, min(args.steps, 20)))
+        for S in (4096, 16384):
+            for causal in (True, False):
+                bench_sdpa(lib, S, max(5, min(args.steps, 20)), causal)
     elif args.what == "copy":
         bench_copy(lib, args.mib, args.steps)
     elif args.what == "rowops":

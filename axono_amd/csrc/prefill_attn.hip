@@ -41,6 +41,9 @@ struct PrefillArgs {
   __half *out;       // [B, S, Hq, D]
   int S, Hq, Hkv, rows, group;
   float scale_log2e;
+  // general form only (GEN): K/V strides in elements, and whether the causal rule applies
+  int64_t kv_batch_stride, kv_head_stride, kv_row_stride;
+  int causal;
 };
 
 // Up to two query heads per workgroup the kernel is held to 256 registers, so that two workgroups share
@@ -48,7 +51,11 @@ struct PrefillArgs {
 // second wavefront per SIMD fills those gaps (B=1, S=4096: 372 -> 219 us).  Left to itself the
 // compiler takes 296 registers.  Sharing every K/V fragment among two tiles of 16 positions per
 // wavefront instead (half the LDS reads per product, one workgroup per CU) measured slower.
-template <int D, int G>
+//
+// GEN = false is the cache form: K/V rows of a head are contiguous, the rule is causal and every query's
+// position lies inside the cache.  GEN = true takes any row/head/batch stride (token-major K/V), an
+// optional causal rule, and queries whose position is past the last key (they see every key).
+template <int D, int G, bool GEN>
 __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel(PrefillArgs a) {
   constexpr int KK = D / 32;   // MFMA steps over d for S^T
   constexpr int DT = D / 16;   // d tiles of O^T
@@ -65,10 +72,20 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
   const int start = a.start ? max(a.start[b], 0) : 0;
   const int p0 = pb * kPosPerWg;
   const int pr = p0 + wave * 16 + c;           // this lane's query (as B column), relative position
-  const int pos = start + pr;                  // its absolute position = last visible key
-  const int wave_last = start + p0 + wave * 16 + 15;
+  int pos = start + pr;                        // its absolute position = last visible key
+  int wave_first = start + p0 + wave * 16;     // smallest and largest position of this wavefront
+  int wave_last = wave_first + 15;
   int k_end = start + min(p0 + kPosPerWg, a.S);  // keys the workgroup needs: [0, k_end)
   k_end = min(k_end, a.rows);
+  if constexpr (GEN) {
+    if (!a.causal) {
+      pos = wave_first = wave_last = a.rows - 1;
+      k_end = a.rows;
+    } else {
+      pos = min(pos, a.rows - 1);
+      wave_first = min(wave_first, a.rows - 1);
+    }
+  }
 
   // Q fragments stay in registers for the whole kernel
   half8_t qf[G][KK];
@@ -82,15 +99,18 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
         qf[t][kk] = *reinterpret_cast<const half8_t *>(qrow + t * D + kk * 32 + g * 8);
   }
 
-  const __half *kbase = a.k + (static_cast<int64_t>(b) * a.Hkv + hk) * a.rows * D;
-  const __half *vbase = a.v + (static_cast<int64_t>(b) * a.Hkv + hk) * a.rows * D;
+  const int64_t kv_off = GEN ? b * a.kv_batch_stride + hk * a.kv_head_stride
+                             : (static_cast<int64_t>(b) * a.Hkv + hk) * a.rows * D;
+  const int64_t row_stride = GEN ? a.kv_row_stride : D;
+  const __half *kbase = a.k + kv_off;
+  const __half *vbase = a.v + kv_off;
   half8_t kst[VEC], vst[VEC];
   auto load_stage = [&](int key0) {
 #pragma unroll
     for (int p = 0; p < VEC; ++p) {
       const int vi = p * kPThreads + tid;
       const int row = vi / UPR, unit = vi % UPR;
-      const int64_t off = static_cast<int64_t>(min(key0 + row, a.rows - 1)) * D + unit * 8;
+      const int64_t off = static_cast<int64_t>(min(key0 + row, a.rows - 1)) * row_stride + unit * 8;
       kst[p] = *reinterpret_cast<const half8_t *>(kbase + off);
       vst[p] = *reinterpret_cast<const half8_t *>(vbase + off);
     }
@@ -150,7 +170,7 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
               sc[t][tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][kk], sc[t][tk], 0, 0, 0);
           }
         // ---- mask, online softmax ----
-        const bool diag = kb + 31 > start + p0 + wave * 16;  // some key of the block may be masked
+        const bool diag = kb + 31 > wave_first;  // some key of the block may be masked
         half8_t pf[G];
 #pragma unroll
         for (int t = 0; t < G; ++t) {
@@ -226,13 +246,13 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
   }
 }
 
-template <int D>
+template <int D, bool GEN>
 int launch_prefill(const PrefillArgs &a, int B, int G, hipStream_t st) {
   const dim3 grid((a.S + kPosPerWg - 1) / kPosPerWg, a.Hq / G, B);
   switch (G) {
-    case 4: hipLaunchKernelGGL((prefill_attn_kernel<D, 4>), grid, dim3(kPThreads), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((prefill_attn_kernel<D, 2>), grid, dim3(kPThreads), 0, st, a); break;
-    default: hipLaunchKernelGGL((prefill_attn_kernel<D, 1>), grid, dim3(kPThreads), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((prefill_attn_kernel<D, 4, GEN>), grid, dim3(kPThreads), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((prefill_attn_kernel<D, 2, GEN>), grid, dim3(kPThreads), 0, st, a); break;
+    default: hipLaunchKernelGGL((prefill_attn_kernel<D, 1, GEN>), grid, dim3(kPThreads), 0, st, a); break;
   }
   return launch_status();
 }
@@ -272,7 +292,35 @@ AXHIP_API int axhip_prefill_attention(const void *q, const void *k_cache, const 
   a.group = group;
   a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
   hipStream_t st = as_stream(stream);
-  return D == 128 ? launch_prefill<128>(a, B, G, st) : launch_prefill<64>(a, B, G, st);
+  a.kv_batch_stride = a.kv_head_stride = a.kv_row_stride = 0;
+  a.causal = 1;
+  return D == 128 ? launch_prefill<128, false>(a, B, G, st) : launch_prefill<64, false>(a, B, G, st);
+}
+
+// Attention of q [Sq,Hq,D] over token-major k/v [Skv,Hkv,D] (fp16, D 64 or 128, 16-byte aligned) on
+// the matrix cores; row t sees min(t+1, Skv) keys under the causal rule, all Skv otherwise.  The caller
+// has checked shapes and pointers.
+int axhip_internal_sdpa_f16_mfma(const void *q, const void *k, const void *v, void *out, int Sq, int Hq,
+                                 int Hkv, int D, int Skv, int is_causal, hipStream_t st) {
+  const int group = Hq / Hkv;
+  const int G = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  PrefillArgs a;
+  a.q = static_cast<const __half *>(q);
+  a.k = static_cast<const __half *>(k);
+  a.v = static_cast<const __half *>(v);
+  a.start = nullptr;
+  a.out = static_cast<__half *>(out);
+  a.S = Sq;
+  a.Hq = Hq;
+  a.Hkv = Hkv;
+  a.rows = Skv;
+  a.group = group;
+  a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
+  a.kv_batch_stride = 0;
+  a.kv_head_stride = D;
+  a.kv_row_stride = static_cast<int64_t>(Hkv) * D;
+  a.causal = is_causal;
+  return D == 128 ? launch_prefill<128, true>(a, 1, G, st) : launch_prefill<64, true>(a, 1, G, st);
 }
 
 }  // extern "C"

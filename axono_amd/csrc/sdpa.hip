@@ -1,19 +1,23 @@
 // General scaled-dot-product attention (prefill, short contexts): q [Sq,Hq,D], k/v [Skv,Hkv,D].
 //
-// For head sizes the decode kernel supports (64/128/256) every query row is treated as one
-// "sequence" of the split-K decode kernel that shares the same K/V (batch stride 0) and sees
+// fp16 with head size 64 or 128 and at least 32 query rows runs the tiled prefill kernel on the matrix
+// cores.  Otherwise, for head sizes the decode kernel supports (64/128/256) every query row is treated
+// as one "sequence" of the split-K decode kernel that shares the same K/V (batch stride 0) and sees
 // len[t] keys: t+1 under the causal rule, Skv otherwise.  K/V are then re-read per query row, mostly
-// from L2; good enough to fill a cache before the timed decode loop, which is all this path is for.
+// from L2.
 // Other head sizes take a plain three-phase kernel (scores to a workspace, softmax, weighted sum).
 #include "common.hpp"
 
 extern "C" int axhip_internal_fill_zero(void *dst, int64_t n, hipStream_t st);
+extern "C" int axhip_internal_sdpa_f16_mfma(const void *q, const void *k, const void *v, void *out, int Sq,
+                                            int Hq, int Hkv, int D, int Skv, int is_causal, hipStream_t st);
 
 namespace axhip {
 namespace {
 
 constexpr int kBlock = 256;
 constexpr int kRowsPerCall = 32768;  // grid.z limit of the decode launch
+constexpr int kMfmaMinRows = 32;     // fewer query rows than this stay on the split-K decode kernel
 
 __global__ void visible_len_kernel(int32_t *len, int t0, int n, int skv, int causal) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -83,6 +87,13 @@ AXHIP_API int axhip_sdpa(const void *q, const void *k, const void *v, void *out,
   if (!q || !k || !v || !out) return AXHIP_INVALID_PTR;
   hipStream_t st = as_stream(stream);
   const int64_t esz = dtype == AXHIP_FLOAT16 ? 2 : 4;
+
+  // fp16 with enough query rows to fill 16-row tiles: the causal prefill kernel on the matrix cores
+  const uintptr_t ptr_bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+                             reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out);
+  if (dtype == AXHIP_FLOAT16 && (D == 64 || D == 128) && Sq >= kMfmaMinRows && Hq <= 65535 * 4 &&
+      (ptr_bits & 15) == 0)
+    return axhip_internal_sdpa_f16_mfma(q, k, v, out, Sq, Hq, Hkv, D, Skv, is_causal, st);
 
   if (D == 64 || D == 128 || D == 256) {
     const int rows_max = Sq < kRowsPerCall ? Sq : kRowsPerCall;

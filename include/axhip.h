@@ -190,7 +190,10 @@ AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
 /* General attention for prefill and short contexts: q [Sq,Hq,D], k/v [Skv,Hkv,D] contiguous,
  * optional causal mask with the reference's rule (keys 0..t visible when Skv >= t+1).
  * Replaces ops::cuda::ScaledDotProductAttention, src/ops/cuda/sequence.cu:105-163,451-472.
- * Any D up to 256; not tuned (it fills the cache before the timed decode loop). */
+ * fp16 with D 64 or 128, 32 or more query rows and 16-byte aligned pointers runs the tiled
+ * matrix-core kernel of axhip_prefill_attention over the token-major K/V; other fp16/fp32 cases
+ * with D 64/128/256 run the split-K decode kernel with one "sequence" per query row; any other
+ * D takes a plain three-phase kernel. */
 AXHIP_API int axhip_sdpa(const void *q, const void *k, const void *v, void *out, int dtype,
                          int Sq, int Hq, int Hkv, int D, int Skv, int is_causal,
                          axhip_stream stream);

@@ -253,6 +253,23 @@ def test_sdpa_prefill_and_small_heads():
         np.testing.assert_allclose(step[0], full[t], rtol=0, atol=TOL32)
 
 
+@pytest.mark.parametrize("Sq,Skv,Hq,Hkv,D", [
+    (300, 300, 8, 2, 128),    # four heads per kv head, ragged last tile of queries
+    (128, 333, 4, 2, 64),     # more keys than queries
+    (260, 100, 6, 2, 128),    # fewer keys than queries: late rows see every key; three heads per kv head
+    (32, 1000, 2, 2, 64),     # the fewest query rows this kernel takes
+])
+def test_sdpa_fp16_on_the_matrix_cores(Sq, Skv, Hq, Hkv, D):
+    """fp16 attention with 32 or more query rows runs the tiled MFMA kernel over token-major K/V."""
+    rng = np.random.default_rng(Sq + Skv)
+    q = h16(rng.standard_normal((Sq, Hq, D)))
+    k = h16(rng.standard_normal((Skv, Hkv, D)))
+    v = h16(rng.standard_normal((Skv, Hkv, D)))
+    f = lambda a: a.astype(np.float32)
+    for causal in (True, False):
+        assert_fp16_close(gu.sdpa(q, k, v, causal), port.sdpa(f(q), f(k), f(v), causal))
+
+
 def test_fp16_output_variants_round_once():
     """Norm / SiLU-mul results stored as fp16 from fp32 inputs equal the fp32 result rounded once."""
     rng = np.random.default_rng(30)

@@ -4,6 +4,7 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
 
@@ -24,6 +25,19 @@ inline hipStream_t as_stream(axhip_stream s) { return reinterpret_cast<hipStream
 // Maps a launch error to a Status value.
 inline int launch_status() {
   return hipGetLastError() == hipSuccess ? AXHIP_OK : AXHIP_DEVICE_ERROR;
+}
+
+// Raises a kernel's dynamic LDS limit above the 64 KB default, once per device (the attribute belongs
+// to the kernel's code object on one device).  `done` holds one bit per device.
+inline int raise_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return AXHIP_DEVICE_ERROR;
+  const uint64_t bit = uint64_t(1) << dev;
+  if (done.load(std::memory_order_acquire) & bit) return AXHIP_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+    return AXHIP_INTERNAL_ERROR;
+  done.fetch_or(bit, std::memory_order_release);
+  return AXHIP_OK;
 }
 
 inline bool is_float_dtype(int dt) { return dt == AXHIP_FLOAT16 || dt == AXHIP_FLOAT32; }

@@ -378,13 +378,9 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
   a.N_next = N_next;
   a.eps = eps;
   a.skip = g_tail_skip;
-  static bool lds_set = false;  // more dynamic LDS than the default limit: raised once per process
-  if (!lds_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(decode_tail_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kXBytes + kRBytes) != hipSuccess)
-      return AXHIP_INTERNAL_ERROR;
-    lds_set = true;
-  }
+  static std::atomic<uint64_t> lds_set{0};  // more dynamic LDS than the default limit
+  const int lds_rc = raise_dynamic_lds(reinterpret_cast<const void *>(decode_tail_kernel), kXBytes + kRBytes, lds_set);
+  if (lds_rc != AXHIP_OK) return lds_rc;
   hipLaunchKernelGGL(decode_tail_kernel, dim3(wgs), dim3(kTailThreads), kXBytes + kRBytes, as_stream(stream), a);
   return launch_status();
 }

@@ -1049,14 +1049,10 @@ int launch_decode_mfma_form(const DecodeArgs &a, int B, hipStream_t st) {
   const dim3 grid(a.dynamic ? a.active * n_hg : a.n_splits, a.dynamic ? 1 : n_hg, a.dynamic ? 1 : B);
   auto kernel = gqa_decode_split_kernel<__half, D, 1, 8, QKV, true>;
   constexpr int lds = mfma_lds_bytes<D>();
-  if (lds > 64 * 1024) {  // more dynamic LDS than the default limit: raised once per process and kernel
-    static bool lds_set = false;
-    if (!lds_set) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
-          hipSuccess)
-        return AXHIP_INTERNAL_ERROR;
-      lds_set = true;
-    }
+  if (lds > 64 * 1024) {  // more dynamic LDS than the default limit
+    static std::atomic<uint64_t> lds_set{0};
+    const int rc = raise_dynamic_lds(reinterpret_cast<const void *>(kernel), lds, lds_set);
+    if (rc != AXHIP_OK) return rc;
   }
   hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, a);
   if (a.n_splits > 1 && !a.fused_merge)

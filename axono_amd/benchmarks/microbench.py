@@ -59,18 +59,30 @@ def _emit(rec):
     print(json.dumps(rec), flush=True)
 
 
-def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag="gqa"):
+def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag="gqa", fp32=False,
+              token_major=False):
+    """token_major: K/V as [B, L, Hkv, D] (the layout of the reference's single-sequence call) instead
+    of the cache layout [B, Hkv, L, D]; fp32: FLOAT32 q / K / V / out."""
     elems = B * Hkv * L * D
+    esz = 4 if fp32 else 2
     if n_rot is None:  # enough distinct buffers to exceed the 256 MB Infinity Cache several times
-        n_rot = max(2, min(8, int(2**30 // (elems * 4)) + 1))
+        n_rot = max(2, min(8, int(2**30 // (elems * 2 * esz)) + 1))
     kv = []
     for r in range(n_rot):
-        kb, vb = DeviceBuffer(elems * 2), DeviceBuffer(elems * 2)
-        _rand_fill(kb, elems * 2, 2 * r)
-        _rand_fill(vb, elems * 2, 2 * r + 1)
+        kb, vb = DeviceBuffer(elems * esz), DeviceBuffer(elems * esz)
+        if fp32:
+            blk = np.random.default_rng(r).standard_normal(min(elems, 1 << 22)).astype(np.float32)
+            for buf in (kb, vb):
+                for off in range(0, elems, blk.size):
+                    n = min(blk.size, elems - off)
+                    check(lib.axhip_memcpy_h2d(buf.ptr + off * 4, blk.ctypes.data, n * 4), "h2d")
+        else:
+            _rand_fill(kb, elems * 2, 2 * r)
+            _rand_fill(vb, elems * 2, 2 * r + 1)
         kv.append((kb, vb))
-    q = DeviceBuffer.from_numpy(np.random.default_rng(9).standard_normal((B, Hq, D)).astype(np.float16))
-    out = DeviceBuffer(B * Hq * D * 2)
+    qh = np.random.default_rng(9).standard_normal((B, Hq, D)).astype(np.float32)
+    q = DeviceBuffer.from_numpy(qh if fp32 else qh.astype(np.float16))
+    out = DeviceBuffer(B * Hq * D * esz)
     wsb = lib.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
     ws = DeviceBuffer(max(wsb, 256))
     dl = DeviceBuffer.from_numpy(np.asarray(lens, np.int32)) if lens is not None else None
@@ -79,16 +91,18 @@ def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag=
     def step():
         kb, vb = kv[state["i"] % n_rot]
         state["i"] += 1
-        check(lib.axhip_gqa_decode(q.ptr, kb.ptr, vb.ptr, dl.ptr if dl else None, out.ptr, ws.ptr, wsb, F16, B,
-                                   Hq, Hkv, D, L, Hkv * L * D, L * D, D, None), "gqa_decode")
+        check(lib.axhip_gqa_decode(q.ptr, kb.ptr, vb.ptr, dl.ptr if dl else None, out.ptr, ws.ptr, wsb,
+                                   F32 if fp32 else F16, B, Hq, Hkv, D, L, Hkv * L * D,
+                                   D if token_major else L * D, Hkv * D if token_major else D, None), "gqa_decode")
 
     us = _time(lib, step, steps)
     L_sum = int(np.sum(lens)) if lens is not None else B * L
-    nbytes = 2 * Hkv * D * 2 * L_sum + 2 * Hq * D * 2 * B
+    nbytes = 2 * Hkv * D * esz * L_sum + 2 * Hq * D * esz * B
     s, c = C.c_int(0), C.c_int(0)
     lib.axhip_gqa_decode_plan(B, Hq, Hkv, L, C.byref(s), C.byref(c))
     gbs = nbytes / us / 1e3
-    _emit({"op": tag, "B": B, "L": L, "ragged": lens is not None, "us": round(us, 2), "bytes": nbytes,
+    _emit({"op": tag, "B": B, "L": L, "dtype": "f32" if fp32 else "f16", "token_major": token_major,
+           "ragged": lens is not None, "us": round(us, 2), "bytes": nbytes,
            "GBps": round(gbs, 1), "pct_hbm_peak": round(100 * gbs / HBM_PEAK, 1), "splits": s.value,
            "chunk": c.value, "kv_buffers": n_rot})
     return us
@@ -263,7 +277,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "copy", "rowops", "linear", "linear-packed", "prefill-attn",
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "copy", "rowops", "linear", "linear-packed", "prefill-attn",
                                      "tail"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
@@ -300,6 +314,11 @@ def main(argv=None):
         for Hq, Hkv, D in ((8, 8, 128), (32, 8, 128), (64, 8, 128), (32, 4, 128), (32, 8, 64), (16, 8, 64), (16, 8, 256)):
             for B, L in ((32, 8192), (16, 4160), (4, 8192), (1, 32768)):
                 bench_gqa(lib, B, L, min(args.steps, 50), Hq=Hq, Hkv=Hkv, D=D, tag=f"gqa_Hq{Hq}_Hkv{Hkv}_D{D}")
+    elif args.what == "gqa-single":
+        # the reference's own call: one sequence, q (1,Hq,D), K/V (L,Hkv,D) token-major, fp32 (and the same in fp16)
+        for fp32 in (True, False):
+            for L in (1024, 2048, 8192, 32768, 131072):
+                bench_gqa(lib, 1, L, min(args.steps, 100), fp32=fp32, token_major=True, tag="gqa_single_sequence")
     elif args.what == "prefill-attn":
         for S in (1024, 4096, 16384):
             bench_prefill_attn(lib, max(1, min(args.B, 65536 // S)), S, max(5, min(args.steps, 20)))

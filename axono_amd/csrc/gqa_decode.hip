@@ -114,7 +114,9 @@ struct Frag8;
 template <>
 struct Frag8<__half> {
   Vec16 v;
+  template <int SECOND>
   __device__ __forceinline__ void load(const __half *p) { v = ld16(p); }
+  template <int SECOND>
   __device__ __forceinline__ void load_stream(const __half *p) { v = ld16_stream(p); }
   __device__ __forceinline__ void zero() { v.w[0] = v.w[1] = v.w[2] = v.w[3] = 0u; }
   // sum_i q[i]*k[i]: four packed fp16 dot-2 with an fp32 accumulator (products are exact in fp32)
@@ -137,16 +139,19 @@ struct Frag8<__half> {
 template <>
 struct Frag8<float> {
   float f[8];
+  // elements 4..7 sit SECOND elements behind p (see FragMap)
+  template <int SECOND>
   __device__ __forceinline__ void load(const float *p) {
-    const Vec16 a = ld16(p), b = ld16(p + 4);
+    const Vec16 a = ld16(p), b = ld16(p + SECOND);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       f[i] = __builtin_bit_cast(float, a.w[i]);
       f[4 + i] = __builtin_bit_cast(float, b.w[i]);
     }
   }
+  template <int SECOND>
   __device__ __forceinline__ void load_stream(const float *p) {
-    const Vec16 a = ld16_stream(p), b = ld16_stream(p + 4);
+    const Vec16 a = ld16_stream(p), b = ld16_stream(p + SECOND);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       f[i] = __builtin_bit_cast(float, a.w[i]);
@@ -168,6 +173,24 @@ struct Frag8<float> {
     for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, f[i], acc[i]);
   }
 };
+
+// Which 8 of a row's D elements lane `dl` of a row group holds.  fp16: 8 consecutive ones (one
+// 16-byte load).  fp32 takes two 16-byte loads; 4 elements from each half of the row, so that the
+// lanes of a row group read a contiguous half row per load instruction (with 8 consecutive elements
+// per lane each instruction would touch every cache line of the row and use half of it).
+template <typename T, int D>
+struct FragMap {
+  static constexpr int kLane = sizeof(T) == 4 ? 4 : 8;        // first element = dl * kLane
+  static constexpr int kSecond = sizeof(T) == 4 ? D / 2 : 4;  // offset of elements 4..7 from there
+};
+
+// Writes a lane's 8 accumulators to their places in an fp32 row of D elements.
+template <typename T, int D>
+__device__ __forceinline__ void store_lane_acc(float *row, int dl, const float (&acc)[8]) {
+  float *p = row + dl * FragMap<T, D>::kLane;
+  *reinterpret_cast<float4 *>(p) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  *reinterpret_cast<float4 *>(p + FragMap<T, D>::kSecond) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+}
 
 struct DecodeArgs {
   const void *q, *k, *v;
@@ -301,8 +324,8 @@ __device__ __forceinline__ void tile_load(const T *kb, const T *vb, int64_t stri
   for (int u = 0; u < U; ++u) {
     const int row = base + u * RG + rg;
     if (!CHECK || row < s1) {
-      kr[u].load_stream(kb + row * stride_s);  // K and V rows are read once: streaming loads
-      vr[u].load_stream(vb + row * stride_s);
+      kr[u].template load_stream<FragMap<T, D>::kSecond>(kb + row * stride_s);  // read once: streaming loads
+      vr[u].template load_stream<FragMap<T, D>::kSecond>(vb + row * stride_s);
     } else {
       kr[u].zero();
       vr[u].zero();
@@ -388,7 +411,9 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   const int rg = tid / LPR, dl = tid % LPR;
   const int hk = h0 / a.group;      // the kv head those G query heads share
 
-  const int64_t kv_off = b * a.stride_b + hk * a.stride_h + dl * 8;
+  constexpr int SEC = FragMap<T, D>::kSecond;
+  const int lane_el = dl * FragMap<T, D>::kLane;  // this lane's first element of a row
+  const int64_t kv_off = b * a.stride_b + hk * a.stride_h + lane_el;
   const T *kb = static_cast<const T *>(a.k) + kv_off;
   const T *vb = static_cast<const T *>(a.v) + kv_off;
 
@@ -433,11 +458,12 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
     }
     __syncthreads();
 #pragma unroll
-    for (int g = 0; g < G; ++g) qf[g].load(&s_q[g][dl * 8]);
+    for (int g = 0; g < G; ++g) qf[g].template load<SEC>(&s_q[g][lane_el]);
   } else {
     const T *q = static_cast<const T *>(a.q);
 #pragma unroll
-    for (int g = 0; g < G; ++g) qf[g].load(q + (static_cast<int64_t>(b) * a.Hq + h0 + g) * D + dl * 8);
+    for (int g = 0; g < G; ++g)
+      qf[g].template load<SEC>(q + (static_cast<int64_t>(b) * a.Hq + h0 + g) * D + lane_el);
   }
 
   float m[G], l[G], acc[G][8];
@@ -461,8 +487,8 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   if constexpr (QKV) {
     if (mine) {  // the new token's key and value: one more row, taken by row group 0
       Frag8<T> kn, vn;
-      kn.load(&s_kv[0][dl * 8]);
-      vn.load(&s_kv[1][dl * 8]);
+      kn.template load<SEC>(&s_kv[0][lane_el]);
+      vn.template load<SEC>(&s_kv[1][lane_el]);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const float d = group_sum<LPR>(qf[g].dot(kn)) * a.scale_log2e;
@@ -490,7 +516,7 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
       s_m[g][rg] = m[g];
       s_l[g][rg] = l[g];
     }
-    Row8<float>::store(&s_acc[g][rg][dl * 8], acc[g]);
+    store_lane_acc<T, D>(s_acc[g][rg], dl, acc[g]);
   }
   __syncthreads();
   for (int o = tid; o < G * D; o += kThreads) {

@@ -108,6 +108,52 @@ def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag=
     return us
 
 
+def bench_gqa_step_form(lib, B, L, steps, Hq=16, Hkv=8, D=128, rows=None, n_rot=4):
+    """The attention launch of a decode step (q/k RMSNorm, M-RoPE and the KV append in its prologue)
+    beside plain attention over the same L + 1 keys of the same caches."""
+    rows = rows or (L + 128) // 128 * 128
+    elems = B * Hkv * rows * D
+    kv = []
+    for r in range(n_rot):
+        kb, vb = DeviceBuffer(elems * 2), DeviceBuffer(elems * 2)
+        _rand_fill(kb, elems * 2, 2 * r)
+        _rand_fill(vb, elems * 2, 2 * r + 1)
+        kv.append((kb, vb))
+    rng = np.random.default_rng(5)
+    width = (Hq + 2 * Hkv) * D
+    qkv = DeviceBuffer.from_numpy(rng.standard_normal((B, width)).astype(np.float32))
+    qh = DeviceBuffer.from_numpy(rng.standard_normal((B, Hq, D)).astype(np.float16))
+    wq = DeviceBuffer.from_numpy(np.ones(D, np.float32))
+    wk = DeviceBuffer.from_numpy(np.ones(D, np.float32))
+    pos = DeviceBuffer.from_numpy(np.full((3, B), L, np.int64))
+    inv = DeviceBuffer.from_numpy((1.0 / (1e6 ** (np.arange(0, D, 2, dtype=np.float32) / D))).astype(np.float32))
+    lens = DeviceBuffer.from_numpy(np.full(B, L, np.int32))
+    lens1 = DeviceBuffer.from_numpy(np.full(B, L + 1, np.int32))
+    out = DeviceBuffer(B * Hq * D * 2)
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, rows)
+    ws = DeviceBuffer(max(wsb, 256))
+    state = {"i": 0}
+
+    def step_form():
+        kb, vb = kv[state["i"] % n_rot]
+        state["i"] += 1
+        check(lib.axhip_gqa_decode_qkv(qkv.ptr, width, qkv.ptr + Hq * D * 4, width, qkv.ptr + (Hq + Hkv) * D * 4, width,
+                                       wq.ptr, wk.ptr, F32, 1e-6, pos.ptr, inv.ptr, 20, 20, lens.ptr, kb.ptr, vb.ptr,
+                                       out.ptr, ws.ptr, wsb, F16, B, Hq, Hkv, D, rows, rows, None), "gqa_decode_qkv")
+
+    def plain():
+        kb, vb = kv[state["i"] % n_rot]
+        state["i"] += 1
+        check(lib.axhip_gqa_decode(qh.ptr, kb.ptr, vb.ptr, lens1.ptr, out.ptr, ws.ptr, wsb, F16, B, Hq, Hkv, D, rows,
+                                   Hkv * rows * D, rows * D, D, None), "gqa_decode")
+
+    nbytes = 2 * Hkv * D * 2 * (L + 1) * B + 2 * Hq * D * 2 * B
+    for name, fn in (("gqa_plain", plain), ("gqa_decode_step_form", step_form)):
+        us = _time(lib, fn, steps)
+        _emit({"op": name, "B": B, "L": L + 1, "cache_rows": rows, "us": round(us, 2), "bytes": nbytes,
+               "GBps": round(nbytes / us / 1e3, 1), "pct_hbm_peak": round(100 * nbytes / us / 1e3 / HBM_PEAK, 1)})
+
+
 def bench_prefill_attn(lib, B, S, steps, Hq=16, Hkv=8, D=128):
     """Causal prefill attention: 4*D flops per visible (query, key) pair and query head."""
     n = B * Hkv * S * D
@@ -277,13 +323,14 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "copy", "rowops", "linear", "linear-packed", "prefill-attn",
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "copy", "rowops", "linear", "linear-packed", "prefill-attn",
                                      "tail"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--mib", type=int, default=1024)
     ap.add_argument("--ragged", action="store_true")
+    ap.add_argument("--rows", type=int, default=0, help="gqa-step: rows the caches are allocated for (default: L rounded up)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--target-wgs", type=int, default=0)
     ap.add_argument("--nt", type=int, default=0, help="linear: 16-row groups of W per wavefront (1, 2, 4)")
@@ -314,6 +361,9 @@ def main(argv=None):
         for Hq, Hkv, D in ((8, 8, 128), (32, 8, 128), (64, 8, 128), (32, 4, 128), (32, 8, 64), (16, 8, 64), (16, 8, 256)):
             for B, L in ((32, 8192), (16, 4160), (4, 8192), (1, 32768)):
                 bench_gqa(lib, B, L, min(args.steps, 50), Hq=Hq, Hkv=Hkv, D=D, tag=f"gqa_Hq{Hq}_Hkv{Hkv}_D{D}")
+    elif args.what == "gqa-step":
+        bench_gqa_step_form(lib, args.B if args.B != 32 else 16, args.L if args.L != 8192 else 4160, args.steps,
+                            rows=args.rows or None)
     elif args.what == "gqa-single":
         # the reference's own call: one sequence, q (1,Hq,D), K/V (L,Hkv,D) token-major, fp32 (and the same in fp16)
         for fp32 in (True, False):

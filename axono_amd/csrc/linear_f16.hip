@@ -41,7 +41,7 @@ struct SkinnyPlan {
 // through LDS, so one launch finishes the product.  Small N gets more wavefronts per workgroup
 // (down to 128 of K each) so that the launch still fills the chip.
 SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
-  // Measured at M = 16 on MI355X (packed weights): two row tiles per wavefront win once N >= 8192
+  // Measured at M = 16 and 32 on MI355X (packed weights): two row tiles per wavefront win once N >= 8192
   // (lm_head 2048 -> 151936: 109 us with NT=2 / 8 wavefronts against 125 us with NT=4 / 4), one tile
   // with 8-16 K slices wins for the small matrices; every kernel costs about 3 us plus its bytes at
   // 5.5-5.7 TB/s.
@@ -50,8 +50,8 @@ SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
   if (g_lin.force_nt > 0)
     p.nt = g_lin.force_nt;
   else
-    p.nt = (p.mt == 2 || N >= 8192) ? 2 : 1;
-  if (p.mt == 2 && p.nt > 2) p.nt = 2;
+    p.nt = N >= 8192 ? 2 : 1;
+
   const int64_t ntiles = (N + p.nt * 16 - 1) / (p.nt * 16);
   int64_t want = g_lin.force_waves > 0 ? g_lin.force_waves : (g_lin.target_waves + ntiles - 1) / ntiles;
   if (g_lin.force_waves == 0 && want < 8) want = 8;
@@ -60,6 +60,9 @@ SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
   while (waves > 4 && K / waves < 128) waves /= 2;
   if (p.nt == 4 && waves > 4) waves = 4;   // LDS: the reduction buffer grows with NT * waves
   if (p.nt * p.mt >= 2 && waves > 8) waves = 8;
+  // 32 rows of x double the LDS strip of a wavefront: with two row tiles of W, four wavefronts per
+  // workgroup keep as many workgroups on a CU as at 16 rows (M = 32, 2048 -> 151936: 117 us against 134)
+  if (g_lin.force_waves == 0 && p.mt == 2 && p.nt == 2 && waves > 4) waves = 4;
   p.waves = waves;
   // with one row tile per workgroup and at most 128 tiles half the CUs would idle: 8 rows per workgroup
   p.half = (p.nt == 1 && ntiles * ((M + p.mt * 16 - 1) / (p.mt * 16)) <= 128) ? 1 : 0;
@@ -557,7 +560,9 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
     else
       dispatch_packed_waves<1, 1, XT>(a, p.waves, half, st);
   } else {
-    if (p.nt == 2)
+    if (p.nt == 4)
+      dispatch_packed_waves<4, 2, XT>(a, p.waves, half, st);
+    else if (p.nt == 2)
       dispatch_packed_waves<2, 2, XT>(a, p.waves, half, st);
     else
       dispatch_packed_waves<1, 2, XT>(a, p.waves, half, st);
@@ -582,11 +587,11 @@ constexpr int kXcds = 8;
 // FULL: K is a multiple of the 128-column step, so no load needs a predicate (rows and tiles past
 // the edge are clamped to valid memory and their results never stored).  Predicated loads compile to
 // branches, after which the compiler waits for every outstanding load before each MFMA group.
-// GM: rows of x per workgroup.  128 gives the larger tile (one workgroup per CU, 87 flop per byte
+// GM: rows of x per workgroup (32 only for the smallest problems, with TW = 1).  128 gives the larger tile (one workgroup per CU, 87 flop per byte
 // moved from L2); 64 halves the registers so that two workgroups share a CU and one's loads hide
 // behind the other's MFMAs.
 template <typename XT, bool FULL, int GM, int TW>
-__global__ __launch_bounds__(256, GM == 64 ? 2 : 1) void linear_gemm_packed_kernel(PackedArgs a, int n_blocks, int m_blocks) {
+__global__ __launch_bounds__(256, GM == 128 ? 1 : (GM == 64 ? 2 : 4)) void linear_gemm_packed_kernel(PackedArgs a, int n_blocks, int m_blocks) {
   constexpr int MT = GM / 16;        // x row tiles per wavefront
   constexpr int XV = GM * 16 / 256;  // 16-byte x vectors staged per thread and step
   __shared__ __attribute__((aligned(16))) _Float16 xs[2][GM * kGK];
@@ -871,6 +876,10 @@ void launch_gemm_packed_tw(const PackedArgs &a, int gm, hipStream_t st) {
   hipLaunchKernelGGL((linear_gemm_packed_kernel<XT, F, G, TW>), grid, dim3(256), 0, st, a, n_blocks, m_blocks)
   if (gm == 128) {
     if (full) AXHIP_GEMM_LAUNCH(true, 128); else AXHIP_GEMM_LAUNCH(false, 128);
+  } else if (gm == 32 && TW == 1) {  // the 32-row tile exists for one row tile of W per wavefront only
+    if constexpr (TW == 1) {
+      if (full) AXHIP_GEMM_LAUNCH(true, 32); else AXHIP_GEMM_LAUNCH(false, 32);
+    }
   } else {
     if (full) AXHIP_GEMM_LAUNCH(true, 64); else AXHIP_GEMM_LAUNCH(false, 64);
   }
@@ -891,8 +900,13 @@ void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
       return;
     }
   }
-  const int gm = (g_gemm_rows == 64 || g_gemm_rows == 128) ? g_gemm_rows : 64;
-  switch (gemm_tiles_per_wave(a, gm)) {
+  int gm = (g_gemm_rows == 32 || g_gemm_rows == 64 || g_gemm_rows == 128) ? g_gemm_rows : 64;
+  const int tw = gemm_tiles_per_wave(a, gm == 32 ? 64 : gm);
+  // a problem that gives no CU a second workgroup even with the smallest weight tile is bounded by the
+  // latency of its K steps: 32 rows of x per workgroup double the workgroups that can overlap
+  if (g_gemm_rows == 0 && tw == 1 && static_cast<int64_t>((a.N + 63) / 64) * ((a.M + 63) / 64) <= 256) gm = 32;
+  if (gm == 32 && tw != 1) gm = 64;
+  switch (tw) {
     case 1: return launch_gemm_packed_tw<XT, 1>(a, gm, st);
     case 2: return launch_gemm_packed_tw<XT, 2>(a, gm, st);
     default: return launch_gemm_packed_tw<XT, 4>(a, gm, st);
@@ -911,7 +925,7 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
   // gemm_rows: 64 or 128 rows of x per GEMM workgroup, plus 1000 t to force t = 1, 2, 4 row tiles of W per wavefront
   g_gemm_tiles = gemm_rows >= 1000 ? gemm_rows / 1000 : 0;
   gemm_rows %= 1000;
-  g_gemm_rows = (gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256) ? gemm_rows : 0;
+  g_gemm_rows = (gemm_rows == 32 || gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256) ? gemm_rows : 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;

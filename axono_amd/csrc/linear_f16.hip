@@ -1013,7 +1013,11 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
   if (!x || !packed_w || !out) return AXHIP_INVALID_PTR;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(packed_w) | reinterpret_cast<uintptr_t>(out)) & 15)
     return AXHIP_INVALID_PTR;
-  if (M > kSkinnyMaxM) {  // MFMA-bound regime: tiled GEMM over the same packed buffer
+  // Up to 64 rows a narrow matrix (N <= 2048) stays with the weight-streaming kernels, two blocks of 32
+  // rows each: the tiled GEMM would have too few workgroups there (M = 64: 2048 -> 2048 6.3 us against
+  // 11.2, 6144 -> 2048 12.9 against 27.4; wider matrices and more rows go the other way).
+  const bool skinny = M <= kSkinnyMaxM || (M <= 2 * kSkinnyMaxM && N <= 2048);
+  if (!skinny) {  // MFMA-bound regime: tiled GEMM over the same packed buffer
     PackedArgs ga;
     ga.x = x;
     ga.wp = static_cast<const __half *>(packed_w);

@@ -729,6 +729,99 @@ __global__ __launch_bounds__(256, GM == 128 ? 1 : (GM == 64 ? 2 : 4)) void linea
   }
 }
 
+// The smallest problems (one row tile of W per wavefront, 64 weight rows x GM rows of x per workgroup,
+// at most two workgroups per CU): a step of 128 K is 4 * GM/16 products per wavefront, far less than a
+// memory latency, so the loads run P steps ahead of the products (W fragments and the x vectors of a
+// step wait in registers; x goes into the LDS double buffer one step before its use).  K is a multiple
+// of P * 128; rows and tiles past the edge are clamped to valid memory and never stored.
+template <typename XT, int GM, int P>
+__global__ __launch_bounds__(256, GM == 64 ? 2 : 4) void linear_gemm_packed_deep_kernel(PackedArgs a, int n_blocks,
+                                                                                      int m_blocks) {
+  constexpr int MT = GM / 16;
+  constexpr int XV = GM * 16 / 256;
+  __shared__ __attribute__((aligned(16))) _Float16 xs[2][GM * kGK];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int id = blockIdx.x;
+  const int xcd = id % kXcds, slot = id / kXcds;
+  const int nb = (slot / m_blocks) * kXcds + xcd, mb = slot % m_blocks;
+  if (nb >= n_blocks) return;
+  const int n_tiles = (a.N + 15) / 16;
+  const int tile = nb * 4 + wave;
+  const int m0 = mb * GM;
+  const XT *x = static_cast<const XT *>(a.x);
+  const int steps = a.KC / 4;
+
+  const __half *wt = a.wp + (static_cast<int64_t>(min(tile, n_tiles - 1)) * a.KC) * 512 + lane * 8;
+  const XT *xp[XV];
+#pragma unroll
+  for (int p = 0; p < XV; ++p) {
+    const int v = p * 256 + tid;
+    xp[p] = x + static_cast<int64_t>(min(m0 + (v >> 4), a.M - 1)) * a.K + (v & 15) * 8;
+  }
+  auto load_step = [&](int step, half8_t (&w)[4], half8_t (&xv)[XV]) __attribute__((always_inline)) {
+    const int sc = min(step, steps - 1);  // past the end: the last step again, never used
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = load_h8(wt + static_cast<int64_t>(sc * 4 + j) * 512);
+#pragma unroll
+    for (int p = 0; p < XV; ++p) xv[p] = load_h8(xp[p] + sc * kGK);
+  };
+  auto store_x = [&](int buf, const half8_t (&xv)[XV]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) {
+      const int v = p * 256 + tid;
+      const int row = v >> 4, unit = v & 15;
+      *reinterpret_cast<half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]) = xv[p];
+    }
+  };
+
+  float4_t acc[MT];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) acc[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  half8_t wf[P][4], xv[P][XV];
+#pragma unroll
+  for (int s = 0; s < P; ++s) load_step(s, wf[s], xv[s]);
+  store_x(0, xv[0]);
+  __syncthreads();
+
+  for (int i0 = 0; i0 < steps; i0 += P) {
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+      const int buf = (i0 + s) & 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        half8_t bf[MT];
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+          const int row = u * 16 + r, unit = j * 4 + g;
+          bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
+        }
+#pragma unroll
+        for (int u = 0; u < MT; ++u) acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[s][j], bf[u], acc[u], 0, 0, 0);
+      }
+      // x of the next step (requested P - 1 steps ago) goes to the other LDS buffer; this step's
+      // registers then take the loads of step i + P
+      store_x(buf ^ 1, xv[(s + 1) % P]);
+      load_step(i0 + s + P, wf[s], xv[s]);
+      __syncthreads();
+    }
+  }
+
+  LinearArgs o;
+  o.bias = a.bias;
+  o.out = a.out;
+  o.M = a.M;
+  o.N = a.N;
+  o.out_f16 = a.out_f16;
+  if (tile >= n_tiles) return;
+#pragma unroll
+  for (int u = 0; u < MT; ++u) {
+    const float v[4] = {acc[u][0], acc[u][1], acc[u][2], acc[u][3]};
+    store_out4(o, m0 + u * 16 + r, tile * 16 + 4 * g, v);
+  }
+}
+
 // 256 weight rows x 128 rows of x with two workgroups per CU.  Against the 256 x 64 tile this halves
 // the W bytes that pass through the CU's vector memory path per product (that path, 64 bytes per
 // clock, is what bounds the smaller tile), but its 128 accumulators leave room for little else in the
@@ -906,6 +999,23 @@ void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
   // latency of its K steps: 32 rows of x per workgroup double the workgroups that can overlap
   if (g_gemm_rows == 0 && tw == 1 && static_cast<int64_t>((a.N + 63) / 64) * ((a.M + 63) / 64) <= 256) gm = 32;
   if (gm == 32 && tw != 1) gm = 64;
+  constexpr int kDeep = 4;  // steps the loads of the smallest tile run ahead
+  // (fp16 x only: fp32 x is converted as it arrives, which would put a wait behind every load)
+  // only while no CU gets a second workgroup: with more of them the L2 bandwidth of these small tiles
+  // is the bound, not the latency of a step
+  if (sizeof(XT) == 2 && tw == 1 && !a.glu && (gm == 32 || gm == 64) && a.K % (kDeep * kGK) == 0 && g_gemm_tiles == 0 &&
+      static_cast<int64_t>((a.N + 63) / 64) * ((a.M + gm - 1) / gm) <= 256) {
+    const int n_blocks = (a.N + 63) / 64, m_blocks = (a.M + gm - 1) / gm;
+    const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
+    const dim3 grid(static_cast<unsigned>(nb_pad) * m_blocks);
+    if constexpr (sizeof(XT) == 2) {
+      if (gm == 32)
+        hipLaunchKernelGGL((linear_gemm_packed_deep_kernel<XT, 32, kDeep>), grid, dim3(256), 0, st, a, n_blocks, m_blocks);
+      else
+        hipLaunchKernelGGL((linear_gemm_packed_deep_kernel<XT, 64, kDeep>), grid, dim3(256), 0, st, a, n_blocks, m_blocks);
+    }
+    return;
+  }
   switch (tw) {
     case 1: return launch_gemm_packed_tw<XT, 1>(a, gm, st);
     case 2: return launch_gemm_packed_tw<XT, 2>(a, gm, st);

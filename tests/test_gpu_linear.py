@@ -113,10 +113,12 @@ def test_packed_weights_config4_shapes(M, K, N):
     assert np.abs(out - gu.linear_f16(x, w)).max() <= 1e-4
 
 
-@pytest.mark.parametrize("M,K,N", [(33, 2048, 2048), (64, 6144, 2048), (50, 520, 130), (64, 2048, 2064), (65, 2048, 2048)])
+@pytest.mark.parametrize("M,K,N", [(33, 2048, 2048), (64, 6144, 2048), (50, 520, 130), (64, 2048, 2064), (65, 2048, 2048),
+                                   (200, 6144, 2048), (100, 1024, 1000), (130, 1536, 4096)])
 def test_packed_weights_33_to_64_rows(M, K, N):
     """Narrow matrices keep the weight-streaming kernels up to 64 rows (two blocks of rows); one column
-    tile more, or one row more, and the tiled GEMM takes over.  Same oracle either side of the switch."""
+    tile more, or one row more, and the tiled GEMM takes over - for problems this small its form whose
+    loads run four K steps ahead (K a multiple of 512).  Same oracle either side of each switch."""
     rng = np.random.default_rng(M + K + N)
     x = h16(rng.standard_normal((M, K)))
     w = h16(0.02 * rng.standard_normal((N, K)))
@@ -124,6 +126,8 @@ def test_packed_weights_33_to_64_rows(M, K, N):
     want = port.linear(x.astype(np.float32), w.astype(np.float32))
     mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
     assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag)
+    # fp32 activations are rounded to fp16 on load: the same result
+    np.testing.assert_array_equal(gu.linear_f16_packed(x.astype(np.float32), w), out)
 
 
 def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():

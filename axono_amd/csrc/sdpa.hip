@@ -91,7 +91,7 @@ AXHIP_API int axhip_sdpa(const void *q, const void *k, const void *v, void *out,
   // fp16 with enough query rows to fill 16-row tiles: the causal prefill kernel on the matrix cores
   const uintptr_t ptr_bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
                              reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out);
-  if (dtype == AXHIP_FLOAT16 && (D == 64 || D == 128) && Sq >= kMfmaMinRows && Hq <= 65535 * 4 &&
+  if (dtype == AXHIP_FLOAT16 && (D == 64 || D == 128) && Sq >= kMfmaMinRows && Hq <= 65535 &&
       (ptr_bits & 15) == 0)
     return axhip_internal_sdpa_f16_mfma(q, k, v, out, Sq, Hq, Hkv, D, Skv, is_causal, st);
 

@@ -44,6 +44,9 @@ PROTOTYPES = {
     "axhip_graph_end_capture": (c_i, [c_vp, C.POINTER(c_vp), C.POINTER(c_sz)]),
     "axhip_graph_abort_capture": (c_i, [c_vp]),
     "axhip_graph_launch": (c_i, [c_vp]),
+    "axhip_graph_launch_async": (c_i, [c_vp]),
+    "axhip_set_ticket_lane": (c_i, [c_i]),
+    "axhip_ticket_lane": (c_i, []),
     "axhip_graph_sync": (c_i, [c_vp]),
     "axhip_graph_destroy": (c_i, [c_vp]),
     "axhip_capture_pool_reset": (c_i, []),

@@ -42,6 +42,11 @@ class HIPGraph:
         self._impl.launch()
         return self
 
+    def launch_async(self) -> "HIPGraph":
+        """Enqueues one replay on the graph's own stream only; see libaxono.HIPGraph.launch_async."""
+        self._impl.launch_async()
+        return self
+
     @property
     def output(self):
         return self._output

@@ -42,9 +42,10 @@ Tuning g_tuning;
 // Ticket counters of the in-kernel merge, one per (sequence, head group).  They start at zero and
 // the merging workgroup puts its counter back to zero, so no launch ever has to clear them.
 // Launches that overlap in time on one device must not share (sequence, head group) slots; calls on
-// one stream, and replays of a captured graph, never overlap.
-constexpr int kTicketSlots = 1 << 16;
-__device__ unsigned int g_tickets[kTicketSlots];
+// one stream, and replays of a captured graph, never overlap.  Launches that do overlap (graphs replayed
+// side by side) come from different ticket lanes: a lane is a region of its own in this array.
+constexpr int kTicketSlots = 1 << 16;  // per ticket lane
+__device__ unsigned int g_tickets[AXHIP_TICKET_LANES * kTicketSlots];
 
 constexpr int kMaxDynBatch = 64;  // batches up to this size deal their workgroups by sequence length
 
@@ -201,6 +202,7 @@ struct DecodeArgs {
   int Hq, group, max_len, chunk, n_splits;
   int dynamic, active, split_stride, B, n_hg;  // see SplitPlan; split_stride = partial slots per (sequence, head)
   int wg_heads;  // query heads per workgroup (the template parameter G on the vector path)
+  int ticket_base;  // first ticket counter of the caller's ticket lane
   int64_t stride_b, stride_h, stride_s;
   float scale_log2e;
   int fused_merge;  // the last workgroup of a (sequence, head group) merges the splits
@@ -549,7 +551,7 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   __shared__ int s_last;
   __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
   if (tid == 0) {
-    unsigned int *ticket = &g_tickets[b * a.n_hg + hg];
+    unsigned int *ticket = &g_tickets[a.ticket_base + b * a.n_hg + hg];
     const unsigned int t = atomicAdd(ticket, 1u);
     s_last = (t == static_cast<unsigned int>(n_valid - 1));
     if (s_last) atomicExch(ticket, 0u);  // ready for the next launch
@@ -636,7 +638,7 @@ __device__ __forceinline__ void finish_range(const DecodeArgs &a, int b, int hg,
   // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
   __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
   if (tid == 0) {
-    unsigned int *ticket = &g_tickets[b * a.n_hg + hg];
+    unsigned int *ticket = &g_tickets[a.ticket_base + b * a.n_hg + hg];
     const unsigned int t = atomicAdd(ticket, 1u);
     *s_last = (t == static_cast<unsigned int>(n_valid - 1));
     if (*s_last) atomicExch(ticket, 0u);  // ready for the next launch
@@ -1135,6 +1137,7 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
                     a.stride_s % 8 == 0 && a.stride_h % 8 == 0 && a.stride_b % 8 == 0;
   const int G = mfma ? mfma_heads_per_workgroup(group) : heads_per_workgroup(group);
   a.wg_heads = G;
+  a.ticket_base = axhip_ticket_lane() * kTicketSlots;
   const SplitPlan plan = plan_splits(B, Hq / G, max_len);
   a.Hq = Hq;
   a.group = group;

@@ -545,10 +545,10 @@ __global__ __launch_bounds__(kArgmaxBlock) void argmax_kernel(const T *__restric
 // (value, index) candidates in device scratch, and the workgroup that takes the last ticket of the row
 // picks the winner.  Ties go to the smaller index, as in the single-workgroup kernel.
 constexpr int kArgmaxParts = 64;
-constexpr int kArgmaxMaxRows = 1024;
-__device__ float g_argmax_val[kArgmaxMaxRows * kArgmaxParts];
-__device__ long long g_argmax_idx[kArgmaxMaxRows * kArgmaxParts];
-__device__ unsigned int g_argmax_ticket[kArgmaxMaxRows];
+constexpr int kArgmaxMaxRows = 1024;  // per ticket lane
+__device__ float g_argmax_val[AXHIP_TICKET_LANES * kArgmaxMaxRows * kArgmaxParts];
+__device__ long long g_argmax_idx[AXHIP_TICKET_LANES * kArgmaxMaxRows * kArgmaxParts];
+__device__ unsigned int g_argmax_ticket[AXHIP_TICKET_LANES * kArgmaxMaxRows];
 
 __device__ __forceinline__ bool better(float ov, int64_t oi, float v, int64_t i) {
   return oi != INT64_MAX && (i == INT64_MAX || ov > v || (ov == v && oi < i));
@@ -556,11 +556,13 @@ __device__ __forceinline__ bool better(float ov, int64_t oi, float v, int64_t i)
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restrict__ x,
-                                                              int64_t *__restrict__ out, int64_t cols, int vec_ok) {
+                                                              int64_t *__restrict__ out, int64_t cols, int vec_ok,
+                                                              int lane_row0) {
   __shared__ float s_val[kBlock / 64];
   __shared__ int64_t s_idx[kBlock / 64];
   __shared__ int s_last;
   const int row = blockIdx.y, part = blockIdx.x;
+  const int trow = lane_row0 + row;  // this row's place in the caller's ticket lane
   const T *xr = x + static_cast<int64_t>(row) * cols;
   // parts start on multiples of 8 elements, so that a row whose length is a multiple of 8 can be read
   // with 16-byte loads; the first maximum wins inside a thread as it does across threads
@@ -627,19 +629,19 @@ __global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restric
         bi = s_idx[w];
       }
     // agent-scope stores: written through, visible to a workgroup on another XCD (no L2 write-back)
-    __hip_atomic_store(&g_argmax_val[row * kArgmaxParts + part], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&g_argmax_idx[row * kArgmaxParts + part], static_cast<long long>(bi), __ATOMIC_RELAXED,
+    __hip_atomic_store(&g_argmax_val[trow * kArgmaxParts + part], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&g_argmax_idx[trow * kArgmaxParts + part], static_cast<long long>(bi), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_s_waitcnt(0);  // both stores have completed before the ticket is taken
-    const unsigned int t = atomicAdd(&g_argmax_ticket[row], 1u);
+    const unsigned int t = atomicAdd(&g_argmax_ticket[trow], 1u);
     s_last = (t == kArgmaxParts - 1);
-    if (s_last) atomicExch(&g_argmax_ticket[row], 0u);
+    if (s_last) atomicExch(&g_argmax_ticket[trow], 0u);
   }
   __syncthreads();
   if (!s_last || threadIdx.x >= 64) return;
   // one wavefront: lane p takes part p (kArgmaxParts == 64)
-  best = __hip_atomic_load(&g_argmax_val[row * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  bi = __hip_atomic_load(&g_argmax_idx[row * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  best = __hip_atomic_load(&g_argmax_val[trow * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  bi = __hip_atomic_load(&g_argmax_idx[trow * kArgmaxParts + threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(best, off, 64);
     const int64_t oi = __shfl_xor(bi, off, 64);
@@ -841,12 +843,13 @@ AXHIP_API int axhip_argmax(const void *x, int64_t *out, int dtype, int64_t rows,
   if (cols >= 16384 && rows <= kArgmaxMaxRows) {
     const dim3 pgrid(kArgmaxParts, static_cast<unsigned>(rows));
     const int vec_ok = (cols % 8 == 0 && aligned16(x)) ? 1 : 0;  // every part of every row then starts 16-byte aligned
+    const int lane_row0 = axhip_ticket_lane() * kArgmaxMaxRows;
     if (dtype == AXHIP_FLOAT16)
       hipLaunchKernelGGL((argmax_parts_kernel<__half>), pgrid, dim3(kBlock), 0, st,
-                         static_cast<const __half *>(x), out, cols, vec_ok);
+                         static_cast<const __half *>(x), out, cols, vec_ok, lane_row0);
     else
       hipLaunchKernelGGL((argmax_parts_kernel<float>), pgrid, dim3(kBlock), 0, st,
-                         static_cast<const float *>(x), out, cols, vec_ok);
+                         static_cast<const float *>(x), out, cols, vec_ok, lane_row0);
     return launch_status();
   }
   const dim3 grid(static_cast<unsigned>(rows));

@@ -126,6 +126,7 @@ void *acquire_locked(int dev, size_t rounded) {
 }
 
 hipStream_t current_stream() { return t_capturing ? t_capture_stream : nullptr; }
+thread_local int t_ticket_lane = 0;
 
 }  // namespace
 }  // namespace axhip
@@ -299,6 +300,13 @@ AXHIP_API int axhip_fill_zero(void *dst, size_t bytes) {
 
 // ---- stream / capture state ----------------------------------------------------------------------
 AXHIP_API axhip_stream axhip_current_stream(void) { return current_stream(); }
+
+AXHIP_API int axhip_set_ticket_lane(int lane) {
+  if (lane < 0 || lane >= AXHIP_TICKET_LANES) return AXHIP_INVALID_ARGUMENT;
+  t_ticket_lane = lane;
+  return AXHIP_OK;
+}
+AXHIP_API int axhip_ticket_lane(void) { return t_ticket_lane; }
 AXHIP_API int axhip_is_capturing(void) { return t_capturing ? 1 : 0; }
 
 AXHIP_API int axhip_synchronize(void) {
@@ -433,6 +441,16 @@ AXHIP_API int axhip_graph_launch(axhip_graph graph) {
   if (hipEventRecord(ge->ev_out, ge->stream) != hipSuccess) return AXHIP_DEVICE_ERROR;
   if (hipStreamWaitEvent(nullptr, ge->ev_out, 0) != hipSuccess) return AXHIP_DEVICE_ERROR;
   return AXHIP_OK;
+}
+
+AXHIP_API int axhip_graph_launch_async(axhip_graph graph) {
+  GraphExec *ge = static_cast<GraphExec *>(graph);
+  if (!ge || !ge->exec) return AXHIP_INVALID_ARGUMENT;
+  if (t_capturing) return AXHIP_INVALID_ARGUMENT;
+  (void)hipGetLastError();
+  // on the graph's own stream only: no edge to or from the default stream, so replays of different
+  // graphs run side by side; replays of one graph keep their order
+  return hipGraphLaunch(ge->exec, ge->stream) == hipSuccess ? AXHIP_OK : AXHIP_DEVICE_ERROR;
 }
 
 AXHIP_API int axhip_graph_sync(axhip_graph graph) {

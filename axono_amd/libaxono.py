@@ -665,6 +665,12 @@ def gqa_decode_attention_qkv(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, ep
 
 
 # ---- graph capture -------------------------------------------------------------------------------
+def set_ticket_lane(lane: int) -> None:
+    """Attention and wide argmax launches issued (or captured) from now on by this thread use the
+    ticket counters of `lane` (0..7); launches that overlap in time on the device need different lanes."""
+    check(_lib_().axhip_set_ticket_lane(int(lane)), "set_ticket_lane")
+
+
 class HIPGraph:
     """The binding-level graph object (the reference's CUDAGraph class, nanobind_module.cpp:1228-1324):
     capture(fn) = reset the capture pool, run fn once with pool recording on, begin capture, run fn
@@ -715,6 +721,14 @@ class HIPGraph:
         if self._graph is None:
             raise RuntimeError("launch() 之前必须先 capture()")
         check(_lib_().axhip_graph_launch(self._graph), "launch")
+
+    def launch_async(self) -> None:
+        """Enqueue one replay on the graph's own stream, unordered against the default stream: replays
+        of different graphs run side by side.  Such graphs are captured under different ticket lanes
+        (set_ticket_lane) and ordered with sync()."""
+        if self._graph is None:
+            raise RuntimeError("launch_async() 之前必须先 capture()")
+        check(_lib_().axhip_graph_launch_async(self._graph), "launch")
 
     def sync(self) -> None:
         if self._graph is not None:

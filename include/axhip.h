@@ -102,6 +102,16 @@ AXHIP_API int axhip_fill_zero(void *dst, size_t bytes);
 /* The stream operators should be given: the calling thread's capture stream while it captures,
  * else the legacy default stream.  Replaces cuda::AxonoCurrentStream, src/core/cuda/graph.cu:58-60. */
 AXHIP_API axhip_stream axhip_current_stream(void);
+
+/* Kernels that finish through static ticket counters (axhip_gqa_decode[_qkv] when it merges key
+ * ranges in the kernel, axhip_argmax over wide rows) take the counters of the calling thread's
+ * ticket lane, 0 .. AXHIP_TICKET_LANES-1 (default 0); a captured launch keeps the lane it was captured
+ * under.  Launches of these kernels that overlap in time on one device must come from different lanes.
+ * A lane holds 8192 (sequence, head group) slots for attention and 128 rows for argmax.  No
+ * reference counterpart (the reference merges in a second kernel, gqa.cu:95-129). */
+#define AXHIP_TICKET_LANES 8
+AXHIP_API int axhip_set_ticket_lane(int lane);
+AXHIP_API int axhip_ticket_lane(void);
 /* 1 while the calling thread is between axhip_graph_begin_capture and end/abort
  * (cuda::IsCapturing, include/axono/core/cuda/capture.h:19-33). */
 AXHIP_API int axhip_is_capturing(void);
@@ -124,6 +134,12 @@ AXHIP_API int axhip_graph_end_capture(axhip_stream stream, axhip_graph *graph_ou
                                       size_t *num_nodes_out);
 AXHIP_API int axhip_graph_abort_capture(axhip_stream stream);
 AXHIP_API int axhip_graph_launch(axhip_graph graph);
+/* One replay on the graph's own stream without any ordering against the default stream: replays of
+ * different graphs then run side by side on the device (replays of one graph keep their order).
+ * The caller orders them against other work with axhip_graph_sync.  Graphs that run side by side
+ * must have been captured under different ticket lanes (axhip_set_ticket_lane) if they hold
+ * attention or argmax launches.  No reference counterpart. */
+AXHIP_API int axhip_graph_launch_async(axhip_graph graph);
 AXHIP_API int axhip_graph_sync(axhip_graph graph);
 AXHIP_API int axhip_graph_destroy(axhip_graph graph);
 

@@ -318,6 +318,44 @@ def test_graph_capture_replay_semantics():
     np.testing.assert_allclose(axono.add(a, b).to_numpy(), b.to_numpy(), rtol=1e-6)
 
 
+def test_graphs_replayed_side_by_side_on_ticket_lanes():
+    """Two graphs, each with an attention launch that merges key ranges in the kernel and a wide argmax
+    (both finish through static ticket counters), captured under different ticket lanes and replayed
+    side by side on their own streams: every replay gives the eager result."""
+    rng = np.random.default_rng(5)
+    graphs, wants, inputs = [], [], []  # the graphs read their inputs at fixed addresses: they stay alive
+    for lane in (0, 1):
+        q = t(rng.standard_normal((1, 16, 128)).astype(np.float32))
+        k = t(rng.standard_normal((4096 + 512 * lane, 8, 128)).astype(np.float32))
+        v = t(rng.standard_normal((4096 + 512 * lane, 8, 128)).astype(np.float32))
+        x = t(rng.standard_normal((8, 40000)).astype(np.float32))
+
+        def body(q=q, k=k, v=v, x=x):
+            return axono.gqa_decode_attention(q, k, v), axono.argmax(x)
+
+        inputs.append((q, k, v, x))
+        wants.append([o.to_numpy().copy() for o in body()])
+        L.set_ticket_lane(lane)
+        try:
+            graphs.append(axono.HIPGraph().capture(body))
+        finally:
+            L.set_ticket_lane(0)
+    assert L._lib_().axhip_ticket_lane() == 0
+    with pytest.raises(RuntimeError):
+        L.set_ticket_lane(8)
+    for _ in range(4):
+        for _ in range(16):
+            for g in graphs:
+                g.launch_async()
+        for g in graphs:
+            g.sync()
+        for g, want in zip(graphs, wants):
+            np.testing.assert_allclose(g.outputs[0].to_numpy(), want[0], rtol=0, atol=1e-6)
+            np.testing.assert_array_equal(g.outputs[1].to_numpy(), want[1])
+    for g in graphs:
+        g.reset()
+
+
 def test_compile_caches_by_signature_and_refreshes_inputs():
     class Block(nn.Module):
         def __init__(self):

@@ -188,6 +188,14 @@ class Qwen3VLTextDecoder(nn.Module):
         act = L.linear_packed(xn, self._packed[name], self._w(name).shape[0], out_dtype=DataType.FLOAT16, glu=True)
         return self._linear(act, p + "mlp.down_proj.weight")
 
+    def forward(self, ids: Tensor, pos: Tensor):
+        """One decode step as a Module call, for `axono.compile(model)`: (logits, next ids).  Like
+        decode_forward it leaves the lengths alone, so running it again for the same step (the warm-up
+        and capture runs of compile) writes the same cache rows; the caller advances the cache
+        (`model.cache.advance()`) and the positions after each step, as the reference's loop does
+        (examples/vlm/qwen3vl/model.py:827-861)."""
+        return self.decode_forward(ids, pos)
+
     def decode_forward(self, ids: Tensor, pos: Tensor, attn_max_len: int | None = None, trace: list | None = None):
         """One token per sequence.  ids INT64 [B]; pos INT64 [3,B]; appends to the cache at
         cache.seq_lens and attends over seq_lens + 1 keys.  Returns (logits FLOAT32 [B,V], next ids

@@ -6,6 +6,7 @@ activation entering each Linear, q and the KV cache)."""
 import numpy as np
 import pytest
 
+from axono_amd import DataType, Tensor
 from axono_amd.examples.qwen3vl_text import Qwen3VLTextDecoder, TextConfig, random_weights
 from oracle.decode_step import OracleDecoder
 
@@ -75,6 +76,39 @@ def test_decode_steps_match_oracle(use_graph):
     for i in range(CFG.num_hidden_layers):
         kc = gpu.cache.get(i)[0].numpy()[:, :, S:S + n_steps].astype(np.float32)
         assert np.abs(kc - cpu.k[i][:, :, S:S + n_steps].astype(np.float32)).max() <= 4e-3
+
+
+def test_compiled_decode_loop_matches_the_captured_step():
+    """The reference's loop shape (examples/vlm/qwen3vl/model.py:827-861) over `axono.compile(model)`:
+    every step refreshes ids / positions in place, replays, and advances the cache from the host side.
+    Same tokens as the device-driven captured step."""
+    import axono_amd as axono
+    n_steps = 5
+    gpu, _, ids = _setup(seed=5)
+    B, S = ids.shape
+    _, g_next = gpu.prefill(ids)
+    first = g_next.to_numpy().copy()
+    gpu.start_decode(first, np.full((3, B), S, np.int64), n_steps)
+    gpu.capture()
+    want = gpu.generate(n_steps)
+
+    gpu2, _, _ = _setup(seed=5)
+    gpu2.prefill(ids)
+    compiled = axono.compile(gpu2)
+    cur = Tensor(DataType.INT64, [B], "hip:0")
+    pos = Tensor(DataType.INT64, [3, B], "hip:0")
+    tok = first
+    got = []
+    for s in range(n_steps):
+        cur.copy_from_numpy(tok)
+        pos.copy_from_numpy(np.full((3, B), S + s, np.int64))
+        logits, nxt = compiled(cur, pos)
+        tok = nxt.to_numpy().copy()
+        got.append(tok)
+        gpu2.cache.advance(1)
+    np.testing.assert_array_equal(np.stack(got), want)
+    np.testing.assert_array_equal(gpu2.cache.seq_lens.to_numpy(), [S + n_steps] * B)
+    assert len(compiled._graphs) == 1
 
 
 def test_eager_and_graph_logits_agree_every_replay():

@@ -45,6 +45,7 @@ PROTOTYPES = {
     "axhip_graph_abort_capture": (c_i, [c_vp]),
     "axhip_graph_launch": (c_i, [c_vp]),
     "axhip_graph_launch_async": (c_i, [c_vp]),
+    "axhip_graph_replay": (c_i, [c_vp]),
     "axhip_set_ticket_lane": (c_i, [c_i]),
     "axhip_ticket_lane": (c_i, []),
     "axhip_graph_sync": (c_i, [c_vp]),

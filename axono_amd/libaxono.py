@@ -712,9 +712,7 @@ class HIPGraph:
     def replay(self) -> None:
         if self._graph is None:
             raise RuntimeError("replay() 之前必须先 capture()")
-        lib = _lib_()
-        check(lib.axhip_graph_launch(self._graph), "replay")
-        check(lib.axhip_graph_sync(self._graph), "replay")
+        check(_lib_().axhip_graph_replay(self._graph), "replay")
 
     def launch(self) -> None:
         """Enqueue one replay without waiting (a serving loop syncs once per many steps)."""

@@ -140,6 +140,9 @@ AXHIP_API int axhip_graph_launch(axhip_graph graph);
  * must have been captured under different ticket lanes (axhip_set_ticket_lane) if they hold
  * attention or argmax launches.  No reference counterpart. */
 AXHIP_API int axhip_graph_launch_async(axhip_graph graph);
+/* One replay that has finished when the call returns, after all earlier default-stream work: the
+ * reference's CudaGraphExec::Replay (launch + stream synchronise, src/core/cuda/graph.cu:123-139). */
+AXHIP_API int axhip_graph_replay(axhip_graph graph);
 AXHIP_API int axhip_graph_sync(axhip_graph graph);
 AXHIP_API int axhip_graph_destroy(axhip_graph graph);
 

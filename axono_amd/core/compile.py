@@ -1,50 +1,65 @@
-"""`compile(model)`: capture the model's forward into a hipGraph keyed by the call signature and
-replay it afterwards.  Mirrors axono/python/axono/core/compile.py:52-174 (mode "normal"): the first
-call with a new signature runs the model once eagerly (warm-up), captures it with the inputs of
-that call as static buffers, and every call refreshes those buffers in place and replays.
-Outputs are the captured call's tensors and are overwritten by the next replay.
+"""`compile(model)`: the model's forward as a replayed hipGraph.
+
+Behaviour follows axono/python/axono/core/compile.py:52-174 (mode "normal"): calls are told apart
+by the shapes, dtypes and devices of their tensor arguments and the values of the others; the first
+call of a kind runs the model once as it is, then captures it with that call's tensors as the
+graph's fixed input buffers; every call of that kind copies its tensors into those buffers (unless
+they are the buffers) and replays.  The results are the captured call's output tensors: the next
+replay overwrites them.
 """
 from __future__ import annotations
 
-from .. import libaxono as _l
+from .. import libaxono as _table
 from .hip_graph import HIPGraph
 
 
-class _TensorArg:
-    __slots__ = ("tensor",)
-
-    def __init__(self, tensor):
-        self.tensor = tensor
-
-    def copy_in(self, value):
-        if value is not self.tensor:
-            self.tensor.copy_from(value)
+def _tensor_like(value) -> bool:
+    return hasattr(value, "shape") and hasattr(value, "dtype")
 
 
-def _is_tensor(a):
-    return hasattr(a, "shape") and hasattr(a, "dtype")
+def _describe(value):
+    """What distinguishes one call from another: a tensor's geometry, anything else by its repr."""
+    if _tensor_like(value):
+        return "tensor", tuple(value.shape), str(value.dtype), str(value.device)
+    return "value", repr(value)
 
 
-def _sig_of(args, kwargs):
-    parts = []
-    for a in args:
-        parts.append(("T", tuple(a.shape), str(a.dtype), str(a.device)) if _is_tensor(a) else ("S", repr(a)))
-    for k in sorted(kwargs):
-        v = kwargs[k]
-        parts.append((k, "T", tuple(v.shape), str(v.dtype), str(v.device)) if _is_tensor(v) else (k, "S", repr(v)))
-    return tuple(parts)
+def _call_key(args, kwargs) -> tuple:
+    return tuple(_describe(a) for a in args) + tuple((name,) + _describe(kwargs[name]) for name in sorted(kwargs))
+
+
+class _CapturedCall:
+    """The graph of one kind of call and the tensors it reads its inputs from."""
+
+    def __init__(self, model, args, kwargs):
+        self.positional = list(args)
+        self.named = dict(kwargs)
+        self.graph = HIPGraph()
+        self.graph.capture(lambda: model(*self.positional, **self.named))
+
+    def run(self, args, kwargs):
+        for fixed, given in zip(self.positional, args):
+            if _tensor_like(fixed) and given is not fixed:
+                fixed.copy_from(given)
+        for name, fixed in self.named.items():
+            if _tensor_like(fixed) and kwargs[name] is not fixed:
+                fixed.copy_from(kwargs[name])
+        self.graph.replay()
+        results = self.graph.outputs
+        return results[0] if len(results) == 1 else tuple(results)
 
 
 class CompiledModel:
     def __init__(self, model, mode: str = "normal"):
         if mode != "normal":
-            raise ValueError(f"axono.compile: 暂不支持 mode={mode!r} (目前只有 'normal')")
-        if not _l.hip_available():
-            raise RuntimeError("axono.compile 需要可用的 HIP 设备")
+            raise ValueError(f"axono.compile: mode {mode!r} is not supported (only 'normal')")
+        if not _table.hip_available():
+            raise RuntimeError("axono.compile needs a HIP device")
         self._model = model
         self._mode = mode
-        self._graphs = {}
+        self._graphs = {}  # call key -> _CapturedCall
 
+    # everything that is not the wrapper's own state is the model's
     def __getattr__(self, name):
         return getattr(object.__getattribute__(self, "_model"), name)
 
@@ -54,39 +69,19 @@ class CompiledModel:
         else:
             setattr(object.__getattribute__(self, "_model"), name, value)
 
-    def _build(self, args, kwargs):
-        static_args = [_TensorArg(a) if _is_tensor(a) else a for a in args]
-        static_kwargs = {k: (_TensorArg(v) if _is_tensor(v) else v) for k, v in kwargs.items()}
-        g = HIPGraph()
-        g.capture(lambda: self._model(
-            *[s.tensor if isinstance(s, _TensorArg) else s for s in static_args],
-            **{k: (s.tensor if isinstance(s, _TensorArg) else s) for k, s in static_kwargs.items()}))
-        return g, static_args, static_kwargs
-
     def __call__(self, *args, **kwargs):
-        sig = _sig_of(args, kwargs)
-        entry = self._graphs.get(sig)
-        if entry is None:
-            self._model(*args, **kwargs)  # warm-up on the real inputs
-            entry = self._build(args, kwargs)
-            self._graphs[sig] = entry
-        g, static_args, static_kwargs = entry
-        for s, a in zip(static_args, args):
-            if isinstance(s, _TensorArg):
-                s.copy_in(a)
-        for k, s in static_kwargs.items():
-            if isinstance(s, _TensorArg):
-                s.copy_in(kwargs[k])
-        g.replay()
-        outs = g.outputs
-        return outs[0] if len(outs) == 1 else tuple(outs)
+        key = _call_key(args, kwargs)
+        captured = self._graphs.get(key)
+        if captured is None:
+            self._model(*args, **kwargs)  # once as it is: lazy initialisation happens outside the capture
+            captured = self._graphs[key] = _CapturedCall(self._model, args, kwargs)
+        return captured.run(args, kwargs)
 
     def forward(self, *args, **kwargs):
         return self(*args, **kwargs)
 
     def __repr__(self):
-        inner = repr(object.__getattribute__(self, "_model"))
-        return f"CompiledModel(mode={self._mode!r}, graphs={len(self._graphs)}, model={inner})"
+        return f"CompiledModel(mode={self._mode!r}, graphs={len(self._graphs)}, model={self._model!r})"
 
 
 def compile(model, mode: str = "normal"):  # noqa: A001 - the reference's name

@@ -7,7 +7,7 @@ import pytest
 
 import axono_amd as axono
 from axono_amd import DataType, Status, Tensor, nn
-from axono_amd.core.compile import _sig_of
+from axono_amd.core.compile import _call_key
 from axono_amd.core.tensor import parse_device
 from axono_amd.device import AxhipError
 
@@ -181,9 +181,9 @@ def test_dynamic_kv_cache_bookkeeping():
 
 def test_compile_signature_keys():
     a, b = Tensor.zeros([2, 3]), Tensor.zeros([2, 3])
-    assert _sig_of((a, 1), {"x": b}) == _sig_of((b, 1), {"x": a})
-    assert _sig_of((a,), {}) != _sig_of((Tensor.zeros([3, 2]),), {})
-    assert _sig_of((a, 1), {}) != _sig_of((a, 2), {})
-    assert _sig_of((a,), {}) != _sig_of((Tensor.zeros([2, 3], DataType.FLOAT16),), {})
+    assert _call_key((a, 1), {"x": b}) == _call_key((b, 1), {"x": a})
+    assert _call_key((a,), {}) != _call_key((Tensor.zeros([3, 2]),), {})
+    assert _call_key((a, 1), {}) != _call_key((a, 2), {})
+    assert _call_key((a,), {}) != _call_key((Tensor.zeros([2, 3], DataType.FLOAT16),), {})
     with pytest.raises(ValueError):
         axono.compile(lambda x: x, mode="max")

@@ -331,6 +331,53 @@ def test_argmax_embedding_add():
 
 # ---- the restatement against the compiled reference, bit for bit ------------------------------
 @needs_ref
+@pytest.mark.parametrize("seed", range(12))
+def test_port_equals_reference_bitwise_over_random_shapes(seed):
+    """Odd sizes, group sizes 1..4, causal and not, more keys than queries and fewer: the restatement and
+    the reference's own C++ agree in every bit."""
+    rng = np.random.default_rng(7000 + seed)
+    hkv = int(rng.integers(1, 4))
+    group = int(rng.integers(1, 5))
+    d = int(rng.choice([2, 6, 8, 20, 64, 128]))
+    sq, skv = int(rng.integers(1, 12)), int(rng.integers(1, 40))
+    q = rng.standard_normal((sq, hkv * group, d)).astype(np.float32)
+    k = rng.standard_normal((skv, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((skv, hkv, d)).astype(np.float32)
+    for causal in (False, True):
+        np.testing.assert_array_equal(port.sdpa(q, k, v, causal), REF.sdpa(q, k, v, causal))
+    rows, hidden = int(rng.integers(1, 9)), int(rng.integers(1, 300))
+    x = (3 * rng.standard_normal((rows, hidden))).astype(np.float32)
+    r = rng.standard_normal((rows, hidden)).astype(np.float32)
+    w = rng.standard_normal(hidden).astype(np.float32)
+    eps = float(rng.choice([1e-6, 1e-5, 1e-3]))
+    for a, b in zip(port.add_rms_norm(x, r, w, eps), REF.add_rms_norm(x, r, w, eps)):
+        np.testing.assert_array_equal(a, b)
+    np.testing.assert_array_equal(port.rms_norm(x, w, eps), REF.rms_norm(x, w, eps))
+    np.testing.assert_array_equal(port.silu_mul(10 * x, r), REF.silu_mul(10 * x, r))
+    heads, dh = int(rng.integers(1, 5)), 2 * int(rng.integers(1, 40))
+    xr = rng.standard_normal((rows, heads, dh)).astype(np.float32)
+    pos = rng.integers(0, 100000, rows).astype(np.int64)
+    theta = float(rng.choice([1e4, 1e6, 5e6]))
+    np.testing.assert_array_equal(port.rope(xr, pos, theta), REF.rope(xr, pos, theta))
+    inv = port.rope_inv_freq(theta, dh)
+    pos3 = rng.integers(0, 100000, (3, rows)).astype(np.int64)
+    half = dh // 2
+    h_sec, w_sec = int(rng.integers(0, half // 3 + 1)), int(rng.integers(0, half // 3 + 1))
+    sec = [half - h_sec - w_sec, h_sec, w_sec]
+    np.testing.assert_array_equal(port.rope_thd(xr, pos3, inv, sec), REF.rope_thd(xr, pos3, inv, sec))
+    c, s_ = REF.mrope_cos_sin(pos3, inv, h_sec, w_sec)
+    for a, b in zip(port.mrope_cos_sin(pos3, inv, h_sec, w_sec), (c, s_)):
+        np.testing.assert_array_equal(a, b)
+    np.testing.assert_array_equal(port.rope_with_cos_sin(xr, c, s_), REF.rope_with_cos_sin(xr, c, s_))
+    m, kk, n = int(rng.integers(1, 20)), int(rng.integers(1, 70)), int(rng.integers(1, 30))
+    xl = rng.standard_normal((m, kk)).astype(np.float32)
+    wl = rng.standard_normal((n, kk)).astype(np.float32)
+    bl = rng.standard_normal(n).astype(np.float32)
+    np.testing.assert_array_equal(port.linear(xl, wl, bl), REF.linear(xl, wl, bl))
+    np.testing.assert_array_equal(port.linear(xl, wl), REF.linear(xl, wl))
+
+
+@needs_ref
 def test_port_equals_reference_bitwise():
     rng = np.random.default_rng(2024)
     q = rng.standard_normal((1, 16, 128)).astype(np.float32)

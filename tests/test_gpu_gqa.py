@@ -420,3 +420,41 @@ def test_workgroups_are_dealt_by_length():
         want = port.gqa_decode_cache_native(q, k, v, lens)
         assert np.abs(out - want).max() <= TOL16, lens
         assert np.all(out[lens == 0] == 0)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_configurations_against_the_oracle(seed):
+    """Batch, head counts (1 to 8 query heads per kv head: the vector kernel and the matrix-core kernel),
+    head size, cache capacity, lengths (zeros included) and dtype drawn at random."""
+    rng = np.random.default_rng(9100 + seed)
+    B = int(rng.integers(1, 10))
+    hkv = int(rng.integers(1, 4))
+    group = int(rng.choice([1, 2, 3, 4, 5, 8]))
+    d = int(rng.choice([64, 128, 256]))
+    lmax = int(rng.choice([1, 17, 130, 700, 2100]))
+    dtype = np.float16 if rng.integers(0, 2) else np.float32
+    lens = rng.integers(0, lmax + 1, B).astype(np.int32)
+    if rng.integers(0, 3) == 0:
+        lens[:] = lmax
+    q = rng.standard_normal((B, hkv * group, d)).astype(np.float32).astype(dtype)
+    k = rng.standard_normal((B, hkv, lmax, d)).astype(np.float32).astype(dtype)
+    v = rng.standard_normal((B, hkv, lmax, d)).astype(np.float32).astype(dtype)
+    got = gqa_decode(q, k, v, seq_lens=lens).astype(np.float32)
+    want = port.gqa_decode_cache(q, k, v, lens)
+    tol = TOL16 if dtype == np.float16 else TOL32
+    assert np.abs(got - want).max() <= tol, (B, hkv, group, d, lmax, dtype, lens, np.abs(got - want).max())
+    assert np.all(got[lens == 0] == 0)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_decode_step_form_random_configurations(seed):
+    """The decode-step form (q/k norm, M-RoPE and append in the attention launch) over random batches,
+    head shapes, capacities and lengths, with the plan left to the library."""
+    rng = np.random.default_rng(9300 + seed)
+    B = int(rng.integers(1, 9))
+    hkv = int(rng.integers(1, 4))
+    group = int(rng.choice([1, 2, 4, 8]))
+    d = int(rng.choice([64, 128]))
+    rows = int(rng.choice([16, 200, 900, 2304]))
+    lens = rng.integers(0, rows, B)  # at least one free row everywhere
+    _check_decode_step_form(hkv * group, hkv, d, lens, rows, rows, forced=(0,), seed=seed)

@@ -257,3 +257,28 @@ def test_packed_gemm_256x128_tile(M, K, N):
     gu_ = port.linear(x.astype(np.float32), w[:n2].astype(np.float32))
     wantg = port.silu_mul(np.ascontiguousarray(gu_[:, : n2 // 2]), np.ascontiguousarray(gu_[:, n2 // 2:]))
     np.testing.assert_allclose(glu, wantg, rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_packed_linear_random_shapes(seed):
+    """Rows, K (a multiple of 8), columns, bias, activation dtype and output dtype at random: every route
+    (weight-streaming kernels, tiled GEMMs of every tile size, their edge handling) against the oracle."""
+    rng = np.random.default_rng(9500 + seed)
+    M = int(rng.choice([1, 5, 16, 31, 32, 33, 64, 65, 130, 300, 520]))
+    K = 8 * int(rng.integers(1, 200))
+    if rng.integers(0, 3) == 0:
+        K = 128 * int(rng.integers(1, 17))
+    N = int(rng.choice([1, 7, 16, 50, 64, 257, 700, 2048, 2300]))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    if rng.integers(0, 2):
+        x = h16(x)
+    w = h16(0.05 * rng.standard_normal((N, K)))
+    b = h16(0.05 * rng.standard_normal(N)) if rng.integers(0, 2) else None
+    xr = x.astype(np.float16).astype(np.float32)
+    want = port.linear(xr, w.astype(np.float32), None if b is None else b.astype(np.float32))
+    mag = np.abs(xr) @ np.abs(w.astype(np.float32)).T + (0 if b is None else np.abs(b.astype(np.float32)))
+    got = gu.linear_f16_packed(x, w, b)
+    assert np.all(np.abs(got - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag), (M, K, N)
+    got16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16).astype(np.float32)
+    ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
+    assert np.all(np.abs(got16 - want) <= 0.5 * ulp + 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag), (M, K, N)

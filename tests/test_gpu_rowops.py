@@ -448,3 +448,52 @@ def test_decode_advance():
     assert l.axhip_decode_advance(None, d_ids.ptr, None, 0, None, None, 0, None, 4, None) == 7
     assert l.axhip_decode_advance(d_nxt.ptr, d_ids.ptr, None, 3, None, None, 0, None, 4, None) == 7
     assert l.axhip_decode_advance(d_nxt.ptr, d_ids.ptr, None, 0, None, None, 0, None, -1, None) == 1
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_row_operators_random_shapes(seed):
+    """Rows and widths at random (widths that are not multiples of 8 take the scalar paths), fp32 and
+    fp16: add_rms_norm, rms_norm, silu_mul, rope, rope_thd and the cos/sin table form."""
+    rng = np.random.default_rng(9700 + seed)
+    rows = int(rng.integers(1, 70))
+    hidden = int(rng.choice([1, 5, 8, 72, 250, 512, 1000, 2048, 5000]))
+    half = bool(rng.integers(0, 2))
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    r = rng.standard_normal((rows, hidden)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    if half:
+        xh, rh = h16(x), h16(r)
+        y, out = gu.add_rms_norm(xh, rh, w, 1e-6)
+        wy, wout = port.add_rms_norm(xh.astype(np.float32), rh.astype(np.float32), w, 1e-6)
+        assert_fp16_close(y, wy)
+        # the norm is computed from the fp32 sum, not from the rounded y
+        assert_fp16_close(out, wout)
+        assert_fp16_close(gu.silu_mul(xh, rh), port.silu_mul(xh.astype(np.float32), rh.astype(np.float32)))
+    else:
+        y, out = gu.add_rms_norm(x, r, w, 1e-6)
+        wy, wout = port.add_rms_norm(x, r, w, 1e-6)
+        np.testing.assert_array_equal(y, wy)
+        np.testing.assert_allclose(out, wout, rtol=0, atol=TOL32 * max(1.0, float(np.abs(wout).max())))
+        np.testing.assert_allclose(gu.rms_norm(x, w, 1e-5), port.rms_norm(x, w, 1e-5), rtol=0,
+                                   atol=TOL32 * max(1.0, float(np.abs(wout).max())))
+        np.testing.assert_allclose(gu.silu_mul(x, r), port.silu_mul(x, r), rtol=2e-6, atol=1e-6)
+    heads, d = int(rng.integers(1, 20)), 2 * int(rng.choice([1, 4, 16, 32, 40, 64, 128]))
+    xr = rng.standard_normal((rows, heads, d)).astype(np.float32)
+    pos = rng.integers(0, 8192, rows).astype(np.int64)
+    pos3 = rng.integers(0, 8192, (3, rows)).astype(np.int64)
+    inv = port.rope_inv_freq(1e6, d)
+    h_sec = w_sec = (d // 2) // 3
+    sec = [d // 2 - 2 * h_sec, h_sec, w_sec]
+    if half:
+        xrh = h16(xr)
+        f = xrh.astype(np.float32)
+        assert_fp16_close(gu.rope(xrh, pos, 1e6), port.rope(f, pos, 1e6))
+        assert_fp16_close(gu.rope_thd(xrh, pos3, inv, sec), port.rope_thd(f, pos3, inv, sec))
+    else:
+        np.testing.assert_allclose(gu.rope(xr, pos, 1e6), port.rope(xr, pos, 1e6), rtol=0, atol=2e-5)
+        np.testing.assert_allclose(gu.rope_thd(xr, pos3, inv, sec), port.rope_thd(xr, pos3, inv, sec), rtol=0, atol=2e-5)
+        c, s_ = gu.mrope_cos_sin(pos3, inv, h_sec, w_sec)
+        wc, ws = port.mrope_cos_sin(pos3, inv, h_sec, w_sec)
+        np.testing.assert_allclose(c, wc, rtol=0, atol=2e-5)
+        np.testing.assert_allclose(s_, ws, rtol=0, atol=2e-5)
+        np.testing.assert_allclose(gu.rope_with_cos_sin(xr, wc, ws), port.rope_with_cos_sin(xr, wc, ws), rtol=0, atol=TOL32)

@@ -497,3 +497,54 @@ def test_row_operators_random_shapes(seed):
         np.testing.assert_allclose(c, wc, rtol=0, atol=2e-5)
         np.testing.assert_allclose(s_, ws, rtol=0, atol=2e-5)
         np.testing.assert_allclose(gu.rope_with_cos_sin(xr, wc, ws), port.rope_with_cos_sin(xr, wc, ws), rtol=0, atol=TOL32)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_general_attention_random_shapes(seed):
+    """Query / key counts, head counts and head sizes at random, causal and not, fp32 and fp16: the
+    matrix-core route (fp16, head size 64 / 128, 32 or more query rows), the split-K route and the
+    plain kernel for other head sizes."""
+    rng = np.random.default_rng(9900 + seed)
+    sq = int(rng.choice([1, 3, 31, 32, 33, 64, 130, 257]))
+    skv = int(rng.choice([1, 5, 64, 100, 257, 600]))
+    hkv = int(rng.integers(1, 4))
+    group = int(rng.choice([1, 2, 3, 4]))
+    d = int(rng.choice([8, 32, 64, 128, 256]))
+    half = bool(rng.integers(0, 2))
+    q = rng.standard_normal((sq, hkv * group, d)).astype(np.float32)
+    k = rng.standard_normal((skv, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((skv, hkv, d)).astype(np.float32)
+    for causal in (False, True):
+        if half:
+            qh, kh, vh = h16(q), h16(k), h16(v)
+            want = port.sdpa(qh.astype(np.float32), kh.astype(np.float32), vh.astype(np.float32), causal)
+            assert_fp16_close(gu.sdpa(qh, kh, vh, causal), want)
+        else:
+            np.testing.assert_allclose(gu.sdpa(q, k, v, causal), port.sdpa(q, k, v, causal), rtol=0, atol=TOL32)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_cache_and_index_operators_random_shapes(seed):
+    rng = np.random.default_rng(9950 + seed)
+    B, hkv, lmax, d = int(rng.integers(1, 9)), int(rng.integers(1, 5)), int(rng.integers(1, 300)), int(rng.choice([8, 64, 128]))
+    dtype = np.float16 if rng.integers(0, 2) else np.float32
+    kc = rng.standard_normal((B, hkv, lmax, d)).astype(dtype)
+    vc = rng.standard_normal((B, hkv, lmax, d)).astype(dtype)
+    kn = rng.standard_normal((B, hkv, d)).astype(dtype)
+    vn = rng.standard_normal((B, hkv, d)).astype(dtype)
+    pos = rng.integers(0, lmax, B).astype(np.int64)
+    wk, wv = kc.copy(), vc.copy()
+    port.kv_append(kn, vn, wk, wv, pos)
+    gk, gv = gu.kv_append(kn, vn, kc, vc, pos)
+    np.testing.assert_array_equal(gk.view(np.uint8), wk.view(np.uint8))
+    np.testing.assert_array_equal(gv.view(np.uint8), wv.view(np.uint8))
+    a = rng.standard_normal((int(rng.integers(1, 50)), hkv, d)).astype(dtype)
+    b = rng.standard_normal((int(rng.integers(1, 5)), hkv, d)).astype(dtype)
+    np.testing.assert_array_equal(gu.concat_axis0(a, b).view(np.uint8), np.concatenate([a, b], 0).view(np.uint8))
+    vocab, dim = int(rng.integers(2, 3000)), int(rng.choice([4, 64, 100]))
+    table = rng.standard_normal((vocab, dim)).astype(dtype)
+    ids = rng.integers(0, vocab, (int(rng.integers(1, 6)), int(rng.integers(1, 9)))).astype(np.int64)
+    np.testing.assert_array_equal(gu.embedding(ids, table).view(np.uint8), table[ids].view(np.uint8))
+    cols = int(rng.choice([1, 7, 1000, 16384, 40000]))
+    lg = rng.standard_normal((int(rng.integers(1, 20)), cols)).astype(np.float32)
+    np.testing.assert_array_equal(gu.argmax(lg), np.argmax(lg, -1))

@@ -373,7 +373,7 @@ def test_prefill_attention_matches_causal_oracle(Hq, Hkv, D, S, start):
         L = start[b] + S
         k = np.ascontiguousarray(np.transpose(kc[b, :, :L], (1, 0, 2)), dtype=np.float32)   # [L, Hkv, D]
         v = np.ascontiguousarray(np.transpose(vc[b, :, :L], (1, 0, 2)), dtype=np.float32)
-        for i in sorted({0, 1, 15, 16, 63, min(64, S - 1), S // 2, S - 2, S - 1}):
+        for i in sorted(i for i in {0, 1, 15, 16, 63, min(64, S - 1), S // 2, S - 2, S - 1} if 0 <= i < S):
             vis = start[b] + i + 1
             want = port.sdpa(q[b, i:i + 1].astype(np.float32), k[:vis], v[:vis], False)[0]
             worst = max(worst, float(np.abs(got[b, i] - want).max()))
@@ -458,3 +458,14 @@ def test_decode_step_form_random_configurations(seed):
     rows = int(rng.choice([16, 200, 900, 2304]))
     lens = rng.integers(0, rows, B)  # at least one free row everywhere
     _check_decode_step_form(hkv * group, hkv, d, lens, rows, rows, forced=(0,), seed=seed)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_prefill_attention_random_configurations(seed):
+    rng = np.random.default_rng(9800 + seed)
+    hkv = int(rng.integers(1, 4))
+    group = int(rng.choice([1, 2, 3, 4, 8]))
+    d = int(rng.choice([64, 128]))
+    S = int(rng.choice([1, 17, 64, 100, 200, 333]))
+    start = [int(s) for s in rng.choice([0, 1, 63, 64, 150], int(rng.integers(1, 4)))]
+    test_prefill_attention_matches_causal_oracle(hkv * group, hkv, d, S, start)

@@ -187,3 +187,21 @@ def test_compile_signature_keys():
     assert _call_key((a,), {}) != _call_key((Tensor.zeros([2, 3], DataType.FLOAT16),), {})
     with pytest.raises(ValueError):
         axono.compile(lambda x: x, mode="max")
+
+
+def test_missing_library_raises_instead_of_falling_back(monkeypatch, tmp_path):
+    """Without libaxhip.so (and with nothing to build it from) loading raises; there is no other path."""
+    from axono_amd import _lib
+
+    def cannot_build():
+        raise RuntimeError("hipcc not available")
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libaxhip.so"))
+    monkeypatch.setattr(_lib._build, "build_library", cannot_build)
+    with pytest.raises(RuntimeError):
+        _lib.load()
+    # a file that is not the library
+    (tmp_path / "libaxhip.so").write_bytes(b"not a shared object")
+    with pytest.raises(RuntimeError):
+        _lib.load()

@@ -57,12 +57,14 @@ def hip_available() -> bool:
 class _Storage:
     """Shared by every alias of a tensor (the reference's shared_ptr<void>)."""
 
-    __slots__ = ("host", "dev", "keep")
+    __slots__ = ("host", "dev", "keep", "version")
 
     def __init__(self, host=None, dev=None, keep=None):
         self.host = host  # np.ndarray of uint8, or None
         self.dev = dev    # DeviceBuffer, or None
         self.keep = keep  # object kept alive for borrowed host memory
+        self.version = 0  # bumped by every host-initiated write (copy_from, copy_from_numpy, fill*):
+        #                   holders of data derived from the contents (packed Linear weights) compare it
 
 
 def _numel(shape):
@@ -172,6 +174,7 @@ class Tensor:
         n = self.num_bytes
         if n == 0:
             return self
+        self._st.version += 1
         lib = _lib.load()
         if self._kind == "cpu" and src._kind == "cpu":
             self._st.host[:n] = src._st.host[:n]
@@ -229,6 +232,7 @@ class Tensor:
         return self
 
     def fill_zero(self) -> "Tensor":
+        self._st.version += 1
         if self._kind == "cpu":
             self._st.host[:] = 0
         elif self.num_bytes:
@@ -301,6 +305,7 @@ class Tensor:
         n = self.num_bytes
         if n == 0:
             return self
+        self._st.version += 1
         if self._kind == "cpu":
             self._st.host[:n] = array.reshape(-1).view(np.uint8)
         else:

@@ -554,7 +554,11 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
 
   // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
   __shared__ int s_last;
-  __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
+  // A workgroup barrier orders the wavefronts but does not wait for their outstanding stores: every
+  // thread drains its own write-through partial stores first, so that all of them have reached memory
+  // when thread 0 takes the ticket behind the barrier.
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
   if (tid == 0) {
     unsigned int *ticket = &g_tickets[a.ticket_base + b * a.n_hg + hg];
     const unsigned int t = atomicAdd(ticket, 1u);
@@ -641,7 +645,10 @@ __device__ __forceinline__ void finish_range(const DecodeArgs &a, int b, int hg,
   if (n_valid == 1 || !a.fused_merge) return;
 
   // ---- in-kernel merge: the workgroup that takes the last ticket combines all splits ------------
-  __syncthreads();  // every wavefront's partial stores have completed before the ticket is taken
+  // every thread drains its own write-through partial stores before the barrier (the barrier alone
+  // does not wait for outstanding stores), so all partials are in memory when the ticket is taken
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
   if (tid == 0) {
     unsigned int *ticket = &g_tickets[a.ticket_base + b * a.n_hg + hg];
     const unsigned int t = atomicAdd(ticket, 1u);

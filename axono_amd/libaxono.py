@@ -189,6 +189,18 @@ def slice(x: Tensor, axis: int, start: int, length: int) -> Tensor:  # noqa: A00
     return out
 
 
+def copy_bytes(dst: Tensor, dst_offset: int, src: Tensor, src_offset: int, nbytes: int) -> None:
+    """dst bytes [dst_offset, +nbytes) = src bytes [src_offset, +nbytes), device to device on the current
+    stream (the axis-0 copy Concat is made of, src/ops/cuda/sequence.cu:500-518).  Used by the KV-cache
+    components to append rows in place."""
+    op = "copy_bytes"
+    _need_hip(op, dst, src)
+    if min(dst_offset, src_offset, nbytes) < 0 or dst_offset + nbytes > dst.num_bytes or src_offset + nbytes > src.num_bytes:
+        raise AxhipError(op, Status.INVALID_ARGUMENT)
+    if nbytes:
+        check(_lib_().axhip_memcpy_d2d(dst.data_ptr + dst_offset, src.data_ptr + src_offset, nbytes), op)
+
+
 def kv_append(k_new: Tensor, v_new: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor) -> None:
     """In place: cache[b,h,pos[b],:] = new[b,h,:] for K and V.  Replaces the concat-append of
     DynamicKVCache.update (axono/python/axono/nn/kv_cache.py:96-102) for a static cache."""

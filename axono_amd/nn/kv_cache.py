@@ -1,7 +1,7 @@
 """KV-cache components (axono/python/axono/nn/kv_cache.py).
 
-`KVCache` is the abstract interface; `DynamicKVCache` is the reference's default (per layer, the
-full k / v tensors, grown by concat along axis 0 — a byte copy, layout (seq, n_kv_head, d_head)).
+`KVCache` is the abstract interface; `DynamicKVCache` is the default component (per layer, the
+full k / v tensors, layout (seq, n_kv_head, d_head), grown along axis 0 by byte copies).
 `StaticKVCache` is this build's cache for the captured decode step: one pre-allocated
 [B, n_kv_head, max_len, d_head] tensor pair per layer, device-resident lengths, and an append that
 writes one row per (sequence, head) instead of re-copying the cache.
@@ -16,48 +16,119 @@ from ..core.types import DataType
 
 
 class KVCache:
-    def update(self, layer_idx: int, k_new, v_new):  # pragma: no cover
-        raise NotImplementedError
+    """Interface of a KV-cache component (axono/python/axono/nn/kv_cache.py:41-68).  A model's attention
+    layer calls `update(layer, k_new, v_new)` with the new tokens' keys / values and then
+    `get(layer)` for everything cached so far; `reset()` starts a new conversation and `len()` is
+    the number of cached positions.  User-written components subclass this."""
 
-    def get(self, layer_idx: int):  # pragma: no cover
-        raise NotImplementedError
+    def update(self, layer_idx: int, k_new, v_new):  # pragma: no cover - interface
+        raise NotImplementedError(f"{type(self).__name__}.update")
 
-    def reset(self):  # pragma: no cover
-        raise NotImplementedError
+    def get(self, layer_idx: int):  # pragma: no cover - interface
+        raise NotImplementedError(f"{type(self).__name__}.get")
 
-    def __len__(self) -> int:  # pragma: no cover
-        raise NotImplementedError
+    def reset(self):  # pragma: no cover - interface
+        raise NotImplementedError(f"{type(self).__name__}.reset")
+
+    def __len__(self) -> int:  # pragma: no cover - interface
+        raise NotImplementedError(f"{type(self).__name__}.__len__")
+
+
+class _GrowableRows:
+    """One tensor of rows (seq, ...) that grows along axis 0: a buffer with spare capacity plus the
+    number of rows in use.  Appending copies only the new rows (byte copy at the end of the used
+    part); the buffer is re-allocated with twice the capacity when it runs out, so the cost of n
+    appends is O(n) rows moved instead of the O(n^2) of a concat per step."""
+
+    __slots__ = ("buf", "rows", "row_shape")
+
+    def __init__(self, first: Tensor, capacity: int):
+        self.row_shape = first.shape[1:]
+        self.rows = 0
+        self.buf = Tensor(first.dtype, [capacity] + self.row_shape, first.device, _zero=False)
+        self.append(first)
+
+    def _row_bytes(self) -> int:
+        return self.buf.num_bytes // self.buf.shape[0]
+
+    def _copy_rows(self, dst: Tensor, dst_row: int, src: Tensor, n_rows: int) -> None:
+        nbytes = n_rows * self._row_bytes()
+        if nbytes == 0:
+            return
+        if dst.is_hip:
+            _l.copy_bytes(dst, dst_row * self._row_bytes(), src, 0, nbytes)
+        else:
+            d = dst.to_numpy().reshape(-1).view(np.uint8)
+            s = src.to_numpy().reshape(-1).view(np.uint8)
+            d[dst_row * self._row_bytes():dst_row * self._row_bytes() + nbytes] = s[:nbytes]
+
+    def append(self, new: Tensor) -> None:
+        if new.shape[1:] != self.row_shape or new.dtype != self.buf.dtype:
+            raise RuntimeError(f"KV cache append: rows of shape {new.shape[1:]} / {new.dtype.name} do not match the "
+                               f"cached {self.row_shape} / {self.buf.dtype.name}")
+        add = int(new.shape[0])
+        cap = int(self.buf.shape[0])
+        if self.rows + add > cap:
+            bigger = Tensor(self.buf.dtype, [max(2 * cap, self.rows + add)] + self.row_shape, self.buf.device, _zero=False)
+            self._copy_rows(bigger, 0, self.buf, self.rows)
+            self.buf = bigger
+        self._copy_rows(self.buf, self.rows, new, add)
+        self.rows += add
+
+    def view(self) -> Tensor:
+        """The rows in use as a tensor [rows, ...] sharing the buffer's memory (a prefix of a
+        contiguous row-major buffer is itself contiguous)."""
+        return Tensor(self.buf.dtype, [self.rows] + self.row_shape, self.buf.device, _storage=self.buf._st)
 
 
 class DynamicKVCache(KVCache):
+    """The default component: per layer, all keys and all values so far as tensors
+    (seq, n_kv_head, d_head); new tokens are appended along axis 0 by a byte copy, so cached values
+    are bit-identical to an uncached forward (axono/python/axono/nn/kv_cache.py:71-117).
+
+    Same observable behaviour as the reference's concat-per-step cache; the storage differs: each layer
+    keeps a buffer with spare capacity and `get` returns tensors over its used prefix."""
+
+    _FIRST_CAPACITY = 64
+
     def __init__(self, n_layers: int, device: str | None = None):
-        self.n_layers = n_layers
+        self.n_layers = int(n_layers)
         self.device = device
-        self._k = [None] * n_layers
-        self._v = [None] * n_layers
+        self._layers: dict = {}   # layer index -> (_GrowableRows for k, _GrowableRows for v)
+
+    def _check_layer(self, layer_idx: int) -> int:
+        li = int(layer_idx)
+        if not 0 <= li < self.n_layers:
+            raise IndexError(f"DynamicKVCache: layer {layer_idx} outside 0..{self.n_layers - 1}")
+        return li
 
     def update(self, layer_idx: int, k_new, v_new) -> None:
-        if self._k[layer_idx] is None:
-            self._k[layer_idx] = k_new
-            self._v[layer_idx] = v_new
-            return
-        self._k[layer_idx] = _l.concat(self._k[layer_idx], k_new, 0)
-        self._v[layer_idx] = _l.concat(self._v[layer_idx], v_new, 0)
+        li = self._check_layer(layer_idx)
+        if self.device is not None:
+            k_new, v_new = k_new.to(self.device), v_new.to(self.device)
+        entry = self._layers.get(li)
+        if entry is None:
+            cap = max(self._FIRST_CAPACITY, 2 * int(k_new.shape[0]))
+            self._layers[li] = (_GrowableRows(k_new, cap), _GrowableRows(v_new, cap))
+        else:
+            entry[0].append(k_new)
+            entry[1].append(v_new)
 
     def get(self, layer_idx: int):
-        if self._k[layer_idx] is None:
-            raise RuntimeError("DynamicKVCache: 尚未 update (prefill 未执行?)")
-        return self._k[layer_idx], self._v[layer_idx]
+        entry = self._layers.get(self._check_layer(layer_idx))
+        if entry is None:
+            raise RuntimeError(f"DynamicKVCache: layer {layer_idx} holds nothing yet (call update first, e.g. by running the prefill)")
+        return entry[0].view(), entry[1].view()
 
     def reset(self) -> None:
-        self._k = [None] * self.n_layers
-        self._v = [None] * self.n_layers
+        self._layers.clear()
 
     def __len__(self) -> int:
-        for k in self._k:
-            if k is not None:
-                return int(k.shape[0])
-        return 0
+        """Cached positions of the lowest-numbered layer that holds any (every layer of a model is
+        updated once per forward, so they agree)."""
+        if not self._layers:
+            return 0
+        return self._layers[min(self._layers)][0].rows
 
 
 class StaticKVCache(KVCache):

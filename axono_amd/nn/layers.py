@@ -35,12 +35,17 @@ class Linear(Module):
         if w.dtype != DataType.FLOAT16:
             raise RuntimeError("linear: the hip operator takes FLOAT16 weights; call cast_linear_fp16() first")
         if w.is_hip and x.num_elements:
-            # the kernels read the packed copy of the weight (made once, on first use)
+            # The kernels read a packed copy of the weight.  It is made on first use and again whenever
+            # the weight's storage was replaced or written since (load_state_dict, copy_from,
+            # copy_from_numpy and fill* write in place and bump the storage's version), so forward
+            # always multiplies by the live weight, as the reference's Linear does (nn/layers.py:72-80).
+            key = (w._st, w._st.version)
+            held = self.__dict__.get("_packed_key")
             packed = self.__dict__.get("_packed")
-            if packed is None or self.__dict__.get("_packed_of") is not w:
+            if packed is None or held is None or held[0] is not key[0] or held[1] != key[1]:
                 packed = _l.pack_linear_weight(w)
                 object.__setattr__(self, "_packed", packed)
-                object.__setattr__(self, "_packed_of", w)
+                object.__setattr__(self, "_packed_key", key)
             return _l.linear_packed(x, packed, self.out_features, b)
         return _l.linear(x, w, b) if b is not None else _l.linear_nobias(x, w)
 

@@ -156,6 +156,34 @@ def test_linear_fp16_module_path(hip_env):
     np.testing.assert_allclose(nb(Tensor.from_numpy(x_np)).to_numpy(), want - b_np.astype(np.float16).astype(np.float32), rtol=0, atol=2e-5)
 
 
+def test_linear_follows_weights_written_after_a_forward(hip_env):
+    """A Linear that has run once keeps a packed copy of its weight; load_state_dict / copy_from /
+    copy_from_numpy write the weight in place, and the next forward must use the new values (the
+    reference's Linear reads the live weight on every call, nn/layers.py:72-80)."""
+    rng = np.random.default_rng(11)
+    x_np = rng.normal(size=(8, 64)).astype(np.float16)
+    lin = nn.Linear(64, 32, bias=False, device="hip")
+    lin.cast_linear_fp16()
+    x = Tensor.from_numpy(x_np)
+
+    def want(w16):
+        return port.linear(x_np.astype(np.float32), w16.astype(np.float32), None)
+
+    w0 = lin.weight.numpy().copy()
+    np.testing.assert_allclose(lin(x).to_numpy(), want(w0), rtol=0, atol=2e-5)
+    w1 = (rng.normal(size=(32, 64)) * 0.05).astype(np.float16)
+    lin.load_state_dict({"weight": w1})
+    np.testing.assert_allclose(lin(x).to_numpy(), want(w1), rtol=0, atol=2e-5)
+    w2 = (rng.normal(size=(32, 64)) * 0.05).astype(np.float16)
+    lin.weight.copy_from_numpy(w2)
+    np.testing.assert_allclose(lin(x).to_numpy(), want(w2), rtol=0, atol=2e-5)
+    w3 = (rng.normal(size=(32, 64)) * 0.05).astype(np.float16)
+    lin.weight.copy_from(Tensor.from_numpy(w3))
+    np.testing.assert_allclose(lin(x).to_numpy(), want(w3), rtol=0, atol=2e-5)
+    lin.weight.fill_zero()
+    assert np.all(lin(x).to_numpy() == 0)
+
+
 def _np_attention(q, k, v, causal):
     sq, hq, d = q.shape
     skv, hkv = k.shape[:2]

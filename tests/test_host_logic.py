@@ -168,15 +168,36 @@ def test_linear_needs_fp16_weights_before_forward():
 
 
 def test_dynamic_kv_cache_bookkeeping():
+    """The reference's component tests (axono/python/tests/nn/test_kv_cache.py:27-73) on host tensors:
+    length, append order, byte-exact contents, independent layers, reset, growth past the first capacity."""
+    rng = np.random.default_rng(3)
     c = nn.DynamicKVCache(3)
     assert len(c) == 0
     with pytest.raises(RuntimeError):
         c.get(0)
-    k = Tensor.zeros([5, 2, 4])
-    c.update(1, k, k)
-    assert len(c) == 5 and c.get(1)[0] is k
+    with pytest.raises(IndexError):
+        c.update(3, Tensor.zeros([1, 2, 4]), Tensor.zeros([1, 2, 4]))
+    ks, vs = [], []
+    for step, rows in enumerate([5, 1, 1, 70, 1, 130]):   # crosses the first capacity (64) twice
+        k = rng.standard_normal((rows, 2, 4)).astype(np.float32)
+        v = rng.standard_normal((rows, 2, 4)).astype(np.float32)
+        ks.append(k)
+        vs.append(v)
+        c.update(1, Tensor.from_numpy(k), Tensor.from_numpy(v))
+        got_k, got_v = c.get(1)
+        assert len(c) == sum(a.shape[0] for a in ks) and got_k.shape == [len(c), 2, 4]
+        np.testing.assert_array_equal(got_k.to_numpy(), np.concatenate(ks, 0))
+        np.testing.assert_array_equal(got_v.to_numpy(), np.concatenate(vs, 0))
+    with pytest.raises(RuntimeError):
+        c.get(0)                                # layers are independent
+    c.update(0, Tensor.from_numpy(ks[0]), Tensor.from_numpy(vs[0]))
+    assert len(c) == 5                          # the lowest-numbered layer that holds something
+    with pytest.raises(RuntimeError):
+        c.update(0, Tensor.zeros([1, 3, 4]), Tensor.zeros([1, 3, 4]))   # row shape differs
     c.reset()
     assert len(c) == 0
+    with pytest.raises(RuntimeError):
+        c.get(1)
 
 
 def test_compile_signature_keys():

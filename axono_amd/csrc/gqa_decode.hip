@@ -47,6 +47,13 @@ Tuning g_tuning;
 constexpr int kTicketSlots = 1 << 16;  // per ticket lane
 __device__ unsigned int g_tickets[AXHIP_TICKET_LANES * kTicketSlots];
 
+// Scratch of the entry point that allocates nothing (axhip_gqa_decode_static): the split partials live here
+// instead of in a caller's workspace.  Every device the library runs on holds its own copy of this array
+// until the process ends.  In host code the array's name is only a stand-in for the symbol: the address
+// on a device comes from hipGetSymbolAddress (static_scratch_on_this_device below) and kernels get that
+// pointer as an argument, exactly as they get a caller's workspace.
+static __device__ __align__(256) unsigned char scratch[AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES];
+
 constexpr int kMaxDynBatch = 64;  // batches up to this size deal their workgroups by sequence length
 
 // How the key axis is cut.  The plan depends only on host-side sizes, so that a captured launch stays
@@ -1141,8 +1148,28 @@ using namespace axhip;
 
 namespace {
 // Split plan, workspace carve-up and launch shared by the entry points.
+// The device address of `scratch` on the current device, looked up once per device (with that device
+// current) and kept: each device holds its own copy of the array at its own address.
+int static_scratch_on_this_device(void **out) {
+  static std::atomic<void *> addr[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return AXHIP_DEVICE_ERROR;
+  void *p = addr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return AXHIP_DEVICE_ERROR;
+    }
+    addr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return AXHIP_OK;
+}
+
+// `static_ws`: the partials go to this device's static scratch instead of a caller's workspace; a plan that
+// needs more than the array holds is refused with AXHIP_OUT_OF_MEMORY.
 int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int dtype, int B, int Hq, int Hkv,
-                    int D, int max_len, axhip_stream stream) {
+                    int D, int max_len, axhip_stream stream, bool static_ws = false) {
   const int group = Hq / Hkv;
   // four or more heads per kv head, fp16: the heads of a kv head become the columns of an MFMA tile
   const bool mfma = g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) &&
@@ -1171,6 +1198,12 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
   if (plan.stride > 1) {
     const size_t acc_elems = static_cast<size_t>(B) * Hq * plan.stride * D;
     const size_t need = (acc_elems + static_cast<size_t>(B) * Hq * plan.stride * 2) * sizeof(float);
+    if (static_ws) {
+      if (need > static_cast<size_t>(AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES)) return AXHIP_OUT_OF_MEMORY;
+      const int rc = static_scratch_on_this_device(&workspace);
+      if (rc != AXHIP_OK) return rc;
+      workspace_bytes = AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES;
+    }
     if (!workspace || workspace_bytes < need) return AXHIP_INVALID_ARGUMENT;
     a.part_acc = static_cast<float *>(workspace);
     a.part_ml = a.part_acc + acc_elems;
@@ -1210,10 +1243,13 @@ AXHIP_API size_t axhip_gqa_decode_workspace_bytes(int B, int Hq, int Hkv, int D,
   return static_cast<size_t>(B) * Hq * kMaxSplits * (D + 2) * sizeof(float);
 }
 
-AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v, const int32_t *seq_lens,
-                               void *out, void *workspace, size_t workspace_bytes, int dtype, int B,
-                               int Hq, int Hkv, int D, int max_len, int64_t stride_b,
-                               int64_t stride_h, int64_t stride_s, axhip_stream stream) {
+}  // extern "C"
+
+namespace {
+int gqa_decode_entry(const void *q, const void *k, const void *v, const int32_t *seq_lens, void *out,
+                     void *workspace, size_t workspace_bytes, int dtype, int B, int Hq, int Hkv, int D,
+                     int max_len, int64_t stride_b, int64_t stride_h, int64_t stride_s, axhip_stream stream,
+                     bool static_ws) {
   if (dtype != AXHIP_FLOAT16 && dtype != AXHIP_FLOAT32) return AXHIP_UNSUPPORTED_TYPE;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || max_len <= 0) return AXHIP_INVALID_ARGUMENT;
   if (Hq % Hkv != 0) return AXHIP_SHAPE_MISMATCH;
@@ -1236,7 +1272,28 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v, cons
   a.stride_b = stride_b;
   a.stride_h = stride_h;
   a.stride_s = stride_s;
-  return plan_and_launch(a, workspace, workspace_bytes, dtype, B, Hq, Hkv, D, max_len, stream);
+  return plan_and_launch(a, workspace, workspace_bytes, dtype, B, Hq, Hkv, D, max_len, stream, static_ws);
+}
+}  // namespace
+
+extern "C" {
+
+AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v, const int32_t *seq_lens,
+                               void *out, void *workspace, size_t workspace_bytes, int dtype, int B,
+                               int Hq, int Hkv, int D, int max_len, int64_t stride_b,
+                               int64_t stride_h, int64_t stride_s, axhip_stream stream) {
+  return gqa_decode_entry(q, k, v, seq_lens, out, workspace, workspace_bytes, dtype, B, Hq, Hkv, D, max_len,
+                          stride_b, stride_h, stride_s, stream, false);
+}
+
+// axhip_gqa_decode with the split partials in the library's static device scratch: no workspace argument,
+// no allocation of any kind on the call path (the kernels, the plan and the results are the same).
+AXHIP_API int axhip_gqa_decode_static(const void *q, const void *k, const void *v, const int32_t *seq_lens,
+                                      void *out, int dtype, int B, int Hq, int Hkv, int D, int max_len,
+                                      int64_t stride_b, int64_t stride_h, int64_t stride_s,
+                                      axhip_stream stream) {
+  return gqa_decode_entry(q, k, v, seq_lens, out, nullptr, 0, dtype, B, Hq, Hkv, D, max_len, stride_b,
+                          stride_h, stride_s, stream, true);
 }
 
 AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float *k, int64_t k_stride,

@@ -192,6 +192,28 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
                                int max_len, int64_t stride_b, int64_t stride_h, int64_t stride_s,
                                axhip_stream stream);
 
+/* axhip_gqa_decode for callers that cannot allocate (code under hipGraph capture, tight serving loops,
+ * harnesses that forbid hipMalloc) and therefore have no workspace to pass: the split partials go to a
+ * static device array inside the library, AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES per device, held until
+ * the process ends.  Same arguments (without workspace), same kernels, same split plan and bit-identical
+ * results; neither the call nor anything it runs allocates or frees memory.  It has no counterpart in the
+ * reference (whose operator allocates three workspace tensors per call, src/ops/cuda/gqa.cu:166-168).
+ *   - a problem whose split plan needs more scratch than the array holds is refused with
+ *     AXHIP_OUT_OF_MEMORY before anything is launched (B * Hq * ranges-per-sequence * (D + 2) * 4 bytes
+ *     are needed; with the default plan ranges-per-sequence <= max(256 / head groups, B), so e.g. every
+ *     batch up to B = 64 at Hq = 16, D = 128 fits);
+ *   - every call on a device shares that device's array, whatever its ticket lane: calls that overlap
+ *     in time on one device race.  Calls on one stream, and replays of one captured graph, never overlap.
+ *     Nothing in the array has to start at zero (a partial is always written before it is read), so the
+ *     previous call's contents are simply overwritten;
+ *   - the array's address is looked up on the first call on each device; make that first call outside a
+ *     graph capture. */
+#define AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES (48u << 20)
+AXHIP_API int axhip_gqa_decode_static(const void *q, const void *k, const void *v,
+                                      const int32_t *seq_lens, void *out, int dtype, int B, int Hq,
+                                      int Hkv, int D, int max_len, int64_t stride_b, int64_t stride_h,
+                                      int64_t stride_s, axhip_stream stream);
+
 /* The split plan the launcher uses for these sizes (it depends on host-side sizes only).  For batches of
  * up to 64 sequences the launch holds a fixed number of workgroups which are dealt to the sequences on the
  * device in proportion to their current lengths (n_splits = workgroup slots per sequence, chunk = keys per

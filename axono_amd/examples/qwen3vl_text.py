@@ -329,6 +329,9 @@ class Qwen3VLTextDecoder(nn.Module):
         self._ids.copy_from_numpy(np.ascontiguousarray(first_ids, dtype=np.int64).reshape(B))
         self._pos.copy_from_numpy(np.ascontiguousarray(first_pos, dtype=np.int64).reshape(3, B))
         bound = min(self._cache.max_len, len(self._cache) + max_new_tokens + 1)
+        # the captured attention launches attend to at most `bound` keys and append only below it:
+        # generate() refuses to run past it (it would silently drop tokens from the cache otherwise)
+        self._decode_bound = bound
         # the tokens of every step are gathered on the device, at the row a device-side counter names
         self._log = Tensor(DataType.INT64, [max(max_new_tokens, 1), B], self._device)
         self._counter = Tensor(DataType.INT64, [1], self._device)
@@ -363,6 +366,14 @@ class Qwen3VLTextDecoder(nn.Module):
         are gathered on the device (by the step itself) and read back once at the end."""
         if max_new_tokens > self._log.shape[0]:
             raise ValueError("generate(): more steps than start_decode() was told to expect")
+        have = len(self._cache)
+        if have + max_new_tokens > self._cache.max_len:
+            raise RuntimeError(f"generate(): the KV cache is full ({have} of {self._cache.max_len} positions used, "
+                               f"{max_new_tokens} more asked for)")
+        if have + max_new_tokens > self._decode_bound:
+            raise RuntimeError(f"generate(): the step was set up by start_decode() for sequences of up to "
+                               f"{self._decode_bound} keys; {have} cached + {max_new_tokens} new exceed that. "
+                               f"Call start_decode() (and capture()) again for the new length")
         self._counter.copy_from_numpy(np.zeros(1, np.int64))
         L.synchronize()
         for _ in range(max_new_tokens):

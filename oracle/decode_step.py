@@ -4,7 +4,8 @@ attention, :384 MLP, :408-436 layer, :483-486 final norm + tied lm_head, :729-76
 
 TEST INFRASTRUCTURE ONLY (parity tests and the benchmark's CPU-baseline leg).
 
-All arithmetic is fp32.  Data formats are those of the build under test and are modelled as
+All arithmetic is fp32 with the default operator set (`oracle.port`); `ops=F64Ops()`
+(oracle/f64_ops.py) evaluates the same sequence in float64 with the same storage roundings.  Data formats are those of the build under test and are modelled as
 roundings of stored values only: Linear weights and the embedding table are fp16; the activation
 entering a Linear is rounded to fp16 (the reference's fp16 Linear does that, src/ops/cuda/linear.cu:110);
 q after RoPE and the k / v rows written to the cache are fp16 (the cache format).
@@ -17,8 +18,8 @@ from . import port
 
 
 def _h(x):
-    """Round to fp16 (IEEE RNE) and widen back exactly."""
-    return np.asarray(x, np.float32).astype(np.float16).astype(np.float32)
+    """Round to fp16 (IEEE RNE, one rounding from the array's own precision) and widen back exactly."""
+    return np.asarray(x).astype(np.float16).astype(np.float32)
 
 
 class OracleDecoder:
@@ -59,7 +60,7 @@ class OracleDecoder:
         k = ops.rope_thd(k, pos3, self.inv_freq, cfg.mrope_section)
         self.k[i][rows_b, :, rows_t] = k.astype(np.float16)
         self.v[i][rows_b, :, rows_t] = v.astype(np.float16)
-        attn = np.empty((R, nq, D), np.float32)
+        attn = np.empty((R, nq, D), getattr(ops, "dtype", np.float32))
         for b in np.unique(rows_b):
             sel = np.nonzero(rows_b == b)[0]
             for r in sel:  # each row attends over the keys up to and including its own position

@@ -206,3 +206,76 @@ def test_decode_steps_match_oracle_with_four_heads_per_kv_head():
         n = S + n_steps
         assert np.abs(kc.numpy()[:, :, :n].astype(np.float32) - cpu.k[i][:, :, :n].astype(np.float32)).max() <= 4e-3
         assert np.abs(vc.numpy()[:, :, :n].astype(np.float32) - cpu.v[i][:, :, :n].astype(np.float32)).max() <= 4e-3
+
+
+def test_generate_refuses_to_run_past_the_bound_the_step_was_captured_for():
+    gpu, _, ids = _setup(seed=13, max_len=40)
+    B, S = ids.shape
+    _, nxt = gpu.prefill(ids)
+    gpu.start_decode(nxt.to_numpy(), np.full((3, B), S, np.int64), 4)
+    gpu.capture()
+    gpu.generate(4)
+    with pytest.raises(RuntimeError, match="start_decode"):
+        gpu.generate(4)                      # 21 + 4 + 4 > the bound of 26 the step was captured for
+    gpu.start_decode(gpu._ids.numpy(), gpu._pos.numpy(), 15)
+    gpu.capture()
+    gpu.generate(15)                         # fills the cache to its 40 positions
+    gpu.start_decode(gpu._ids.numpy(), gpu._pos.numpy(), 1)
+    with pytest.raises(RuntimeError, match="full"):
+        gpu.generate(1)
+
+
+def test_device_is_no_farther_from_the_float64_evaluation_than_the_fp32_restatement():
+    """Two correct fp32 pipelines drift apart at the fp16 storage points of a decode step (a 1e-7 difference
+    can round to the other fp16 neighbour).  The yardstick is the same op sequence in float64 with the
+    same storage points (oracle/f64_ops.py): over several decode steps from identical caches, the
+    device's logits are no farther from it than 1.5 x the fp32 restatement's are (with a floor of one
+    fp16 flip's worth), and each layer evaluated from the device's own input to that layer stays within
+    2e-3 of both."""
+    from oracle.f64_ops import F64Ops
+
+    gpu, cpu32, ids = _setup(seed=17)
+    cfg = CFG
+    B, S = ids.shape
+    _, g_next = gpu.prefill(ids)
+    cpu64 = OracleDecoder(cfg, cpu32.w, B, gpu.cache.max_len, ops=F64Ops())
+
+    def sync_caches(n):
+        for i in range(cfg.num_hidden_layers):
+            kc, vc = gpu.cache.get(i)
+            for c in (cpu32, cpu64):
+                c.k[i][:] = kc.numpy()
+                c.v[i][:] = vc.numpy()
+        cpu32.lens[:] = n
+        cpu64.lens[:] = n
+
+    cur = g_next.to_numpy().copy()
+    d_gpu, d_cpu, layer_gpu, layer_cpu = 0.0, 0.0, 0.0, 0.0
+    for s in range(4):
+        n = S + s
+        sync_caches(n)
+        pos = np.full((3, B), n, np.int64)
+        idt, post = Tensor(DataType.INT64, [B], "hip:0"), Tensor(DataType.INT64, [3, B], "hip:0")
+        idt.copy_from_numpy(cur)
+        post.copy_from_numpy(pos)
+        trace = []
+        g_logits, g_tok = gpu.decode_forward(idt, post, trace=trace)
+        g_logits, g_tok = g_logits.to_numpy().copy(), g_tok.to_numpy().copy()
+        h_gpu = [t.to_numpy().copy() for t in trace]
+        l64, _ = cpu64.decode_step(cur, pos)
+        l32, _ = cpu32.decode_step(cur, pos)
+        d_gpu = max(d_gpu, float(np.abs(g_logits - l64).max()))
+        d_cpu = max(d_cpu, float(np.abs(l32 - l64).max()))
+        # layer by layer from the device's own inputs
+        cpu32.lens[:] = n
+        cpu64.lens[:] = n
+        o64, _ = cpu64.decode_layers_teacher_forced(h_gpu, pos)
+        o32, _ = cpu32.decode_layers_teacher_forced(h_gpu, pos)
+        for i in range(cfg.num_hidden_layers):
+            layer_gpu = max(layer_gpu, float(np.abs(h_gpu[i + 1] - o64[i]).max()))
+            layer_cpu = max(layer_cpu, float(np.abs(o32[i] - o64[i]).max()))
+        gpu.cache.advance(1)
+        cur = g_tok
+    assert d_gpu <= max(1.5 * d_cpu, 1e-3), (d_gpu, d_cpu)
+    assert layer_gpu <= 2e-3 and layer_cpu <= 2e-3, (layer_gpu, layer_cpu)
+    assert layer_gpu <= max(1.5 * layer_cpu, 1e-3), (layer_gpu, layer_cpu)

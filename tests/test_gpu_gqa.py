@@ -173,49 +173,128 @@ def test_invariants_full_size_headline():
     assert np.abs(out[:1] - want0).max() <= TOL16
 
 
-def test_largest_config_periodic_cache():
-    """B=64, L=32768 fp16 (8.6 GB of cache, the largest configuration): every (sequence, kv head) row of
-    the cache repeats a block of 1024 random keys and values, built on the device by doubling copies.
-    Attention over r whole repetitions equals attention over one block (every copy of a key gets the same
-    weight), so the oracle on the 1024-key block checks the full-size launch - with all sequences full
-    (whole workgroups per sequence) and with ragged multiples of the block (the end-to-end cut)."""
+class _PeriodicCache:
+    """The largest configuration's cache on the device: K and V [64, 8, 32768, 128] fp16 (8.6 GB), every
+    (sequence, kv head) row repeating a block of P = 1024 random keys / values (uploaded once per row and
+    doubled by device copies).  Attention over r whole repetitions of a block equals attention over the
+    block (every copy of a key gets the same weight), so the oracle on the block checks full-size launches;
+    a length r*P + t is checked by the oracle on that sequence's rows written out on the host."""
     B, Hq, Hkv, D, L, P = 64, 16, 8, 128, 32768, 1024
-    rng = np.random.default_rng(64)
-    q = rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16)
-    kp = rng.standard_normal((B, Hkv, P, D)).astype(np.float32).astype(np.float16)
-    vp = rng.standard_normal((B, Hkv, P, D)).astype(np.float32).astype(np.float16)
-    l = lib()
-    row_bytes, blk = L * D * 2, P * D * 2
-    bufs = []
-    for host in (kp, vp):
-        big = gu.DeviceBuffer(B * Hkv * row_bytes)
-        for r in range(B * Hkv):
-            base = big.ptr + r * row_bytes
-            gu.check(l.axhip_memcpy_h2d(base, host.reshape(B * Hkv, -1)[r].ctypes.data, blk), "h2d")
-            have = blk
-            while have < row_bytes:
-                gu.check(l.axhip_memcpy_d2d(base + have, base, have), "d2d")
-                have *= 2
-        bufs.append(big)
-    dk, dv = bufs
-    dq = gu.dev(q)
-    out = gu.DeviceBuffer(q.nbytes)
-    wsb = l.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
-    ws = gu.DeviceBuffer(max(wsb, 256))
-    want = port.gqa_decode_cache_native(q, kp, vp, np.full(B, P, np.int32))
-    ragged = (P * rng.integers(1, L // P + 1, B)).astype(np.int32)
-    ragged[:3] = [L, P, 0]
-    for lens in (np.full(B, L, np.int32), ragged):
-        dl = gu.dev(lens)
-        gu.check(l.axhip_gqa_decode(dq.ptr, dk.ptr, dv.ptr, dl.ptr, out.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, L,
-                                    Hkv * L * D, L * D, D, None), "gqa_decode")
+
+    def __init__(self):
+        rng = np.random.default_rng(64)
+        B, Hq, Hkv, D, L, P = self.B, self.Hq, self.Hkv, self.D, self.L, self.P
+        self.q = rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16)
+        self.kp = rng.standard_normal((B, Hkv, P, D)).astype(np.float32).astype(np.float16)
+        self.vp = rng.standard_normal((B, Hkv, P, D)).astype(np.float32).astype(np.float16)
+        l = lib()
+        row_bytes, blk = L * D * 2, P * D * 2
+        bufs = []
+        for host in (self.kp, self.vp):
+            big = gu.DeviceBuffer(B * Hkv * row_bytes)
+            for r in range(B * Hkv):
+                base = big.ptr + r * row_bytes
+                gu.check(l.axhip_memcpy_h2d(base, host.reshape(B * Hkv, -1)[r].ctypes.data, blk), "h2d")
+                have = blk
+                while have < row_bytes:
+                    gu.check(l.axhip_memcpy_d2d(base + have, base, have), "d2d")
+                    have *= 2
+            bufs.append(big)
+        self.dk, self.dv = bufs
+        self.dq = gu.dev(self.q)
+        self.block_out = port.gqa_decode_cache_native(self.q, self.kp, self.vp, np.full(B, P, np.int32))
+
+    def run(self, B, max_len, lens):
+        """The first B sequences of the cache, attended up to lens[b] <= max_len keys (rows keep the big
+        cache's strides: the batched layout with Lmax = 32768)."""
+        l = lib()
+        out = gu.DeviceBuffer(B * self.Hq * self.D * 2)
+        wsb = l.axhip_gqa_decode_workspace_bytes(B, self.Hq, self.Hkv, self.D, max_len)
+        ws = gu.DeviceBuffer(max(wsb, 256))
+        dl = gu.dev(np.asarray(lens, np.int32))
+        gu.check(l.axhip_gqa_decode(self.dq.ptr, self.dk.ptr, self.dv.ptr, dl.ptr, out.ptr, ws.ptr, wsb, gu.F16, B,
+                                    self.Hq, self.Hkv, self.D, max_len, self.Hkv * self.L * self.D, self.L * self.D,
+                                    self.D, None), "gqa_decode")
         gu.synchronize()
-        got = out.download(np.float16, q.shape).astype(np.float32)
-        live = lens > 0
-        assert np.abs(got[live] - want[live]).max() <= TOL16, lens
-        assert np.all(got[~live] == 0)
-    for b in (dk, dv):
-        b.release()
+        return out.download(np.float16, (B, self.Hq, self.D)).astype(np.float32)
+
+    def oracle_rows(self, b, length):
+        """The oracle on sequence b's first `length` keys, written out on the host."""
+        reps = -(-length // self.P)
+        k = np.ascontiguousarray(np.tile(self.kp[b:b + 1], (1, 1, reps, 1))[:, :, :length])
+        v = np.ascontiguousarray(np.tile(self.vp[b:b + 1], (1, 1, reps, 1))[:, :, :length])
+        return port.gqa_decode_cache_native(self.q[b:b + 1], k, v, np.array([length], np.int32))[0]
+
+    def release(self):
+        self.dk.release()
+        self.dv.release()
+
+
+@pytest.fixture(scope="module")
+def periodic_cache():
+    c = _PeriodicCache()
+    yield c
+    c.release()
+
+
+@pytest.mark.parametrize("B", [1, 8, 32, 64])
+@pytest.mark.parametrize("L", [1024, 8192, 32768])
+def test_config3_sweep_points_at_full_size(B, L, periodic_cache):
+    """Every point of the B x L sweep at its full size, uniform lengths, default split plan."""
+    c = periodic_cache
+    got = c.run(B, L, np.full(B, L, np.int32))
+    assert np.abs(got - c.block_out[:B]).max() <= TOL16, (B, L)
+
+
+def test_largest_config_ragged_whole_blocks(periodic_cache):
+    """B=64, Lmax=32768 with ragged multiples of the block (the end-to-end cut of the key axis), a full,
+    a one-block and an empty sequence."""
+    c = periodic_cache
+    rng = np.random.default_rng(65)
+    lens = (c.P * rng.integers(1, c.L // c.P + 1, c.B)).astype(np.int32)
+    lens[:3] = [c.L, c.P, 0]
+    got = c.run(c.B, c.L, lens)
+    live = lens > 0
+    assert np.abs(got[live] - c.block_out[live]).max() <= TOL16
+    assert np.all(got[~live] == 0)
+
+
+def test_config3_ragged_batch_arbitrary_lengths(periodic_cache):
+    """The ragged batch of the sweep: B=32, lengths uniform in [512, 32768] and not multiples of anything
+    (both ends of the interval and an odd length forced in), Lmax = 32768.  Each sequence is checked by
+    the oracle on its own rows written out on the host."""
+    c = periodic_cache
+    rng = np.random.default_rng(3232)
+    B = 32
+    lens = rng.integers(512, 32769, B).astype(np.int32)
+    lens[0], lens[1], lens[2], lens[3] = 512, 32768, 32767, 513
+    got = c.run(B, c.L, lens)
+    worst = 0.0
+    for b in range(B):
+        worst = max(worst, float(np.abs(got[b] - c.oracle_rows(b, int(lens[b]))).max()))
+    assert worst <= TOL16, worst
+
+
+def test_more_than_64_sequences_take_the_static_plan_by_default():
+    """Batches above 64 sequences are cut by the host-side static plan (every sequence into n_splits
+    ranges from the grid).  Default tuning: 80 sequences of Hq16/Hkv8 (one range each), and 80 sequences
+    with one head group, which the plan cuts into several ranges merged in the kernel."""
+    rng = np.random.default_rng(80)
+    l = lib()
+    for (B, hq, hkv, Lmax, want_splits) in ((80, 16, 8, 1500, 1), (80, 2, 1, 4096, 4), (200, 2, 1, 700, 2)):
+        lens = rng.integers(1, Lmax + 1, B).astype(np.int32)
+        lens[:4] = [Lmax, 0, 1, 257]
+        import ctypes as C
+        ns, ch = C.c_int(0), C.c_int(0)
+        l.axhip_gqa_decode_plan(B, hq, hkv, Lmax, C.byref(ns), C.byref(ch))
+        assert ns.value == want_splits, (B, hq, ns.value)
+        q = rng.standard_normal((B, hq, 128)).astype(np.float32).astype(np.float16)
+        k = rng.standard_normal((B, hkv, Lmax, 128)).astype(np.float32).astype(np.float16)
+        v = rng.standard_normal((B, hkv, Lmax, 128)).astype(np.float32).astype(np.float16)
+        got = gqa_decode(q, k, v, lens).astype(np.float32)
+        want = port.gqa_decode_cache_native(q, k, v, lens)
+        assert np.abs(got - want).max() <= TOL16, (B, hq)
+        assert np.all(got[1] == 0)
 
 
 def test_error_codes():

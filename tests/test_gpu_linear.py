@@ -49,85 +49,43 @@ def test_config4_shapes(M, K, N):
     check_linear(x, w)
 
 
-def test_lm_head_slice_and_full_M16():
+@pytest.fixture(scope="module")
+def lm_head_weight():
+    """The lm_head of the 2B shape: 151936 x 2048 fp16 ~ N(0, 0.02) (622 MB on the device)."""
     rng = np.random.default_rng(99)
-    K, N = 2048, 151936
-    w = h16(0.02 * rng.standard_normal((N, K)))
-    x = h16(rng.standard_normal((16, K)))
+    return h16(0.02 * rng.standard_normal((151936, 2048), dtype=np.float32))
+
+
+def _lm_head_columns(N, step):
+    # a regular subsample plus both ends of the matrix (first / last weight-row tiles, N % 256 != 0)
+    return np.unique(np.concatenate([np.arange(0, N, step), np.arange(0, 40), np.arange(N - 40, N)]))
+
+
+@pytest.mark.parametrize("M", [1, 16, 32, 512])
+def test_lm_head_every_row_count(M, lm_head_weight):
+    """2048 -> 151936 at every row count of the benchmark configuration, row-major and packed weights:
+    the oracle on a column subsample (the full CPU product takes minutes), the summation-order bound of
+    check_linear, and the two weight layouts bit-identical to each other over the whole output."""
+    w = lm_head_weight
+    N, K = w.shape
+    rng = np.random.default_rng(1000 + M)
+    x = h16(rng.standard_normal((M, K)))
     out = gu.linear_f16(x, w)
-    # the oracle on every 37th output column (the full 16x151936x2048 CPU product takes minutes)
-    cols = np.arange(0, N, 37)
-    want = port.linear(x.astype(np.float32), w[cols].astype(np.float32))
-    assert np.abs(out[:, cols] - want).max() <= 1e-4
-    # linearity in x: f(2x) = 2 f(x) exactly (scaling by 2 is exact in fp16 and fp32)
-    np.testing.assert_array_equal(gu.linear_f16(h16(2 * x.astype(np.float32)), w), 2 * out)
-
-
-def test_fp32_activations_bias_odd_shapes():
-    rng = np.random.default_rng(5)
-    for (M, K, N) in [(8, 64, 32), (3, 72, 50), (17, 136, 33), (33, 520, 130), (130, 264, 190)]:
-        x = rng.standard_normal((M, K)).astype(np.float32)  # fp32 in, as the reference's Linear.forward passes
-        w = h16(0.05 * rng.standard_normal((N, K)))
-        b = h16(0.05 * rng.standard_normal(N))
-        check_linear(x, w, b)
-        check_linear(x, w)
-
-
-def test_fp16_output_variant():
-    rng = np.random.default_rng(6)
-    x = h16(rng.standard_normal((16, 2048)))
-    w = h16(0.02 * rng.standard_normal((2048, 2048)))
-    out16 = gu.linear_f16(x, w, out_dtype=np.float16)
-    want = port.linear(x.astype(np.float32), w.astype(np.float32))
-    assert np.abs(out16.astype(np.float32) - want).max() <= 2e-3 * max(1.0, np.abs(want).max() / 2)
-
-
-def test_matches_fp32_linear_loosely_like_reference_test():
-    """tests/core/test_fp16.py:28-46 of the reference: fp16 Linear vs fp32 Linear at 5e-2."""
-    rng = np.random.default_rng(1)
-    x = rng.normal(size=(8, 64)).astype(np.float32)
-    w = (rng.normal(size=(32, 64)) * 0.05).astype(np.float32)
-    b = (rng.normal(size=(32,)) * 0.05).astype(np.float32)
-    out = gu.linear_f16(x, h16(w), h16(b))
-    np.testing.assert_allclose(out, x @ w.T + b, rtol=5e-2, atol=5e-2)
-
-
-def test_error_codes():
-    l = gu.lib()
-    assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 60, 8, None, 0, None) == 1  # K % 8
-    assert l.axhip_linear_f16(None, 2, None, None, None, 5, 4, 64, 8, None, 0, None) == 3  # x dtype
-    assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 64, 8, None, 0, None) == 7  # null pointers
-
-
-@pytest.mark.parametrize("M", [1, 16, 32])
-@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 4096)])
-def test_packed_weights_config4_shapes(M, K, N):
-    """The packed-weight kernels give the oracle's result and agree with the row-major path."""
-    rng = np.random.default_rng(M * 11 + K + N)
-    x = h16(rng.standard_normal((M, K)))
-    w = h16(0.02 * rng.standard_normal((N, K)))
-    out = gu.linear_f16_packed(x, w)
-    want = port.linear(x.astype(np.float32), w.astype(np.float32))
-    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
-    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag)
-    assert np.abs(out - gu.linear_f16(x, w)).max() <= 1e-4
-
-
-@pytest.mark.parametrize("M,K,N", [(33, 2048, 2048), (64, 6144, 2048), (50, 520, 130), (64, 2048, 2064), (65, 2048, 2048),
-                                   (200, 6144, 2048), (100, 1024, 1000), (130, 1536, 4096)])
-def test_packed_weights_33_to_64_rows(M, K, N):
-    """Narrow matrices keep the weight-streaming kernels up to 64 rows (two blocks of rows); one column
-    tile more, or one row more, and the tiled GEMM takes over - for problems this small its form whose
-    loads run four K steps ahead (K a multiple of 512).  Same oracle either side of each switch."""
-    rng = np.random.default_rng(M + K + N)
-    x = h16(rng.standard_normal((M, K)))
-    w = h16(0.02 * rng.standard_normal((N, K)))
-    out = gu.linear_f16_packed(x, w)
-    want = port.linear(x.astype(np.float32), w.astype(np.float32))
-    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
-    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag)
-    # fp32 activations are rounded to fp16 on load: the same result
-    np.testing.assert_array_equal(gu.linear_f16_packed(x.astype(np.float32), w), out)
+    assert out.shape == (M, N) and np.isfinite(out).all()
+    cols = _lm_head_columns(N, 37 if M <= 32 else 301)
+    x32, w32 = x.astype(np.float32), w[cols].astype(np.float32)
+    want = port.linear(x32, w32)
+    bound = 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * (np.abs(x32) @ np.abs(w32).T)
+    err = np.abs(out[:, cols] - want)
+    assert np.all(err <= bound), (M, float(err.max()))
+    packed = gu.linear_f16_packed(x, w)
+    err_p = np.abs(packed[:, cols] - want)
+    assert np.all(err_p <= bound), (M, float(err_p.max()))
+    if M == 16:
+        # at this row count the two skinny kernels cut K the same way: the same sums in the same order
+        np.testing.assert_array_equal(packed, out)
+    else:
+        assert np.abs(packed - out).max() <= 2 * float(bound.max())
 
 
 def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
@@ -143,18 +101,6 @@ def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
     l = gu.lib()
     assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 33, 60, 8, 0, None) == 1  # K % 8
     assert l.axhip_linear_f16_packed_bytes(17, 40) == 2 * 2 * 1024
-
-
-def test_packed_lm_head_M16():
-    rng = np.random.default_rng(98)
-    K, N = 2048, 151936
-    w = h16(0.02 * rng.standard_normal((N, K)))
-    x = h16(rng.standard_normal((16, K)))
-    out = gu.linear_f16_packed(x, w)
-    cols = np.arange(0, N, 41)
-    want = port.linear(x.astype(np.float32), w[cols].astype(np.float32))
-    assert np.abs(out[:, cols] - want).max() <= 1e-4
-    assert np.abs(out[:, -7:] - port.linear(x.astype(np.float32), w[-7:].astype(np.float32))).max() <= 1e-4
 
 
 @pytest.mark.parametrize("M,K,I", [(16, 2048, 6144), (1, 2048, 6144), (32, 256, 96), (5, 72, 32)])

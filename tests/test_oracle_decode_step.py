@@ -69,3 +69,65 @@ def test_single_layer_wiring_against_numpy():
     h = h + h16(act) @ W["layers.0.mlp.down_proj.weight"].T
     want = h16(rms(h, W["norm.weight"])) @ W["embed_tokens.weight"].T
     np.testing.assert_allclose(logits[0], want, rtol=0, atol=2e-5)
+
+
+def test_f64_operator_set_agrees_with_the_fp32_oracle_operators():
+    """oracle/f64_ops.py (the float64 yardstick) against the restatement, operator by operator, on random
+    inputs: they evaluate the same functions, so they agree to fp32 rounding."""
+    from oracle import port
+    from oracle.f64_ops import F64Ops
+
+    f = F64Ops()
+    rng = np.random.default_rng(12)
+    q = rng.standard_normal((3, 4, 16)).astype(np.float32)
+    k = rng.standard_normal((7, 2, 16)).astype(np.float32)
+    v = rng.standard_normal((7, 2, 16)).astype(np.float32)
+    for causal in (False, True):
+        np.testing.assert_allclose(f.sdpa(q, k, v, causal), port.sdpa(q, k, v, causal), rtol=0, atol=2e-6)
+    x = rng.standard_normal((5, 64)).astype(np.float32)
+    r = rng.standard_normal((5, 64)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    np.testing.assert_allclose(f.rms_norm(x, w, 1e-6), port.rms_norm(x, w, 1e-6), rtol=0, atol=2e-6)
+    np.testing.assert_allclose(f.rms_norm(x, None, 1e-5), port.rms_norm(x, None, 1e-5), rtol=0, atol=2e-6)
+    y64, o64 = f.add_rms_norm(x, r, w, 1e-6)
+    y32, o32 = port.add_rms_norm(x, r, w, 1e-6)
+    np.testing.assert_allclose(y64, y32, rtol=0, atol=1e-6)
+    np.testing.assert_allclose(o64, o32, rtol=0, atol=2e-6)
+    np.testing.assert_allclose(f.silu_mul(x, r), port.silu_mul(x, r), rtol=0, atol=2e-6)
+    wl = (0.1 * rng.standard_normal((9, 64))).astype(np.float32)
+    np.testing.assert_allclose(f.linear(x, wl), port.linear(x, wl), rtol=0, atol=1e-5)
+    b = rng.standard_normal(9).astype(np.float32)
+    np.testing.assert_allclose(f.linear(x, wl, b), port.linear(x, wl, b), rtol=0, atol=1e-5)
+    # M-RoPE with distinct (t, h, w) positions and sections that leave some channels on T
+    xr = rng.standard_normal((6, 3, 16)).astype(np.float32)
+    pos = rng.integers(0, 50, (3, 6)).astype(np.int64)
+    inv = port.rope_inv_freq(1e4, 16)
+    np.testing.assert_allclose(f.rope_thd(xr, pos, inv, [4, 2, 2]), port.rope_thd(xr, pos, inv, [4, 2, 2]), rtol=0,
+                               atol=5e-6)
+    ids = rng.integers(0, 5, 8)
+    np.testing.assert_array_equal(f.embedding(ids, x), port.embedding(ids, x).astype(np.float64))
+    np.testing.assert_array_equal(f.argmax(x), port.argmax(x))
+
+
+def test_f64_decode_step_is_the_same_op_sequence():
+    """The float64 evaluation of a prefill + decode step stays within fp32-rounding distance of the fp32
+    restatement on a shallow model (where fp16 boundary flips have no depth to grow in), and keeps the
+    cache-vs-longer-prefill identity itself."""
+    from oracle.f64_ops import F64Ops
+
+    w = _weights(2)
+    rng = np.random.default_rng(6)
+    B, S = 2, 7
+    ids = rng.integers(0, CFG.vocab_size, (B, S + 1)).astype(np.int64)
+    a32 = OracleDecoder(CFG, w, B, 32)
+    a64 = OracleDecoder(CFG, w, B, 32, ops=F64Ops())
+    a32.prefill(ids[:, :S])
+    a64.prefill(ids[:, :S])
+    pos = np.full((3, B), S, np.int64)
+    l32, _ = a32.decode_step(ids[:, S], pos)
+    l64, _ = a64.decode_step(ids[:, S], pos)
+    assert l64.dtype == np.float64
+    assert np.abs(l64 - l32).max() <= 2e-3     # two layers: at most a few fp16 flips of 1 ulp each
+    b64 = OracleDecoder(CFG, w, B, 32, ops=F64Ops())
+    full64, _ = b64.prefill(ids)
+    np.testing.assert_allclose(l64, full64, rtol=0, atol=1e-9)

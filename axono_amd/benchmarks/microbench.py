@@ -55,8 +55,27 @@ def _rand_fill(buf, nbytes, seed):
         off += n
 
 
+# When a list is put here, records are appended to it instead of being printed (bench.py collects the
+# per-configuration tables of its JSON line this way).
+SINK = None
+
+
 def _emit(rec):
-    print(json.dumps(rec), flush=True)
+    if SINK is not None:
+        SINK.append(rec)
+    else:
+        print(json.dumps(rec), flush=True)
+
+
+def collect(fn, *args, **kwargs):
+    """Runs one of the bench_* functions and returns the records it would have printed."""
+    global SINK
+    prev, SINK = SINK, []
+    try:
+        fn(*args, **kwargs)
+        return SINK
+    finally:
+        SINK = prev
 
 
 def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag="gqa", fp32=False,
@@ -233,13 +252,13 @@ def bench_copy(lib, mib, steps):
            "GBps_read_plus_write": round(gbs, 1), "pct_hbm_peak": round(100 * gbs / HBM_PEAK, 1)})
 
 
-def bench_rowops(lib, steps=200):
+def bench_rowops(lib, steps=200, row_counts=(32, 4096, 65536)):
     rng = np.random.default_rng(0)
 
     def h(shape, scale=1.0):
         return DeviceBuffer.from_numpy((scale * rng.standard_normal(shape)).astype(np.float32).astype(np.float16))
 
-    for rows in (32, 4096, 65536):
+    for rows in row_counts:
         x, r, w = h((rows, 2048)), h((rows, 2048)), h((2048,))
         y, o = DeviceBuffer(rows * 4096), DeviceBuffer(rows * 4096)
         us = _time(lib, lambda: check(lib.axhip_add_rms_norm(x.ptr, r.ptr, w.ptr, 1e-6, y.ptr, o.ptr, F16, F16,

@@ -32,6 +32,84 @@ def step_bytes(cfg: TextConfig, batch: int, context: int) -> int:
     return weights + kv
 
 
+def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) -> list:
+    """Where a decode step goes, kernel by kernel: every kind of launch of the step is captured as a graph
+    of that launch for all layers (each layer's own weights and caches, so nothing is served from the
+    memory-side cache) and replayed `reps` times between host clock reads.  Rows: calls per step, us per call
+    inside such a back-to-back graph, algorithmic bytes per call and the fraction of HBM peak that is.
+    Run it after the timed loop: the attention launches overwrite the cache row at the current length."""
+    from ..core.hip_graph import HIPGraph
+    from ..core.tensor import Tensor
+    from ..core.types import DataType
+
+    cfg, B = model._cfg, model._batch
+    nl, H, D = cfg.num_hidden_layers, cfg.hidden_size, cfg.head_dim
+    nq, nkv, I, V = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.intermediate_size, cfg.vocab_size
+    rng = np.random.default_rng(0)
+
+    def dev(shape, dtype):
+        a = rng.standard_normal(shape).astype(np.float32)
+        return Tensor.from_numpy_ref(np.ascontiguousarray(a.astype(np.float16) if dtype == DataType.FLOAT16 else a)).to(model._device)
+
+    xn = dev((B, H), DataType.FLOAT16)
+    h = dev((B, H), DataType.FLOAT32)
+    qkv = dev((B, (nq + 2 * nkv) * D), DataType.FLOAT32)
+    attn = dev((B, nq * D), DataType.FLOAT16)
+    act = dev((B, I), DataType.FLOAT16)
+    o32 = dev((B, H), DataType.FLOAT32)
+    logits = dev((B, V), DataType.FLOAT32)
+    lens = model.cache.seq_lens
+    W = model._w
+
+    def layers(fn):
+        return lambda: [fn(f"layers.{i}.", i) for i in range(nl)]
+
+    def lin_bytes(K, N, out_b):
+        return 2 * K * N + 2 * B * K + out_b * B * N
+
+    kinds = [
+        ("qkv Linear 2048->4096", nl, lin_bytes(H, (nq + 2 * nkv) * D, 4),
+         layers(lambda p, i: model._linear(xn, p + "self_attn.qkv_proj.weight"))),
+        ("attention (q/k norm + M-RoPE + KV append + split-K decode + merge)", nl,
+         2 * nkv * D * 2 * B * (context + 1) + B * (nq + 2 * nkv) * D * 4 + B * nq * D * 2,
+         layers(lambda p, i: L.gqa_decode_attention_qkv(
+             qkv, W(p + "self_attn.q_norm.weight"), W(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, model._pos,
+             model._inv_freq, cfg.mrope_section, lens, *model.cache.get(i), nq, model._decode_bound,
+             workspace=model._attn_ws))),
+        ("o_proj Linear 2048->2048", nl, lin_bytes(nq * D, H, 4),
+         layers(lambda p, i: model._linear(attn, p + "self_attn.o_proj.weight"))),
+        ("add + RMSNorm (fp32 residual, fp16 out)", 2 * nl, B * H * (4 + 4 + 4 + 2) + 4 * H,
+         lambda: [L.add_rms_norm(o32, h, W(f"layers.{i // 2}.post_attention_layernorm.weight"), cfg.rms_norm_eps,
+                                 DataType.FLOAT16) for i in range(2 * nl)]),
+        ("gate+up Linear 2048->12288 + SiLU-mul", nl, lin_bytes(H, 2 * I, 1),
+         layers(lambda p, i: L.linear_packed(xn, model._packed[p + "mlp.gate_up_proj.weight"], 2 * I,
+                                             out_dtype=DataType.FLOAT16, glu=True))),
+        ("down Linear 6144->2048", nl, lin_bytes(I, H, 4), layers(lambda p, i: model._linear(act, p + "mlp.down_proj.weight"))),
+        ("lm_head Linear 2048->151936", 1, lin_bytes(H, V, 4), lambda: [model._linear(xn, "embed_tokens.weight")]),
+        ("argmax over 151936", 1, B * V * 4, lambda: [L.argmax(logits)]),
+        ("embedding + first RMSNorm", 1, B * H * (2 + 4 + 2),
+         lambda: [L.embedding_rms_norm(model._ids, W("embed_tokens.weight"), W("layers.0.input_layernorm.weight"),
+                                       cfg.rms_norm_eps)]),
+    ]
+    rows = []
+    for name, calls, nbytes, fn in kinds:
+        g = HIPGraph()
+        g.capture(fn)
+        g.replay()
+        L.synchronize()
+        # the graph replays on its own stream: host clock around the launch ... sync of `reps` replays
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g.launch_async()
+        g.sync()
+        us = (time.perf_counter() - t0) * 1e6 / (reps * calls)
+        g.reset()
+        rows.append({"kernel": name, "calls_per_step": calls, "us_per_call": round(us, 2),
+                     "us_per_step": round(us * calls, 1), "bytes_per_call": int(nbytes),
+                     "frac_hbm_peak": round(nbytes / (us * 1e-6) / (HBM_PEAK_GBS * 1e9), 4)})
+    return rows
+
+
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
         cpu_step_hook=None, cfg: TextConfig | None = None, fused_tail: bool = False) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
@@ -85,7 +163,16 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     assert toks.shape == (decode_steps, batch) and toks.min() >= 0 and toks.max() < cfg.vocab_size
     log(f"[decode] {decode_steps} replays: {ms_step:.3f} ms/step, {tok_s:.0f} tok/s "
         f"({100 * tok_s / ceiling:.1f}% of the {ceiling:.0f} tok/s HBM ceiling)")
+    table = per_kernel_table(model, context + decode_steps)
+    in_kernels = sum(r["us_per_step"] for r in table)
+    for r in table:
+        log(f"[decode]   {r['kernel']:<68s} {r['calls_per_step']:3d} x {r['us_per_call']:7.2f} us = {r['us_per_step']:7.1f} us"
+            f"  ({100 * r['frac_hbm_peak']:.1f}% of HBM peak)")
+    log(f"[decode]   sum of the per-kind graphs {in_kernels:.0f} us of the {ms_step * 1e3:.0f} us step")
     result.update({
+        "per_kernel": {"how": "each kind of launch captured for all layers (own weights / caches) and replayed back to "
+                              "back; host clock around 10 replays; bytes are algorithmic",
+                       "rows": table, "sum_us_per_step": round(in_kernels, 1)},
         "metric": "decode tok/s 2B-shape B=16", "value": round(tok_s, 1), "unit": "tok/s",
         "ms_per_step": round(ms_step, 4), "steps": decode_steps, "batch": batch, "context": context,
         "graph_nodes": g.num_nodes, "bytes_per_step": int(avg_bytes),

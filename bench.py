@@ -245,6 +245,99 @@ def cpu_decode_step_hook(cfg, weights, model, first, pos, batch, max_len, log):
 
 
 
+def _cpu_min_us(fn, budget_s=0.6, max_runs=50):
+    """min wall time of fn() in microseconds over a bounded number of runs."""
+    fn()
+    best, spent, n = float("inf"), 0.0, 0
+    while spent < budget_s and n < max_runs:
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best, spent, n = min(best, dt), spent + dt, n + 1
+    return round(best * 1e6, 1)
+
+
+def config_tables(lib, with_cpu=True):
+    """BASELINE's configurations 2, 3 and 4, every point timed with HIP events on the device (through the
+    C ABI, buffers rotated so that nothing is served from the 256 MB memory-side cache) and, where it costs
+    under about a second, the CPU restatement of the same operator on the same shape beside it."""
+    from axono_amd.benchmarks import microbench as mb
+
+    out = {"peaks": {"hbm_GBps": HBM_PEAK_GBS, "mfma_f16_dense_TFLOPs": mb.MFMA_F16_PEAK},
+           "timing": "HIP events around back-to-back launches on the stream the kernels run on; us per launch"}
+    port = None
+    if with_cpu:
+        import oracle
+        port = oracle.port
+        out["cpu_threads"] = port.num_threads()
+    rng = np.random.default_rng(2)
+
+    def h16(*shape, scale=1.0):
+        return (scale * rng.standard_normal(shape)).astype(np.float32).astype(np.float16).astype(np.float32)
+
+    # ---- config 2: the fused elementwise operators at B = 32 -----------------------------------------
+    c2 = []
+    for r in mb.collect(mb.bench_rowops, lib, 200, (32,)):
+        c2.append({"op": r["op"], "us": r["us"], "bytes": r["bytes"], "GBps": r["GBps"],
+                   "frac_hbm": round(r["GBps"] / HBM_PEAK_GBS, 5)})
+    if port is not None:
+        x, res, w = h16(32, 2048), h16(32, 2048), 1 + 0.02 * h16(2048)
+        g, u = h16(32, 6144), h16(32, 6144)
+        q, k = h16(32, 16, 128), h16(32, 8, 128)
+        pos = rng.integers(0, 8192, 32).astype(np.int64)
+        kc = np.zeros((32, 8, 8192, 128), np.float16)
+        vc = np.zeros_like(kc)
+        kn, vn = k.astype(np.float16), h16(32, 8, 128).astype(np.float16)
+        cpu = {"add_rms_norm": lambda: port.add_rms_norm(x, res, w, 1e-6), "silu_mul": lambda: port.silu_mul(g, u),
+               "rope": lambda: (port.rope(q, pos, 1e6), port.rope(k, pos, 1e6)),
+               "kv_append": lambda: port.kv_append(kn, vn, kc, vc, pos)}
+        for rec in c2:
+            for name, fn in cpu.items():
+                if rec["op"].startswith(name):
+                    rec["cpu_us"] = _cpu_min_us(fn)
+        del kc, vc
+    out["config2_elementwise_B32"] = c2
+
+    # ---- config 3: the decode-attention sweep --------------------------------------------------------
+    c3 = []
+    cpu_seq_us = {}
+    if port is not None:
+        for L in (1024, 8192, 32768):
+            q1, k1, v1 = h16(1, 16, 128), h16(L, 8, 128), h16(L, 8, 128)
+            cpu_seq_us[L] = _cpu_min_us(lambda: port.sdpa(q1, k1, v1, False), budget_s=0.8)
+    points = [(B, L, None) for B in (1, 8, 32, 64) for L in (1024, 8192, 32768)]
+    points.append((32, 32768, np.random.default_rng(0).integers(512, 32769, 32)))
+    for B, L, lens in points:
+        nbytes = gqa_bytes(B, int(lens.sum()) if lens is not None else B * L)
+        steps = int(max(10, min(200, 0.15 / (nbytes / 6e12))))
+        r = mb.collect(mb.bench_gqa, lib, B, L, steps, lens)[0]
+        rec = {"B": B, "L": L, "ragged_512_32768": lens is not None, "us": r["us"], "bytes": r["bytes"],
+               "GBps": r["GBps"], "frac_hbm": round(r["GBps"] / HBM_PEAK_GBS, 4),
+               "plan": {"ranges_per_sequence": r["splits"], "keys_per_range": r["chunk"]}, "kv_buffers": r["kv_buffers"]}
+        if lens is None and L in cpu_seq_us:
+            rec["cpu_us_one_sequence"] = cpu_seq_us[L]
+        c3.append(rec)
+    out["config3_gqa_decode_sweep"] = c3
+
+    # ---- config 4: the fp16 Linear ---------------------------------------------------------------------
+    c4 = []
+    shapes = [(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)]
+    for r in mb.collect(mb.bench_linear, lib, 40, shapes, (1, 16, 32, 512), True, 0):
+        M, K, N = r["M"], r["K"], r["N"]
+        rec = {"M": M, "K": K, "N": N, "us": r["us"], "weight_copies_rotated": r["weight_copies"]}
+        if M <= 32:
+            rec.update({"bound": "hbm", "bytes": r["bytes"], "GBps": r["GBps"], "frac_hbm": round(r["GBps"] / HBM_PEAK_GBS, 4)})
+        else:
+            rec.update({"bound": "mfma", "flops": 2 * M * K * N, "TFLOPs": r["TFLOPs"],
+                        "frac_mfma": round(r["TFLOPs"] / mb.MFMA_F16_PEAK, 4)})
+        if port is not None and 2.0 * M * K * N <= 2.1e9:
+            xw, ww = h16(M, K), h16(N, K, scale=0.02)
+            rec["cpu_us"] = _cpu_min_us(lambda: port.linear(xw, ww), budget_s=0.5, max_runs=5)
+        c4.append(rec)
+    out["config4_linear_f16_packed"] = c4
+    return out
+
+
 def smoke_parity(lib):
     """Small invocation checked against the oracle; raises on mismatch."""
     import oracle
@@ -278,6 +371,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode-step", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-point tables of configurations 2-4")
     ap.add_argument("--decode-steps", type=int, default=128)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -342,6 +436,10 @@ def main():
         if qwen3vl_text_bench is not None:
             hook = None if args.no_cpu_baseline else cpu_decode_step_hook
             result["decode_step"] = qwen3vl_text_bench.run(decode_steps=args.decode_steps, log=log, cpu_step_hook=hook)
+
+    if not args.no_configs:
+        result["configs"] = config_tables(lib, with_cpu=not args.no_cpu_baseline)
+        log(f"configs 2-4: {sum(len(v) for v in result['configs'].values() if isinstance(v, list))} points timed")
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_gqa()

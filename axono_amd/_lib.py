@@ -48,6 +48,7 @@ PROTOTYPES = {
     "axhip_graph_replay": (c_i, [c_vp]),
     "axhip_set_ticket_lane": (c_i, [c_i]),
     "axhip_ticket_lane": (c_i, []),
+    "axhip_reset_tickets": (c_i, []),
     "axhip_graph_sync": (c_i, [c_vp]),
     "axhip_graph_destroy": (c_i, [c_vp]),
     "axhip_capture_pool_reset": (c_i, []),
@@ -72,8 +73,10 @@ PROTOTYPES = {
     "axhip_silu_mul": (c_i, [c_vp, c_vp, c_vp, c_i, c_i64, c_vp]),
     "axhip_rms_norm": (c_i, [c_vp, c_vp, c_f, c_vp, c_i, c_i, c_i64, c_i64, c_vp]),
     "axhip_add": (c_i, [c_vp, c_vp, c_vp, c_i, c_i64, c_vp]),
+    "axhip_transpose": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "axhip_cast": (c_i, [c_vp, c_i, c_vp, c_i, c_i64, c_vp]),
     "axhip_rope": (c_i, [c_vp, c_vp, c_f, c_vp, c_i, c_i64, c_i64, c_i64, c_vp]),
+    "axhip_rope_qk": (c_i, [c_vp, c_vp, c_vp, c_f, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "axhip_rope_thd": (c_i, [c_vp, c_vp, c_vp, c_i, c_i, c_i, c_vp, c_i, c_i64, c_i64, c_i64, c_vp]),
     "axhip_mrope_cos_sin": (c_i, [c_vp, c_vp, c_i, c_i, c_vp, c_vp, c_i64, c_i64, c_vp]),
     "axhip_rope_with_cos_sin": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_vp]),
@@ -85,9 +88,6 @@ PROTOTYPES = {
     "axhip_linear_f16_packed": (c_i, [c_vp, c_i, c_vp, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_i, c_vp]),
     "axhip_embedding": (c_i, [c_vp, c_i, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_vp]),
     "axhip_argmax": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
-    "axhip_decode_layer_tail": (c_i, [c_vp] * 12 + [c_i] * 5 + [c_f, c_vp]),
-    "axhip_decode_layer_tail_status": (c_i, [c_i, c_vp]),
-    "axhip_decode_layer_tail_tune": (None, [c_i, c_i]),
     "axhip_prefill_attention": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_gqa_decode_qkv": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i, c_i, c_vp,
                                    c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),

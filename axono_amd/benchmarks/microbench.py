@@ -206,42 +206,6 @@ def bench_sdpa(lib, S, steps, causal, Hq=16, Hkv=8, D=128):
            "TFLOPs": round(fl / us / 1e6, 1), "pct_mfma_f16_peak": round(100 * fl / us / 1e6 / MFMA_F16_PEAK, 2)})
 
 
-def bench_tail(lib, steps, M=16, H=2048, K1=2048, I=6144, N_next=4096, rot=8):
-    """The persistent layer-tail launch, weights rotated through `rot` copies; with phases skipped one
-    by one (timing only) to see where the time goes."""
-    rng = np.random.default_rng(0)
-    sets = []
-    for _ in range(rot):
-        ws = []
-        for n, k, glu in ((H, K1, 0), (2 * I, H, 1), (H, I, 0), (N_next, H, 0)):
-            w = DeviceBuffer.from_numpy((0.02 * rng.standard_normal((n, k))).astype(np.float32).astype(np.float16))
-            p = DeviceBuffer(lib.axhip_linear_f16_packed_bytes(n, k))
-            check(lib.axhip_linear_f16_pack(w.ptr, p.ptr, n, k, glu, None), "pack")
-            check(lib.axhip_synchronize(), "sync")
-            ws.append(p)
-        sets.append(ws)
-    attn = DeviceBuffer.from_numpy(rng.standard_normal((M, K1)).astype(np.float32).astype(np.float16))
-    h = DeviceBuffer.from_numpy(rng.standard_normal((M, H)).astype(np.float32))
-    nw = DeviceBuffer.from_numpy(np.ones(H, np.float32))
-    h_mid, act, h_out, y = DeviceBuffer(M * H * 4), DeviceBuffer(M * I * 2), DeviceBuffer(M * H * 4), DeviceBuffer(M * N_next * 4)
-    st = {"i": 0}
-
-    def step():
-        o, gu_, d, n = sets[st["i"] % rot]
-        st["i"] += 1
-        check(lib.axhip_decode_layer_tail(attn.ptr, h.ptr, o.ptr, nw.ptr, gu_.ptr, d.ptr, nw.ptr, n.ptr, h_mid.ptr, act.ptr,
-                                          h_out.ptr, y.ptr, M, H, K1, I, N_next, 1e-6, None), "tail")
-
-    nb = 2 * (H * K1 + 2 * I * H + H * I + N_next * H)
-    for skip, what in ((0, "all phases"), (31, "barriers only"), (31 + 64, "barriers only, no cache invalidate"), (30, "o_proj"), (13, "gate_up + norm"), (27, "down"),
-                       (7, "next linear + norm"), (15, "norm staging x2")):
-        lib.axhip_decode_layer_tail_tune(0, skip)
-        us = _time(lib, step, steps)
-        _emit({"op": "decode_layer_tail", "M": M, "N_next": N_next, "what": what, "us": round(us, 2),
-               "weight_GBps_if_all": round(nb / us / 1e3, 1)})
-    lib.axhip_decode_layer_tail_tune(0, 0)
-
-
 def bench_copy(lib, mib, steps):
     n = mib * 2**20
     a, b = DeviceBuffer(n), DeviceBuffer(n)
@@ -276,13 +240,12 @@ def bench_rowops(lib, steps=200, row_counts=(32, 4096, 65536)):
         qo, ko = DeviceBuffer(rows * 16 * 256), DeviceBuffer(rows * 8 * 256)
         pos = DeviceBuffer.from_numpy(rng.integers(0, 8192, rows).astype(np.int64))
 
-        def rope2():
-            check(lib.axhip_rope(qx.ptr, pos.ptr, 1e6, qo.ptr, F16, rows, 16, 128, None), "rope")
-            check(lib.axhip_rope(kx.ptr, pos.ptr, 1e6, ko.ptr, F16, rows, 8, 128, None), "rope")
+        def rope_qk():
+            check(lib.axhip_rope_qk(qx.ptr, kx.ptr, pos.ptr, 1e6, qo.ptr, ko.ptr, F16, rows, 16, 8, 128, None), "rope")
 
-        us = _time(lib, rope2, steps)
+        us = _time(lib, rope_qk, steps)
         nb = 2 * rows * 24 * 128 * 2
-        _emit({"op": "rope q+k (2 launches)", "rows": rows, "us": round(us, 2), "bytes": nb,
+        _emit({"op": "rope q+k (one launch)", "rows": rows, "us": round(us, 2), "bytes": nb,
                "GBps": round(nb / us / 1e3, 1), "pct_hbm_peak": round(100 * nb / us / 1e3 / HBM_PEAK, 2)})
     B, Hkv, Lmax, D = 32, 8, 8192, 128
     kc, vc = DeviceBuffer(B * Hkv * Lmax * D * 2), DeviceBuffer(B * Hkv * Lmax * D * 2)
@@ -342,8 +305,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "copy", "rowops", "linear", "linear-packed", "prefill-attn",
-                                     "tail"])
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -373,8 +335,6 @@ def main(argv=None):
                 bench_gqa(lib, B, L, max(10, min(args.steps, int(2e9 // (B * L * 4096)) + 10)))
         lens = np.random.default_rng(0).integers(512, 32769, 32)
         bench_gqa(lib, 32, 32768, 20, lens, tag="gqa_ragged_512_32768")
-    elif args.what == "tail":
-        bench_tail(lib, args.steps)
     elif args.what == "gqa-shapes":
         # other head shapes: group sizes 1, 4 and 8 (four and more run on the matrix cores), D = 64 and 256
         for Hq, Hkv, D in ((8, 8, 128), (32, 8, 128), (64, 8, 128), (32, 4, 128), (32, 8, 64), (16, 8, 64), (16, 8, 256)):

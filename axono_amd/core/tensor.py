@@ -231,6 +231,60 @@ class Tensor:
             self._shape = shape
         return self
 
+    def transpose(self, dim0: int = -2, dim1: int = -1) -> "Tensor":
+        """A new tensor with two dimensions exchanged (a copy: tensors carry no strides).  Negative
+        indices count from the end; equal dims return an alias (Tensor::Transpose,
+        src/core/tensor.cpp:386-424; device kernel src/core/cuda/tensor/transpose.cu)."""
+        nd = self.ndim
+        d0 = dim0 + nd if dim0 < 0 else dim0
+        d1 = dim1 + nd if dim1 < 0 else dim1
+        if not (0 <= d0 < nd and 0 <= d1 < nd):
+            raise ValueError(f"Transpose: invalid dims, ndim={nd}, dim0={dim0}, dim1={dim1}")
+        if d0 == d1:
+            return self.__copy__()
+        if d0 > d1:
+            d0, d1 = d1, d0
+        shape = list(self._shape)
+        shape[d0], shape[d1] = shape[d1], shape[d0]
+        out = Tensor(self._dtype, shape, self._device, _zero=False)
+        if self.num_elements == 0:
+            return out
+        if self._kind == "cpu":
+            src = self._as_numpy(raw_f16=True)
+            out._st.host[:] = np.ascontiguousarray(np.swapaxes(src, d0, d1)).reshape(-1).view(np.uint8)
+            return out
+        outer, mid, inner = _numel(self._shape[:d0]) if d0 else 1, 1, 1
+        for s_ in self._shape[d0 + 1:d1]:
+            mid *= s_
+        for s_ in self._shape[d1 + 1:]:
+            inner *= s_
+        from ..device import current_stream
+        check(_lib.load().axhip_transpose(self.data_ptr, out.data_ptr, DTYPE_SIZE[self._dtype], outer, self._shape[d0],
+                                          mid, self._shape[d1], inner, current_stream()), "transpose")
+        return out
+
+    @property
+    def T(self) -> "Tensor":  # noqa: N802 - the reference's name (core/tensor.py:281-290)
+        return self.transpose()
+
+    # ---- arithmetic: only what the decode path has a kernel for --------------------------------
+    def __add__(self, other) -> "Tensor":
+        """Same-shape elementwise sum on the device (the residual add of a decoder layer); the
+        reference's `+` also broadcasts a bias row and takes scalars through its generic elementwise
+        family, which this build does not carry."""
+        from .. import libaxono
+        if not isinstance(other, Tensor):
+            return NotImplemented
+        return libaxono.add(self, other)
+
+    __radd__ = __add__
+
+    def _no_operator(self, *_):
+        raise NotImplementedError("this build carries the decode path only: of the arithmetic operators, "
+                                  "`+` on equal shapes has a kernel; use NumPy on to_numpy() for the rest")
+
+    __sub__ = __mul__ = __truediv__ = __matmul__ = __neg__ = __abs__ = _no_operator
+
     def fill_zero(self) -> "Tensor":
         self._st.version += 1
         if self._kind == "cpu":
@@ -270,6 +324,69 @@ class Tensor:
             raise ValueError(f"unsupported dtype {arr.dtype}")
         st = _Storage(host=arr.reshape(-1).view(np.uint8), keep=array)
         return cls(dt, list(arr.shape), "cpu", _storage=st)
+
+    @classmethod
+    def from_borrowed(cls, array: np.ndarray) -> "Tensor":
+        """Zero-copy host tensor over a C-contiguous float32 array, or over a uint16 array holding
+        FLOAT16 bit patterns (nanobind_module.cpp:218-236); the array is kept alive by the tensor."""
+        arr = np.asarray(array)
+        if not arr.flags["C_CONTIGUOUS"]:
+            raise ValueError("from_borrowed needs a C-contiguous array")
+        if arr.dtype == np.float32:
+            dt = DataType.FLOAT32
+        elif arr.dtype in (np.uint16, np.float16):
+            dt = DataType.FLOAT16
+        else:
+            raise RuntimeError("from_borrowed: only FLOAT32 / FLOAT16 (as uint16 bit patterns)")
+        return cls(dt, list(arr.shape), "cpu", _storage=_Storage(host=arr.reshape(-1).view(np.uint8), keep=array))
+
+    @classmethod
+    def from_borrowed_i64(cls, array: np.ndarray) -> "Tensor":
+        """Zero-copy host tensor over a C-contiguous int64 array (nanobind_module.cpp:237-250)."""
+        arr = np.asarray(array)
+        if arr.dtype != np.int64 or not arr.flags["C_CONTIGUOUS"]:
+            raise RuntimeError("from_borrowed_i64: a C-contiguous INT64 array is required")
+        return cls(DataType.INT64, list(arr.shape), "cpu", _storage=_Storage(host=arr.reshape(-1).view(np.uint8), keep=array))
+
+    # data_<dtype>() accessors of the binding (nanobind_module.cpp:325-372): a host tensor gives a view
+    # sharing its memory, a device tensor a host copy; the element type is not checked against the
+    # tensor's dtype except for data_float16, which returns int16 bit patterns of a FLOAT16 tensor.
+    def _data_as(self, npdt) -> np.ndarray:
+        npdt = np.dtype(npdt)
+        if self.num_bytes % npdt.itemsize or DTYPE_SIZE[self._dtype] != npdt.itemsize:
+            raise RuntimeError(f"data accessor: {self._dtype.name} elements are not {npdt.itemsize} bytes wide")
+        if self._kind == "cpu":
+            return self._st.host[:self.num_bytes].view(npdt).reshape(self._shape)
+        out = np.empty(self._shape, dtype=npdt)
+        if self.num_bytes:
+            check(_lib.load().axhip_memcpy_d2h(out.ctypes.data, self.data_ptr, self.num_bytes), "data")
+        return out
+
+    def data_int8(self):
+        return self._data_as(np.int8)
+
+    def data_int16(self):
+        return self._data_as(np.int16)
+
+    def data_int32(self):
+        return self._data_as(np.int32)
+
+    def data_int64(self):
+        return self._data_as(np.int64)
+
+    def data_float16(self):
+        if self._dtype != DataType.FLOAT16:
+            raise RuntimeError("data_float16: the tensor is not FLOAT16")
+        return self._data_as(np.int16)
+
+    def data_float32(self):
+        return self._data_as(np.float32)
+
+    def data_float64(self):
+        return self._data_as(np.float64)
+
+    def data_bool(self):
+        return self._data_as(np.bool_)
 
     def _host_typed(self, raw_f16: bool):
         npdt = DTYPE_TO_NUMPY[self._dtype]

@@ -8,7 +8,7 @@
 #include <cstddef>
 #include <cstdint>
 
-#include "axhip.h"
+#include "axhip_experimental.h"  // includes axhip.h
 
 namespace axhip {
 
@@ -39,6 +39,31 @@ inline int raise_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t
   done.fetch_or(bit, std::memory_order_release);
   return AXHIP_OK;
 }
+
+// Compute units of the current device (hipDeviceProp_t::multiProcessorCount), read once per device;
+// 256 (an MI355X) when no device can be asked, so that host-only callers of the planners get the
+// plans of the part the kernels are written for.
+inline int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
+// Zeroes the static ticket counters of the current device (defined beside the counters; see
+// axhip_reset_tickets).  Host-side, synchronous.
+int reset_attention_tickets();
+int reset_argmax_tickets();
 
 inline bool is_float_dtype(int dt) { return dt == AXHIP_FLOAT16 || dt == AXHIP_FLOAT32; }
 

@@ -30,9 +30,10 @@ constexpr int kChunkAlign = 128;      // key ranges start on multiples of this
 constexpr int kMinChunk = 256;
 
 struct Tuning {
-  int target_workgroups = 256;  // workgroups that stream at a time: one per CU keeps HBM busy with
-                                // streaming loads (measured: 256 workgroups 153 us, 1024 163 us at
-                                // B=32 L=8192), and nothing has to be merged when a sequence is one
+  int target_workgroups = 0;    // workgroups that stream at a time; 0 = one per compute unit of the
+                                // device, which keeps HBM busy with streaming loads (measured on the
+                                // 256 CUs of an MI355X: 256 workgroups 153 us, 1024 163 us at B=32
+                                // L=8192), and nothing has to be merged when a sequence is one
   int force_splits = 0;         // > 0: fixed split count for every sequence (measurement sweeps)
   int mfma_groups = 1;          // 0: head groups of four and more stay on the vector path (measurement sweeps)
   int separate_merge = 0;       // 1: merge in a second kernel; 0: the last workgroup of a sequence merges
@@ -53,6 +54,15 @@ __device__ unsigned int g_tickets[AXHIP_TICKET_LANES * kTicketSlots];
 // on a device comes from hipGetSymbolAddress (static_scratch_on_this_device below) and kernels get that
 // pointer as an argument, exactly as they get a caller's workspace.
 static __device__ __align__(256) unsigned char scratch[AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES];
+
+}  // namespace
+int reset_attention_tickets() {
+  void *p = nullptr;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_tickets)) != hipSuccess || !p) return AXHIP_DEVICE_ERROR;
+  if (hipDeviceSynchronize() != hipSuccess) return AXHIP_DEVICE_ERROR;
+  return hipMemset(p, 0, sizeof(unsigned int) * AXHIP_TICKET_LANES * kTicketSlots) == hipSuccess ? AXHIP_OK : AXHIP_DEVICE_ERROR;
+}
+namespace {
 
 constexpr int kMaxDynBatch = 64;  // batches up to this size deal their workgroups by sequence length
 
@@ -77,10 +87,11 @@ struct SplitPlan {
 
 SplitPlan plan_splits(int B, int head_groups, int max_len) {
   SplitPlan p{};
+  const long target_workgroups = g_tuning.target_workgroups > 0 ? g_tuning.target_workgroups : device_cu_count();
   const long hgs = head_groups > 0 ? head_groups : 1;
   const long Bc = B > 0 ? B : 1;
   if (g_tuning.force_splits == 0 && Bc <= kMaxDynBatch) {
-    long active = (g_tuning.target_workgroups + hgs - 1) / hgs;
+    long active = (target_workgroups + hgs - 1) / hgs;
     // no point in ranges shorter than kMinChunk - except that up to eight ranges per sequence may go down
     // to half of that: a short single sequence is all latency, and one tile per workgroup instead of two
     // saves a memory round trip (B=1, L=1024: 8.0 -> 6.9 us; with more ranges the merge eats the gain)
@@ -103,7 +114,7 @@ SplitPlan plan_splits(int B, int head_groups, int max_len) {
     s = g_tuning.force_splits;
   } else {
     const long pairs = Bc * hgs;
-    s = (g_tuning.target_workgroups + pairs - 1) / pairs;
+    s = (target_workgroups + pairs - 1) / pairs;
     const long cap = (max_len + kMinChunk - 1) / kMinChunk;
     if (s > cap) s = cap;
   }
@@ -1220,7 +1231,7 @@ extern "C" {
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits) {
   // a negative target selects the two-kernel form for a forced split count (split kernel + merge kernel)
   g_tuning.separate_merge = target_workgroups < 0 ? 1 : 0;
-  g_tuning.target_workgroups = target_workgroups > 0 ? target_workgroups : Tuning().target_workgroups;
+  g_tuning.target_workgroups = target_workgroups > 0 ? target_workgroups : 0;
   // force_splits >= 1000: keep large head groups on the vector path (for comparison), splits = force_splits - 1000
   g_tuning.mfma_groups = force_splits >= 1000 ? 0 : 1;
   if (force_splits >= 1000) force_splits -= 1000;

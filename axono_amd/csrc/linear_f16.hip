@@ -26,7 +26,7 @@ constexpr int kSkinnyMaxM = 32;
 constexpr int kMaxWaves = 16;   // wavefronts per workgroup of the skinny kernel (K slices)
 
 struct LinearTuning {
-  int target_waves = 2048;  // wavefronts to aim for in the skinny kernel (256 CUs x 8)
+  int target_waves = 0;     // wavefronts to aim for in the skinny kernel; 0 = 8 per compute unit of the device
   int force_nt = 0;         // > 0: rows-of-16 per wavefront (1, 2 or 4)
   int force_waves = 0;      // > 0: wavefronts (K slices) per workgroup (4, 8 or 16)
 };
@@ -53,7 +53,8 @@ SkinnyPlan plan_skinny(int64_t M, int64_t K, int64_t N) {
     p.nt = N >= 8192 ? 2 : 1;
 
   const int64_t ntiles = (N + p.nt * 16 - 1) / (p.nt * 16);
-  int64_t want = g_lin.force_waves > 0 ? g_lin.force_waves : (g_lin.target_waves + ntiles - 1) / ntiles;
+  const int64_t target_waves = g_lin.target_waves > 0 ? g_lin.target_waves : 8 * device_cu_count();
+  int64_t want = g_lin.force_waves > 0 ? g_lin.force_waves : (target_waves + ntiles - 1) / ntiles;
   if (g_lin.force_waves == 0 && want < 8) want = 8;
   int waves = 4;
   while (waves < want && waves < kMaxWaves) waves *= 2;
@@ -953,7 +954,8 @@ int gemm_tiles_per_wave(const PackedArgs &a, int gm) {
   if (g_gemm_tiles == 1 || g_gemm_tiles == 2 || g_gemm_tiles == 4) return g_gemm_tiles;
   const int64_t m_blocks = (a.M + gm - 1) / gm;
   int tw = 4;
-  while (tw > 1 && ((a.N + 64 * tw - 1) / (64 * tw)) * m_blocks < 256) tw /= 2;
+  const int cus = device_cu_count();
+  while (tw > 1 && ((a.N + 64 * tw - 1) / (64 * tw)) * m_blocks < cus) tw /= 2;
   if (a.glu && tw < 2) tw = 2;  // the gated epilogue needs a gate tile and its up tile in one wavefront
   return tw;
 }
@@ -986,7 +988,7 @@ void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
     // 41.2 us against 45.7 with the 64-row tile)
     const bool fits = a.K % kGK == 0 && static_cast<int64_t>(a.M) * a.K < (1ll << 32);
     const int64_t tiles128 = static_cast<int64_t>((a.N + 255) / 256) * ((a.M + 127) / 128);
-    if (fits && (g_gemm_rows == 256 || (g_gemm_rows == 0 && g_gemm_tiles == 0 && tiles128 >= 192))) {
+    if (fits && (g_gemm_rows == 256 || (g_gemm_rows == 0 && g_gemm_tiles == 0 && tiles128 >= 3 * device_cu_count() / 4))) {
       const int n_blocks = (a.N + 255) / 256, m_blocks = (a.M + 127) / 128;
       const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
       hipLaunchKernelGGL((linear_gemm_packed_128_kernel<XT>), dim3(static_cast<unsigned>(nb_pad) * m_blocks), dim3(256), 0,
@@ -998,14 +1000,14 @@ void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
   const int tw = gemm_tiles_per_wave(a, gm == 32 ? 64 : gm);
   // a problem that gives no CU a second workgroup even with the smallest weight tile is bounded by the
   // latency of its K steps: 32 rows of x per workgroup double the workgroups that can overlap
-  if (g_gemm_rows == 0 && tw == 1 && static_cast<int64_t>((a.N + 63) / 64) * ((a.M + 63) / 64) <= 256) gm = 32;
+  if (g_gemm_rows == 0 && tw == 1 && static_cast<int64_t>((a.N + 63) / 64) * ((a.M + 63) / 64) <= device_cu_count()) gm = 32;
   if (gm == 32 && tw != 1) gm = 64;
   constexpr int kDeep = 4;  // steps the loads of the smallest tile run ahead
   // (fp16 x only: fp32 x is converted as it arrives, which would put a wait behind every load)
   // only while no CU gets a second workgroup: with more of them the L2 bandwidth of these small tiles
   // is the bound, not the latency of a step
   if (sizeof(XT) == 2 && tw == 1 && !a.glu && (gm == 32 || gm == 64) && a.K % (kDeep * kGK) == 0 && g_gemm_tiles == 0 &&
-      static_cast<int64_t>((a.N + 63) / 64) * ((a.M + gm - 1) / gm) <= 256) {
+      static_cast<int64_t>((a.N + 63) / 64) * ((a.M + gm - 1) / gm) <= device_cu_count()) {
     const int n_blocks = (a.N + 63) / 64, m_blocks = (a.M + gm - 1) / gm;
     const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
     const dim3 grid(static_cast<unsigned>(nb_pad) * m_blocks);
@@ -1037,7 +1039,7 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
   g_gemm_tiles = gemm_rows >= 1000 ? gemm_rows / 1000 : 0;
   gemm_rows %= 1000;
   g_gemm_rows = (gemm_rows == 32 || gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256) ? gemm_rows : 0;
-  g_lin.target_waves = target_waves > 0 ? target_waves : LinearTuning().target_waves;
+  g_lin.target_waves = target_waves > 0 ? target_waves : 0;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;
 }

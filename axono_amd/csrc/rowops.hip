@@ -402,6 +402,94 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(RopeArgs a, FreqTable ft, 
   }
 }
 
+// Row-blocked form for the common case (dim/2 a multiple of 8, at most 256, rows 16-byte aligned): a
+// workgroup takes RPW = 256 / (dim/2) rows (at least one), first evaluates each row's dim/2 angles once -
+// one accurate sincosf per thread - into LDS, then rotates every head of those rows, of one tensor or of
+// two that share the positions (q and k of a layer: one launch), 16 bytes per access.  The angle
+// arithmetic, which bounds the per-thread form above (one sincosf per 8 elements of a head), is paid
+// once per row instead of once per head.
+struct RopeRowsArgs {
+  const void *x1, *x2;   // [rows, heads1, dim], [rows, heads2, dim] (x2 may be null with heads2 = 0)
+  void *out1, *out2;
+  const int64_t *pos;
+  const float *inv_freq;
+  int64_t rows;
+  int heads1, heads2, dim, h_lim, w_lim;
+};
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kBlock) void rope_rows_kernel(RopeRowsArgs a, FreqTable ft) {
+  const int half = a.dim / 2;
+  const int rpw = half >= kBlock ? 1 : kBlock / half;  // rows per workgroup
+  __shared__ float s_cos[kBlock], s_sin[kBlock];
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpw;
+  const int tid = threadIdx.x;
+  if (tid < rpw * half) {
+    const int r = tid / half, i = tid - r * half;
+    const int64_t row = row0 + r;
+    float sn = 0.f, cs = 1.f;
+    if (row < a.rows) {
+      float ang;
+      if (MODE == kRopeTheta) {
+        ang = static_cast<float>(a.pos[row]) * ft.f[i];
+      } else {
+        const float f = a.inv_freq[i];
+        const int64_t *p = a.pos + row;
+        if (i % 3 == 1 && i < a.h_lim) p += a.rows;
+        else if (i % 3 == 2 && i < a.w_lim) p += 2 * a.rows;
+        ang = static_cast<float>(*p) * f;
+      }
+      sincosf(ang, &sn, &cs);
+    }
+    s_cos[tid] = cs;
+    s_sin[tid] = sn;
+  }
+  __syncthreads();
+  const int chunks = half / 8;
+  const int heads = a.heads1 + a.heads2;
+  const int per_row = heads * chunks;
+  const int items = rpw * per_row;
+  for (int it = tid; it < items; it += kBlock) {
+    const int r = it / per_row, rem = it - r * per_row;
+    const int64_t row = row0 + r;
+    if (row >= a.rows) break;
+    const int hd = rem / chunks, ch = rem - hd * chunks;
+    const bool second = hd >= a.heads1;
+    const int64_t off = second ? (row * a.heads2 + (hd - a.heads1)) * a.dim : (row * a.heads1 + hd) * a.dim;
+    const T *src = static_cast<const T *>(second ? a.x2 : a.x1) + off + ch * 8;
+    T *dst = static_cast<T *>(second ? a.out2 : a.out1) + off + ch * 8;
+    float lo[8], hi[8], olo[8], ohi[8];
+    Row8<T>::load_stream(src, lo);
+    Row8<T>::load_stream(src + half, hi);
+    const float *c = s_cos + r * half + ch * 8, *sn = s_sin + r * half + ch * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      olo[j] = lo[j] * c[j] - hi[j] * sn[j];
+      ohi[j] = hi[j] * c[j] + lo[j] * sn[j];
+    }
+    Row8<T>::store_stream(dst, olo);
+    Row8<T>::store_stream(dst + half, ohi);
+  }
+}
+
+template <int MODE>
+int launch_rope_rows(const RopeRowsArgs &a, const FreqTable &ft, int dtype, hipStream_t st) {
+  const int half = a.dim / 2;
+  const int rpw = half >= kBlock ? 1 : kBlock / half;
+  const unsigned grid = static_cast<unsigned>((a.rows + rpw - 1) / rpw);
+  if (dtype == AXHIP_FLOAT16)
+    hipLaunchKernelGGL((rope_rows_kernel<__half, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft);
+  else
+    hipLaunchKernelGGL((rope_rows_kernel<float, MODE>), dim3(grid), dim3(kBlock), 0, st, a, ft);
+  return launch_status();
+}
+
+// Whether the row-blocked kernel applies: whole 8-pair chunks, 16-byte aligned head rows.
+inline bool rope_rows_ok(int dtype, int64_t dim, const void *x, const void *out) {
+  const int64_t half = dim / 2, esz = dtype == AXHIP_FLOAT16 ? 2 : 4;
+  return half % 8 == 0 && half <= kMaxHalf && (dim * esz) % 16 == 0 && (half * esz) % 16 == 0 && aligned16(x) && aligned16(out);
+}
+
 template <int MODE>
 int launch_rope(const RopeArgs &a, const FreqTable &ft, int dtype, hipStream_t st) {
   if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
@@ -409,6 +497,10 @@ int launch_rope(const RopeArgs &a, const FreqTable &ft, int dtype, hipStream_t s
   if (a.rows == 0) return AXHIP_OK;
   if (!a.x || !a.out) return AXHIP_INVALID_PTR;
   if (!aligned16(a.x) || !aligned16(a.out)) return AXHIP_INVALID_ARGUMENT;
+  if (MODE != kRopeTable && rope_rows_ok(dtype, a.dim, a.x, a.out) && a.rows < (int64_t(1) << 31)) {
+    RopeRowsArgs r{a.x, nullptr, a.out, nullptr, a.pos, a.inv_freq, a.rows, a.heads, 0, a.dim, a.h_lim, a.w_lim};
+    return launch_rope_rows<(MODE == kRopeTable ? kRopeTheta : MODE)>(r, ft, dtype, st);
+  }
   const int chunks = (a.dim / 2 + 7) / 8;
   // heads per thread: as many as still leave about a thousand workgroups
   int hpt = 1;
@@ -549,6 +641,14 @@ constexpr int kArgmaxMaxRows = 1024;  // per ticket lane
 __device__ float g_argmax_val[AXHIP_TICKET_LANES * kArgmaxMaxRows * kArgmaxParts];
 __device__ long long g_argmax_idx[AXHIP_TICKET_LANES * kArgmaxMaxRows * kArgmaxParts];
 __device__ unsigned int g_argmax_ticket[AXHIP_TICKET_LANES * kArgmaxMaxRows];
+}  // namespace
+int reset_argmax_tickets() {
+  void *p = nullptr;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_argmax_ticket)) != hipSuccess || !p) return AXHIP_DEVICE_ERROR;
+  if (hipDeviceSynchronize() != hipSuccess) return AXHIP_DEVICE_ERROR;
+  return hipMemset(p, 0, sizeof(unsigned int) * AXHIP_TICKET_LANES * kArgmaxMaxRows) == hipSuccess ? AXHIP_OK : AXHIP_DEVICE_ERROR;
+}
+namespace {
 
 __device__ __forceinline__ bool better(float ov, int64_t oi, float v, int64_t i) {
   return oi != INT64_MAX && (i == INT64_MAX || ov > v || (ov == v && oi < i));
@@ -653,6 +753,36 @@ __global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restric
   if (threadIdx.x == 0) out[row] = bi == INT64_MAX ? 0 : bi;
 }
 
+
+// dst = src with two dimensions exchanged.  The contiguous source is seen as [outer, A, mid, B, inner]
+// and the destination as [outer, B, mid, A, inner]; one element per thread step, stores coalesced.
+template <typename E>
+__global__ __launch_bounds__(kBlock) void transpose_kernel(const E *__restrict__ src, E *__restrict__ dst, int64_t n,
+                                                            int64_t A, int64_t mid, int64_t Bd, int64_t inner) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) {
+    int64_t t = i / inner;
+    const int64_t in = i - t * inner;
+    const int64_t a = t % A;
+    t /= A;
+    const int64_t m = t % mid;
+    t /= mid;
+    const int64_t b = t % Bd;
+    const int64_t o = t / Bd;
+    dst[i] = src[(((o * A + a) * mid + m) * Bd + b) * inner + in];
+  }
+}
+
+template <typename E>
+int launch_transpose(const void *src, void *dst, int64_t n, int64_t A, int64_t mid, int64_t Bd, int64_t inner,
+                     hipStream_t st) {
+  unsigned grid = blocks_for(n, kBlock);
+  if (grid > 65536u) grid = 65536u;
+  hipLaunchKernelGGL((transpose_kernel<E>), dim3(grid), dim3(kBlock), 0, st, static_cast<const E *>(src),
+                     static_cast<E *>(dst), n, A, mid, Bd, inner);
+  return launch_status();
+}
+
 }  // namespace
 }  // namespace axhip
 
@@ -699,6 +829,23 @@ AXHIP_API int axhip_add(const void *a, const void *b, void *out, int dtype, int6
   return launch_binary<AddOp>(a, b, out, dtype, n, as_stream(stream));
 }
 
+AXHIP_API int axhip_transpose(const void *src, void *dst, int elem_bytes, int64_t outer, int64_t dim_a, int64_t mid,
+                              int64_t dim_b, int64_t inner, axhip_stream stream) {
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) return AXHIP_UNSUPPORTED_TYPE;
+  if (outer < 0 || dim_a < 0 || mid < 0 || dim_b < 0 || inner < 0) return AXHIP_INVALID_ARGUMENT;
+  const int64_t n = outer * dim_a * mid * dim_b * inner;
+  if (n == 0) return AXHIP_OK;
+  if (!src || !dst) return AXHIP_INVALID_PTR;
+  if (src == dst) return AXHIP_INVALID_ARGUMENT;
+  hipStream_t st = as_stream(stream);
+  switch (elem_bytes) {
+    case 1: return launch_transpose<uint8_t>(src, dst, n, dim_a, mid, dim_b, inner, st);
+    case 2: return launch_transpose<uint16_t>(src, dst, n, dim_a, mid, dim_b, inner, st);
+    case 4: return launch_transpose<uint32_t>(src, dst, n, dim_a, mid, dim_b, inner, st);
+    default: return launch_transpose<uint64_t>(src, dst, n, dim_a, mid, dim_b, inner, st);
+  }
+}
+
 AXHIP_API int axhip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n,
                          axhip_stream stream) {
   if (!is_float_dtype(src_dtype) || !is_float_dtype(dst_dtype)) return AXHIP_UNSUPPORTED_TYPE;
@@ -731,6 +878,25 @@ AXHIP_API int axhip_rope(const void *x, const int64_t *pos, float theta, void *o
   RopeArgs a{x, out, pos, nullptr, nullptr, nullptr, rows, static_cast<int>(heads),
              static_cast<int>(dim), 0, 0};
   return launch_rope<kRopeTheta>(a, ft, dtype, as_stream(stream));
+}
+
+AXHIP_API int axhip_rope_qk(const void *q, const void *k, const int64_t *pos, float theta, void *q_out, void *k_out,
+                            int dtype, int64_t rows, int64_t q_heads, int64_t k_heads, int64_t dim, axhip_stream stream) {
+  if (!is_float_dtype(dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (dim <= 0 || dim % 2 != 0 || dim / 2 > kMaxHalf || q_heads <= 0 || k_heads <= 0 || rows < 0) return AXHIP_INVALID_ARGUMENT;
+  if (rows == 0) return AXHIP_OK;
+  if (!q || !k || !q_out || !k_out || !pos) return AXHIP_INVALID_PTR;
+  if (!rope_rows_ok(dtype, dim, q, q_out) || !rope_rows_ok(dtype, dim, k, k_out) || rows >= (int64_t(1) << 31)) {
+    // odd head sizes: the general kernel, one launch per tensor
+    const int rc = axhip_rope(q, pos, theta, q_out, dtype, rows, q_heads, dim, stream);
+    return rc != AXHIP_OK ? rc : axhip_rope(k, pos, theta, k_out, dtype, rows, k_heads, dim, stream);
+  }
+  FreqTable ft;
+  for (int64_t i = 0; i < dim / 2; ++i)
+    ft.f[i] = std::pow(theta, -2.0f * static_cast<float>(i) / static_cast<float>(dim));
+  RopeRowsArgs r{q, k, q_out, k_out, pos, nullptr, rows, static_cast<int>(q_heads), static_cast<int>(k_heads),
+                 static_cast<int>(dim), 0, 0};
+  return launch_rope_rows<kRopeTheta>(r, ft, dtype, as_stream(stream));
 }
 
 AXHIP_API int axhip_rope_thd(const void *x, const int64_t *pos, const float *inv_freq, int t_sec,

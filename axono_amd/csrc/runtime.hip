@@ -93,11 +93,28 @@ void evict_locked(size_t limit) {
   }
 }
 
+// The eviction queue is only consumed while the cache is over its budget, and a block that is reused
+// leaves its entry behind: once stale entries outnumber the cached blocks the queue is rebuilt from its
+// valid entries (the newest entry of every block that is cached now), oldest first as before.
+void compact_evict_locked() {
+  if (g_evict.size() <= 2 * g_cached.size() + 64) return;
+  std::deque<std::pair<uint64_t, void *>> kept;
+  std::unordered_map<void *, bool> seen;
+  for (auto it = g_evict.rbegin(); it != g_evict.rend(); ++it) {
+    auto c = g_cached.find(it->second);
+    if (c == g_cached.end() || c->second != it->first || seen.count(it->second)) continue;
+    seen[it->second] = true;
+    kept.push_front(*it);
+  }
+  g_evict.swap(kept);
+}
+
 void cache_block_locked(void *ptr, const Block &b) {
   const uint64_t key = key_of(b.device, b.size);
   g_free[key].push_back(ptr);
   g_cached[ptr] = key;
   g_evict.emplace_back(key, ptr);
+  compact_evict_locked();
   g_cached_bytes += b.size;
   evict_locked(budget_locked());
 }
@@ -263,10 +280,25 @@ AXHIP_API size_t axhip_cache_budget(void) {
   return budget_locked();
 }
 
+AXHIP_API int axhip_reset_tickets(void) {
+  if (t_capturing) return AXHIP_INVALID_ARGUMENT;
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return AXHIP_OK;  // no device: no counters
+  }
+  const int a = reset_attention_tickets(), b = reset_argmax_tickets();
+  return a != AXHIP_OK ? a : b;
+}
+
 AXHIP_API int axhip_empty_cache(void) {
-  std::lock_guard<std::mutex> lk(g_mu);
-  evict_locked(0);
-  return AXHIP_OK;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    evict_locked(0);
+  }
+  // the clean-up call of a process that recovers from a failed launch: counters a killed launch left
+  // behind go back to zero as well (not while capturing: it synchronises the device)
+  return t_capturing ? AXHIP_OK : axhip_reset_tickets();
 }
 
 // ---- copies ------------------------------------------------------------------------------------

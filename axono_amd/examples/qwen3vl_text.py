@@ -165,10 +165,6 @@ class Qwen3VLTextDecoder(nn.Module):
         self._attn_ws = Tensor(DataType.INT8, [max(wsb, 256)], device)
         self._graph = None
         self._graph_out = None
-        # True: decode batches of at most 16 rows run each layer's post-attention part as ONE persistent
-        # launch (92 graph nodes instead of 232).  Measured slower at the 2B shape (the barriers between its
-        # phases cost what the kernel boundaries cost), so it is off unless asked for.
-        self.fused_tail = False
 
     # ---- pieces ----------------------------------------------------------------------------
     def _w(self, name):
@@ -211,33 +207,6 @@ class Qwen3VLTextDecoder(nn.Module):
                                      cfg.rms_norm_eps)  # [B,H] each
         nl = cfg.num_hidden_layers
         nqd = cfg.num_attention_heads * cfg.head_dim
-        if self.fused_tail and L.decode_layer_tail_supported(B, cfg.hidden_size, nqd, cfg.intermediate_size, 16):
-            # Per layer: the attention launch (q/k norm, M-RoPE, KV append inside), its merge, and ONE
-            # persistent launch for everything behind the attention including the next layer's qkv
-            # projection (after the last layer: the final norm and the lm_head).
-            qkv = self._linear(xn, "layers.0.self_attn.qkv_proj.weight")
-            for i in range(nl):
-                p = f"layers.{i}."
-                if trace is not None:
-                    trace.append(h)
-                kc, vc = cache.get(i)
-                attn = L.gqa_decode_attention_qkv(qkv, self._w(p + "self_attn.q_norm.weight"),
-                                                  self._w(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, pos,
-                                                  self._inv_freq, cfg.mrope_section, cache.seq_lens, kc, vc,
-                                                  cfg.num_attention_heads, max_len, workspace=self._attn_ws)
-                if i + 1 < nl:
-                    nxt_norm, nxt_lin = f"layers.{i + 1}.input_layernorm.weight", f"layers.{i + 1}.self_attn.qkv_proj.weight"
-                else:
-                    nxt_norm, nxt_lin = "norm.weight", "embed_tokens.weight"  # tied lm_head
-                _, h, qkv = L.decode_layer_tail(
-                    attn.reshape([B, nqd]), h, self._packed[p + "self_attn.o_proj.weight"],
-                    self._w(p + "post_attention_layernorm.weight"), self._packed[p + "mlp.gate_up_proj.weight"],
-                    self._packed[p + "mlp.down_proj.weight"], self._w(nxt_norm), self._packed[nxt_lin],
-                    cfg.intermediate_size, self._w(nxt_lin).shape[0], cfg.rms_norm_eps)
-            if trace is not None:
-                trace.append(h)
-            logits = qkv
-            return logits, L.argmax(logits)
         for i in range(nl):
             p = f"layers.{i}."
             if trace is not None:

@@ -111,7 +111,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
 
 
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
-        cpu_step_hook=None, cfg: TextConfig | None = None, fused_tail: bool = False) -> dict:
+        cpu_step_hook=None, cfg: TextConfig | None = None) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
     after the prefill with the model positioned at the first decode step (the benchmark passes a
     hook that times and compares a CPU restatement of one step); its dict is merged into the result."""
@@ -122,7 +122,6 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     max_len = context + decode_steps + 1
     max_len = (max_len + 127) // 128 * 128
     model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0")
-    model.fused_tail = fused_tail
     rng = np.random.default_rng(seed + 1)
     ids = rng.integers(0, cfg.vocab_size, (batch, context)).astype(np.int64)
 
@@ -193,14 +192,11 @@ def main(argv=None):
     ap.add_argument("--gqa-two-kernels", type=int, default=0, metavar="SPLITS",
                     help="attention with a fixed split count and a second merge kernel (the default deals "
                          "workgroups by length and merges in the last workgroup)")
-    ap.add_argument("--fused-tail", action="store_true",
-                    help="each layer's post-attention part as one persistent launch (measured slower; off by default)")
     args = ap.parse_args(argv)
     if args.gqa_two_kernels:
         from .. import _lib
         _lib.load().axhip_gqa_decode_tune(-1, args.gqa_two_kernels)
-    res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
-              fused_tail=args.fused_tail)
+    res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True))
     print(json.dumps(res), flush=True)
 
 

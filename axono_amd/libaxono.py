@@ -309,6 +309,25 @@ def rope(x: Tensor, pos_ids: Tensor, theta: float = 10000.0) -> Tensor:
     return out
 
 
+def rope_qk(q: Tensor, k: Tensor, pos_ids: Tensor, theta: float = 10000.0):
+    """rope(q, pos_ids, theta) and rope(k, pos_ids, theta) in one launch (the two calls of a decoder layer,
+    examples/vlm/qwen3vl/model.py:358-359, share the positions).  Returns (q_out, k_out); same bits as the
+    two separate calls."""
+    op = "rope"
+    _need_hip(op, q, k, pos_ids)
+    _rope_check(op, q)
+    _rope_check(op, k)
+    rows, hq, dim = q.shape
+    if k.shape[0] != rows or k.shape[2] != dim or k.dtype != q.dtype:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if pos_ids.num_elements != rows or pos_ids.dtype != DataType.INT64:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    qo, ko = _new(q.dtype, q.shape, q), _new(k.dtype, k.shape, k)
+    check(_lib_().axhip_rope_qk(q.data_ptr, k.data_ptr, pos_ids.data_ptr, float(theta), qo.data_ptr, ko.data_ptr,
+                                int(q.dtype), rows, hq, k.shape[1], dim, current_stream()), op)
+    return qo, ko
+
+
 def rope_with_cos_sin(x: Tensor, cos: Tensor, sin: Tensor) -> Tensor:
     """nanobind_module.cpp:968-990 -> RopeWithCosSin (sequence.cpp:96-135)."""
     op = "rope_with_cos_sin"
@@ -571,43 +590,6 @@ def qkv_norm_rope_append(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, eps: f
 
 
 TAIL_MAX_ROWS = 16
-
-
-def decode_layer_tail_supported(rows: int, hidden: int, k1: int, inter: int, n_next: int) -> bool:
-    """Shapes axhip_decode_layer_tail is written for."""
-    return (0 < rows <= TAIL_MAX_ROWS and hidden == 2048 and k1 % 2048 == 0 and inter % 2048 == 0 and n_next % 16 == 0)
-
-
-def decode_layer_tail(attn: Tensor, h_in: Tensor, w_o: Tensor, w_post: Tensor, w_gate_up: Tensor, w_down: Tensor,
-                      w_next: Tensor, w_next_linear: Tensor, inter: int, n_next: int, eps: float):
-    """Everything of a decoder layer behind the attention in one launch (rows <= 16): returns
-    (h_mid, h_out, y) = (residual stream after the attention block, residual stream leaving the layer,
-    rmsnorm(h_out, w_next) . W_next^T).  attn FLOAT16 [rows, K1]; h_in FLOAT32 [rows, H]; the four
-    weights are packed (`pack_linear_weight`, gate+up with glu=True); norm weights FLOAT32 [H]."""
-    op = "decode_layer_tail"
-    _need_hip(op, attn, h_in, w_o, w_post, w_gate_up, w_down, w_next, w_next_linear)
-    if attn.dtype != DataType.FLOAT16 or h_in.dtype != DataType.FLOAT32 or w_post.dtype != DataType.FLOAT32 \
-            or w_next.dtype != DataType.FLOAT32:
-        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
-    hidden = h_in.shape[-1]
-    rows = h_in.num_elements // hidden
-    k1 = attn.num_elements // rows if rows else 0
-    lib = _lib_()
-    if (w_post.num_elements != hidden or w_next.num_elements != hidden
-            or w_o.num_bytes != lib.axhip_linear_f16_packed_bytes(hidden, k1)
-            or w_gate_up.num_bytes != lib.axhip_linear_f16_packed_bytes(2 * inter, hidden)
-            or w_down.num_bytes != lib.axhip_linear_f16_packed_bytes(hidden, inter)
-            or w_next_linear.num_bytes != lib.axhip_linear_f16_packed_bytes(n_next, hidden)):
-        raise AxhipError(op, Status.SHAPE_MISMATCH)
-    h_mid = _new(DataType.FLOAT32, [rows, hidden], h_in)
-    act = _new(DataType.FLOAT16, [rows, inter], h_in)
-    h_out = _new(DataType.FLOAT32, [rows, hidden], h_in)
-    y = _new(DataType.FLOAT32, [rows, n_next], h_in)
-    check(lib.axhip_decode_layer_tail(attn.data_ptr, h_in.data_ptr, w_o.data_ptr, w_post.data_ptr, w_gate_up.data_ptr,
-                                      w_down.data_ptr, w_next.data_ptr, w_next_linear.data_ptr, h_mid.data_ptr,
-                                      act.data_ptr, h_out.data_ptr, y.data_ptr, rows, hidden, k1, inter, n_next,
-                                      float(eps), current_stream()), op)
-    return h_mid, h_out, y
 
 
 def prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, start: Tensor | None = None) -> Tensor:

@@ -107,11 +107,18 @@ AXHIP_API axhip_stream axhip_current_stream(void);
  * ranges in the kernel, axhip_argmax over wide rows) take the counters of the calling thread's
  * ticket lane, 0 .. AXHIP_TICKET_LANES-1 (default 0); a captured launch keeps the lane it was captured
  * under.  Launches of these kernels that overlap in time on one device must come from different lanes.
- * A lane holds 8192 (sequence, head group) slots for attention and 128 rows for argmax.  No
+ * A lane holds 65536 (sequence, head group) slots for attention and 1024 rows for argmax.  No
  * reference counterpart (the reference merges in a second kernel, gqa.cu:95-129). */
 #define AXHIP_TICKET_LANES 8
 AXHIP_API int axhip_set_ticket_lane(int lane);
 AXHIP_API int axhip_ticket_lane(void);
+/* Puts every ticket counter of the current device back to zero.  The counters are self-resetting (the
+ * workgroup that takes the last ticket clears it), so this is only needed for recovery: a launch that
+ * ended abnormally (a device error reported by a later call) can leave counters non-zero, and every later
+ * launch of the same slot would then merge early or never.  Synchronises the device; refused with
+ * AXHIP_INVALID_ARGUMENT while the calling thread captures a graph; call it while no attention / argmax
+ * launch is in flight.  axhip_empty_cache calls it as part of its clean-up.  No reference counterpart. */
+AXHIP_API int axhip_reset_tickets(void);
 /* 1 while the calling thread is between axhip_graph_begin_capture and end/abort
  * (cuda::IsCapturing, include/axono/core/cuda/capture.h:19-33). */
 AXHIP_API int axhip_is_capturing(void);
@@ -214,19 +221,15 @@ AXHIP_API int axhip_gqa_decode_static(const void *q, const void *k, const void *
                                       int Hkv, int D, int max_len, int64_t stride_b, int64_t stride_h,
                                       int64_t stride_s, axhip_stream stream);
 
-/* The split plan the launcher uses for these sizes (it depends on host-side sizes only).  For batches of
- * up to 64 sequences the launch holds a fixed number of workgroups which are dealt to the sequences on the
- * device in proportion to their current lengths (n_splits = workgroup slots per sequence, chunk = keys per
- * workgroup if every sequence had max_len keys): whole workgroups per sequence when that is within an eighth
- * of the even share, otherwise equal runs of keys over the sequences laid end to end; the last workgroup of
- * a sequence merges its ranges.
- * Measurement hook: target_workgroups = workgroups to keep streaming (default 256, one per CU; a negative
- * value selects a second merge kernel for a forced split count), force_splits > 0 cuts every sequence into
- * that many ranges (+ 1000: head groups of four and more stay on the vector ALUs instead of the matrix cores,
- * for comparison); 0 restores the defaults.  No reference counterpart (the reference hard-codes
- * min(256, ceil(L/64)), gqa.cu:158-160). */
+/* The split plan the launcher uses for these sizes (it depends on host-side sizes only, so a captured launch
+ * stays valid while the device-side lengths change).  For batches of up to 64 sequences the launch holds a
+ * fixed number of workgroups (one per compute unit) which are dealt to the sequences on the device in
+ * proportion to their current lengths (n_splits = workgroup slots per sequence, chunk = keys per workgroup if
+ * every sequence had max_len keys): whole workgroups per sequence when that is within an eighth of the even
+ * share, otherwise equal runs of keys over the sequences laid end to end; the last workgroup of a sequence
+ * merges its ranges.  Larger batches cut every sequence into n_splits ranges of chunk keys.  No reference
+ * counterpart (the reference hard-codes min(256, ceil(L/64)), gqa.cu:158-160). */
 AXHIP_API void axhip_gqa_decode_plan(int B, int Hq, int Hkv, int max_len, int *n_splits, int *chunk);
-AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
 
 /* General attention for prefill and short contexts: q [Sq,Hq,D], k/v [Skv,Hkv,D] contiguous,
  * optional causal mask with the reference's rule (keys 0..t visible when Skv >= t+1).
@@ -292,6 +295,14 @@ AXHIP_API int axhip_rms_norm_ex(const void *x, const void *weight, float eps, vo
 AXHIP_API int axhip_add(const void *a, const void *b, void *out, int dtype, int64_t n,
                         axhip_stream stream);
 
+/* dst = src with two dimensions exchanged (a copy; any element size of 1, 2, 4 or 8 bytes).  The
+ * contiguous source is described as [outer, dim_a, mid, dim_b, inner] and the destination is
+ * [outer, dim_b, mid, dim_a, inner]: for Tensor::Transpose(d0 < d1) outer / mid / inner are the products of
+ * the extents before d0, between d0 and d1, and after d1.  Replaces cuda::tensor::TransposeKernel
+ * (src/core/cuda/tensor/transpose.cu:17-143, called from src/core/tensor.cpp:386-424). */
+AXHIP_API int axhip_transpose(const void *src, void *dst, int elem_bytes, int64_t outer, int64_t dim_a,
+                              int64_t mid, int64_t dim_b, int64_t inner, axhip_stream stream);
+
 /* fp16 <-> fp32 conversion, IEEE round-to-nearest-even.  Replaces Half2FloatKernel /
  * Float2HalfKernel, src/core/cuda/tensor/kernel.cu:175-223 (Tensor::CastTo on device). */
 AXHIP_API int axhip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n,
@@ -307,6 +318,15 @@ AXHIP_API int axhip_cast(const void *src, int src_dtype, void *dst, int dst_dtyp
  * dim <= 512. */
 AXHIP_API int axhip_rope(const void *x, const int64_t *pos, float theta, void *out, int dtype,
                          int64_t rows, int64_t heads, int64_t dim, axhip_stream stream);
+
+/* axhip_rope on the q and the k heads of the same rows in one launch (they share the positions, so each
+ * row's angles are evaluated once): q [rows, q_heads, dim] -> q_out, k [rows, k_heads, dim] -> k_out.  Same
+ * arithmetic as two axhip_rope calls, bit for bit.  The reference's operator takes one tensor per call
+ * (src/ops/cuda/sequence.cu:318-342) and its model calls it twice per layer
+ * (examples/vlm/qwen3vl/model.py:358-359). */
+AXHIP_API int axhip_rope_qk(const void *q, const void *k, const int64_t *pos, float theta, void *q_out,
+                            void *k_out, int dtype, int64_t rows, int64_t q_heads, int64_t k_heads,
+                            int64_t dim, axhip_stream stream);
 
 /* M-RoPE with interleaved T/H/W channels: pos device int64[3, rows], inv_freq device fp32[dim/2];
  * channel i uses H if i%3==1 && i<3*h_sec, W if i%3==2 && i<3*w_sec, else T (t_sec is unused, as
@@ -339,13 +359,6 @@ AXHIP_API int axhip_rope_with_cos_sin(const void *x, const float *cos_t, const f
  * bias/zero fill + cublasGemmEx).  K % 8 == 0.  `workspace` holds split-K partial sums for skinny
  * M: at least axhip_linear_f16_workspace_bytes(M,K,N) bytes (may be 0, then pass NULL). */
 AXHIP_API size_t axhip_linear_f16_workspace_bytes(int64_t M, int64_t K, int64_t N);
-/* Measurement hook for the skinny-M kernel's plan (0 restores a default): wavefronts to aim for,
- * 16-row groups of W per wavefront (1, 2 or 4), wavefronts (K slices) per workgroup (4, 8, 16);
- * for the M > 32 GEMM, the tile: 64 or 128 rows of x per workgroup (128: one workgroup per CU), 256 = the
- * 256 x 128 tile at two workgroups per CU (the default for large problems), plus 1000 t to force t = 1, 2 or 4 row
- * tiles of W per wavefront (64, 128 or 256 weight rows per workgroup; by default the largest that still
- * gives every CU a workgroup).  No reference counterpart (the reference leaves the choice to cuBLAS). */
-AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows);
 AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const void *bias,
                                void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
                                void *workspace, size_t workspace_bytes, axhip_stream stream);
@@ -432,29 +445,6 @@ AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float
                                    void *k_cache, void *v_cache, void *out, void *workspace,
                                    size_t workspace_bytes, int cache_dtype, int B, int Hq, int Hkv, int D,
                                    int cache_rows, int max_len, axhip_stream stream);
-
-/* Everything of a decoder layer behind the attention, for M <= 16 rows, in one persistent launch:
- *   h_mid = attn . Wo^T + h_in;  act = silu(g) * u with [g | u] = rmsnorm(h_mid, w_post) . Wgu^T;
- *   h_out = act . Wd^T + h_mid;  y = rmsnorm(h_out, w_next) . Wn^T
- * i.e. o_proj, AddRmsNorm, gate/up + SiluMul, down_proj, AddRmsNorm and the next Linear (the next layer's
- * qkv projection or the lm_head) of examples/vlm/qwen3vl/model.py:371-373,384,408-436,483-486, with the
- * arithmetic of the single operators.  attn fp16 [M,K1]; h_in / h_mid / h_out fp32 [M,H]; act fp16 [M,I]
- * scratch; y fp32 [M,N_next]; norm weights fp32 [H]; the four weight matrices packed by
- * axhip_linear_f16_pack (gate+up with glu = 1).  H <= 2048 and a multiple of 2048 / ... see the checks:
- * H, K1 and I must be multiples of 2048 (K slices of whole 128-column steps for 16 wavefronts), N_next a
- * multiple of 16.  The workgroups of the launch synchronise among themselves and must all be resident
- * (one per CU is launched): launches of this entry point must not overlap on a device.  No reference
- * counterpart. */
-AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const void *w_o, const float *w_post,
-                                      const void *w_gate_up, const void *w_down, const float *w_next,
-                                      const void *w_next_linear, float *h_mid, void *act, float *h_out, float *y,
-                                      int M, int H, int K1, int I, int N_next, float eps, axhip_stream stream);
-/* Barrier waits of axhip_decode_layer_tail that ran out (0 in a healthy process); reset != 0 also clears the
- * barrier state (only while no such launch is in flight).  Measurement hook: workgroups to launch (0 = one
- * per CU, at most 256); skip_phases: bit p set = phase p + 1 does no work, bit 4 = no norm staging, bit 6 =
- * no cache invalidate behind the barriers (timing only: results are then meaningless). */
-AXHIP_API int axhip_decode_layer_tail_status(int reset, unsigned *failed_waits);
-AXHIP_API void axhip_decode_layer_tail_tune(int workgroups, int skip_phases);
 
 /* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
  * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0.  out_dtype

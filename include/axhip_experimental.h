@@ -1,0 +1,34 @@
+/*
+ * axhip_experimental.h - measurement hooks of libaxhip.so.  NOT part of the drop-in boundary (axhip.h):
+ * these entry points exist so that tests can force every kernel variant and benchmarks can sweep plans.
+ * They set process-global, unsynchronised state: call them from one thread while no operator call is in
+ * flight, and restore the defaults (all arguments 0) afterwards.  No reference counterparts (the
+ * reference hard-codes its split count, src/ops/cuda/gqa.cu:158-160, and leaves GEMM algorithm choice to
+ * cuBLAS, src/ops/cuda/linear.cu:131-138).
+ */
+#ifndef AXHIP_EXPERIMENTAL_H_
+#define AXHIP_EXPERIMENTAL_H_
+
+#include "axhip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Decode attention split plan.  target_workgroups = workgroups to keep streaming (default: one per compute
+ * unit; a negative value selects a second merge kernel for a forced split count instead of the in-kernel
+ * merge), force_splits > 0 cuts every sequence into that many ranges (+ 1000: head groups of four and more
+ * stay on the vector ALUs instead of the matrix cores, for comparison); 0 restores the defaults. */
+AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
+
+/* fp16 Linear plans (0 restores a default).  Skinny M: wavefronts to aim for, 16-row groups of W per
+ * wavefront (1, 2 or 4), wavefronts (K slices) per workgroup (4, 8, 16).  M > 32 GEMM, gemm_rows: 64 or 128
+ * rows of x per workgroup (128: one workgroup per CU), 256 = the 256 x 128 tile at two workgroups per CU
+ * (the default for large problems), plus 1000 t to force t = 1, 2 or 4 row tiles of W per wavefront (64, 128
+ * or 256 weight rows per workgroup; by default the largest that still gives every CU a workgroup). */
+AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXHIP_EXPERIMENTAL_H_ */

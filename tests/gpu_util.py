@@ -102,6 +102,16 @@ def rope(x, pos, theta):
     return do.download(x.dtype, x.shape)
 
 
+def rope_qk(q, k, pos, theta):
+    rows, hq, dim = q.shape
+    hk = k.shape[1]
+    dq, dk, dp = dev(q), dev(k), dev(np.asarray(pos, np.int64))
+    oq, ok = DeviceBuffer(q.nbytes), DeviceBuffer(k.nbytes)
+    _run("axhip_rope_qk", dq.ptr, dk.ptr, dp.ptr, theta, oq.ptr, ok.ptr, dt(q), rows, hq, hk, dim, None)
+    synchronize()
+    return oq.download(q.dtype, q.shape), ok.download(k.dtype, k.shape)
+
+
 def rope_thd(x, pos3, inv_freq, section):
     rows, heads, dim = x.shape
     dx, dp, df, do = dev(x), dev(np.asarray(pos3, np.int64)), dev(np.asarray(inv_freq, np.float32)), DeviceBuffer(x.nbytes)

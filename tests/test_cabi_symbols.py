@@ -8,9 +8,15 @@ from axono_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "axhip.h")).read()
+def declared_symbols(headers=("axhip.h", "axhip_experimental.h")):
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in headers)
     return sorted(set(re.findall(r"AXHIP_API\s+[\w\s\*]+?\b(axhip_\w+)\s*\(", text)))
+
+
+def test_measurement_hooks_are_not_part_of_the_boundary_header():
+    boundary = declared_symbols(("axhip.h",))
+    assert not [n for n in boundary if n.endswith("_tune")]
+    assert sorted(declared_symbols(("axhip_experimental.h",))) == ["axhip_gqa_decode_tune", "axhip_linear_f16_tune"]
 
 
 def test_header_declares_the_path():

@@ -140,6 +140,34 @@ def test_rope_fp16_config2():
     np.testing.assert_allclose(gu.rope(x, pos, 1e6), port.rope(x, pos, 1e6), rtol=0, atol=TOL32)
 
 
+@pytest.mark.parametrize("rows,hq,hk,dim", [(32, 16, 8, 128), (4099, 16, 8, 128), (7, 3, 5, 64), (130, 4, 2, 96),
+                                            (9, 2, 1, 512), (5, 2, 2, 8)])
+def test_rope_q_and_k_in_one_launch(rows, hq, hk, dim):
+    """axhip_rope_qk: the q and k heads of the same rows in one launch, bit-identical to two axhip_rope
+    calls and within tolerance of the oracle; fp16 and fp32; row counts that leave the last workgroup
+    partly empty; head sizes of 64 / 96 / 512 and one (8) that takes the general kernel."""
+    rng = np.random.default_rng(rows + dim)
+    pos = rng.integers(0, 8192, rows).astype(np.int64)
+    for dtype in (np.float16, np.float32):
+        q = rng.standard_normal((rows, hq, dim)).astype(np.float32).astype(dtype)
+        k = rng.standard_normal((rows, hk, dim)).astype(np.float32).astype(dtype)
+        gq, gk = gu.rope_qk(q, k, pos, 1e6)
+        bits = np.uint16 if dtype == np.float16 else np.uint32
+        np.testing.assert_array_equal(gq.view(bits), gu.rope(q, pos, 1e6).view(bits))
+        np.testing.assert_array_equal(gk.view(bits), gu.rope(k, pos, 1e6).view(bits))
+        if dtype == np.float16:
+            assert_fp16_close(gq, port.rope(q, pos, 1e6))
+            assert_fp16_close(gk, port.rope(k, pos, 1e6))
+        else:
+            np.testing.assert_allclose(gq, port.rope(q, pos, 1e6), rtol=0, atol=TOL32)
+            np.testing.assert_allclose(gk, port.rope(k, pos, 1e6), rtol=0, atol=TOL32)
+    l = gu.lib()
+    assert l.axhip_rope_qk(None, None, None, 1e6, None, None, 5, 4, 2, 1, 7, None) == 1    # odd dim
+    assert l.axhip_rope_qk(None, None, None, 1e6, None, None, 5, 4, 2, 1, 8, None) == 7    # null pointers
+    assert l.axhip_rope_qk(None, None, None, 1e6, None, None, 5, 0, 2, 1, 8, None) == 0    # no rows
+    assert l.axhip_rope_qk(None, None, None, 1e6, None, None, 2, 4, 2, 1, 8, None) == 3    # INT32 data
+
+
 def test_mrope_family():
     rng = np.random.default_rng(23)
     rows = 33

@@ -57,6 +57,28 @@ def test_tensor_device_round_trip_and_zero_init(hip_env):
         Tensor(DataType.FLOAT32, [1], "hip:7")
 
 
+def test_transpose_and_plus_on_the_device():
+    """Tensor.transpose / T on hip (axhip_transpose) for every element width and dim pair, and `+`."""
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((3, 5, 4, 7)).astype(np.float32)
+    d = t(a)
+    for d0, d1 in ((0, 1), (0, 3), (1, 2), (2, 3), (1, 3), (-1, -2), (3, 0)):
+        np.testing.assert_array_equal(d.transpose(d0, d1).to_numpy(), np.swapaxes(a, d0, d1))
+    np.testing.assert_array_equal(t(a[0, 0]).T.to_numpy(), a[0, 0].T)
+    h = a.astype(np.float16)
+    np.testing.assert_array_equal(t(h).transpose(1, 3).numpy(), np.swapaxes(h, 1, 3))
+    i64 = rng.integers(-9, 9, (6, 10)).astype(np.int64)
+    np.testing.assert_array_equal(ids_t(i64).T.to_numpy(), i64.T)
+    big = rng.standard_normal((1024, 2048)).astype(np.float32)
+    np.testing.assert_array_equal(t(big).T.to_numpy(), big.T)
+    assert d.transpose(2, 2).data_ptr == d.data_ptr        # equal dims: an alias
+    b = rng.standard_normal(a.shape).astype(np.float32)
+    np.testing.assert_array_equal((d + t(b)).to_numpy(), a + b)
+    np.testing.assert_array_equal(d.data_float32(), a)     # a device tensor's accessor is a host copy
+    with pytest.raises(NotImplementedError):
+        d * d
+
+
 def test_fused_ops_reference_cases():
     rs = np.random.RandomState(0)
     g, u = rs.randn(37, 53).astype(np.float32), rs.randn(37, 53).astype(np.float32)
@@ -431,6 +453,37 @@ def test_allocator_cache_and_budget():
     del z
     assert L.cached_bytes() <= 1 << 20
     L.set_cache_budget(64 << 30)
+    # many release / reuse cycles of a few sizes (the eviction queue is compacted, the cache stays exact)
+    L.empty_cache()
+    for i in range(5000):
+        t1 = Tensor(DataType.INT8, [4096 * (1 + i % 3)], DEV, _zero=False)
+        del t1
+    assert L.cached_bytes() == 4096 * (1 + 2 + 3)
+    L.set_cache_budget(4096 * 3)                   # oldest first: the newest block that still fits stays
+    assert 0 < L.cached_bytes() <= 4096 * 3
+    L.set_cache_budget(64 << 30)
+    L.empty_cache()
+    assert L.cached_bytes() == 0
+
+
+def test_ticket_counters_can_be_reset_for_recovery():
+    """axhip_reset_tickets (also part of empty_cache) zeroes the static ticket counters; attention that
+    merges key ranges in the kernel and the wide argmax give the same results before and after."""
+    from axono_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(31)
+    q = rng.standard_normal((1, 16, 128)).astype(np.float32)
+    k = rng.standard_normal((3000, 8, 128)).astype(np.float32)
+    v = rng.standard_normal((3000, 8, 128)).astype(np.float32)
+    x = rng.standard_normal((3, 151936)).astype(np.float32)
+    before = axono.gqa_decode_attention(t(q), t(k), t(v)).to_numpy()
+    am_before = axono.argmax(t(x)).to_numpy()
+    assert lib.axhip_reset_tickets() == 0
+    L.empty_cache()
+    np.testing.assert_array_equal(axono.gqa_decode_attention(t(q), t(k), t(v)).to_numpy(), before)
+    np.testing.assert_array_equal(axono.argmax(t(x)).to_numpy(), am_before)
+    np.testing.assert_array_equal(am_before, x.argmax(-1))
+    np.testing.assert_allclose(before, port.gqa_decode(q, k, v), rtol=0, atol=1e-5)
 
 
 def test_axm_weights_go_straight_to_the_device(tmp_path):

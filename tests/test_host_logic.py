@@ -226,3 +226,45 @@ def test_missing_library_raises_instead_of_falling_back(monkeypatch, tmp_path):
     (tmp_path / "libaxhip.so").write_bytes(b"not a shared object")
     with pytest.raises(RuntimeError):
         _lib.load()
+
+
+def test_tensor_transpose_borrowed_and_accessors_on_host():
+    """Tensor.transpose / T, from_borrowed[_i64] and the data_<dtype>() accessors of the reference's binding
+    (axono/python/src/nanobind_module.cpp:206-377) on host tensors."""
+    a = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+    t = Tensor.from_numpy(a)
+    np.testing.assert_array_equal(t.transpose().to_numpy(), np.swapaxes(a, -2, -1))
+    np.testing.assert_array_equal(t.transpose(0, 2).to_numpy(), np.swapaxes(a, 0, 2))
+    np.testing.assert_array_equal(t.transpose(-1, 0).to_numpy(), np.swapaxes(a, 0, 2))
+    assert t.transpose(1, 1).shape == [2, 3, 4]
+    m = Tensor.from_numpy(a[0])
+    np.testing.assert_array_equal(m.T.to_numpy(), a[0].T)
+    with pytest.raises(ValueError):
+        t.transpose(0, 3)
+    # borrowed memory is shared, both ways
+    b = np.ones((2, 5), np.float32)
+    tb = Tensor.from_borrowed(b)
+    b[1, 2] = 7
+    assert tb.dtype == DataType.FLOAT32 and tb.to_numpy()[1, 2] == 7
+    tb.data_float32()[0, 0] = -3
+    assert b[0, 0] == -3
+    h = np.array([1.0, -0.5, 65504.0], np.float16)
+    th = Tensor.from_borrowed(h.view(np.uint16))
+    assert th.dtype == DataType.FLOAT16
+    np.testing.assert_array_equal(th.data_float16(), h.view(np.int16))
+    np.testing.assert_array_equal(th.numpy(), h)
+    ti = Tensor.from_borrowed_i64(np.arange(4, dtype=np.int64))
+    assert ti.dtype == DataType.INT64 and list(ti.data_int64()) == [0, 1, 2, 3]
+    with pytest.raises(RuntimeError):
+        Tensor.from_borrowed(np.zeros(3, np.float64))
+    with pytest.raises(RuntimeError):
+        Tensor.from_borrowed_i64(np.zeros(3, np.int32))
+    with pytest.raises(RuntimeError):
+        tb.data_float16()
+    with pytest.raises(RuntimeError):
+        tb.data_int64()                      # 4-byte elements are not read as 8-byte ones
+    assert tb.data_int32().dtype == np.int32   # same width: the bits reinterpreted, as the binding does
+    # operators outside the decode path say so instead of computing something else
+    for bad in (lambda: tb - tb, lambda: tb * tb, lambda: tb / tb, lambda: tb @ tb, lambda: -tb, lambda: abs(tb)):
+        with pytest.raises(NotImplementedError):
+            bad()

@@ -64,6 +64,9 @@ PROTOTYPES = {
                                c_i64, c_i64, c_i64, c_vp]),
     "axhip_gqa_decode_static": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i,
                                       c_i64, c_i64, c_i64, c_vp]),
+    "axhip_gqa_decode_paged": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_i,
+                                     c_vp]),
+    "axhip_kv_append_paged": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_sdpa": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_kv_append": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_concat": (c_i, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),

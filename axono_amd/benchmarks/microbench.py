@@ -2,6 +2,7 @@
 
     python -m axono_amd.benchmarks.microbench gqa   [--B 32 --L 8192 --steps 100 --ragged]
     python -m axono_amd.benchmarks.microbench gqa-sweep
+    python -m axono_amd.benchmarks.microbench gqa-paged
     python -m axono_amd.benchmarks.microbench copy  [--mib 1024 --steps 20]
     python -m axono_amd.benchmarks.microbench rowops
     python -m axono_amd.benchmarks.microbench linear
@@ -125,6 +126,53 @@ def bench_gqa(lib, B, L, steps, lens=None, n_rot=None, Hq=16, Hkv=8, D=128, tag=
            "GBps": round(gbs, 1), "pct_hbm_peak": round(100 * gbs / HBM_PEAK, 1), "splits": s.value,
            "chunk": c.value, "kv_buffers": n_rot})
     return us
+
+
+def bench_gqa_paged(lib, B, L, steps, lens=None, Hq=16, Hkv=8, D=128, n_rot=None, seed=0):
+    """Decode attention over a paged cache (pools [n_pages, Hkv, 128, D] fp16) whose pages were handed out in a
+    random order, beside the dense cache of the same size."""
+    P = 128
+    pages_per_seq = (L + P - 1) // P
+    n_pages = B * pages_per_seq
+    elems = n_pages * Hkv * P * D
+    if n_rot is None:
+        n_rot = max(2, min(8, int(2**30 // (elems * 4)) + 1))
+    pools = []
+    for r in range(n_rot):
+        kb, vb = DeviceBuffer(elems * 2), DeviceBuffer(elems * 2)
+        _rand_fill(kb, elems * 2, 2 * r)
+        _rand_fill(vb, elems * 2, 2 * r + 1)
+        pools.append((kb, vb))
+    rng = np.random.default_rng(seed)
+    table = rng.permutation(n_pages).astype(np.int32).reshape(B, pages_per_seq)
+    dt_ = DeviceBuffer.from_numpy(table)
+    q = DeviceBuffer.from_numpy(rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16))
+    out = DeviceBuffer(B * Hq * D * 2)
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, L)
+    ws = DeviceBuffer(max(wsb, 256))
+    dl = DeviceBuffer.from_numpy(np.asarray(lens, np.int32)) if lens is not None else None
+    state = {"i": 0}
+
+    def paged():
+        kb, vb = pools[state["i"] % n_rot]
+        state["i"] += 1
+        check(lib.axhip_gqa_decode_paged(q.ptr, kb.ptr, vb.ptr, dt_.ptr, dl.ptr if dl else None, out.ptr, ws.ptr, wsb, F16,
+                                         B, Hq, Hkv, D, L, pages_per_seq, n_pages, None), "gqa_decode_paged")
+
+    def dense():  # the same buffers read as a dense [B, Hkv, pages_per_seq * 128, D] cache
+        kb, vb = pools[state["i"] % n_rot]
+        state["i"] += 1
+        rows = pages_per_seq * P
+        check(lib.axhip_gqa_decode(q.ptr, kb.ptr, vb.ptr, dl.ptr if dl else None, out.ptr, ws.ptr, wsb, F16, B, Hq, Hkv, D, L,
+                                   Hkv * rows * D, rows * D, D, None), "gqa_decode")
+
+    L_sum = int(np.sum(lens)) if lens is not None else B * L
+    nbytes = 2 * Hkv * D * 2 * L_sum + 2 * Hq * D * 2 * B
+    for name, fn in (("gqa_dense", dense), ("gqa_paged_random_pages", paged)):
+        us = _time(lib, fn, steps)
+        _emit({"op": name, "B": B, "L": L, "ragged": lens is not None, "pages": n_pages, "us": round(us, 2), "bytes": nbytes,
+               "GBps": round(nbytes / us / 1e3, 1), "pct_hbm_peak": round(100 * nbytes / us / 1e3 / HBM_PEAK, 1),
+               "kv_buffers": n_rot})
 
 
 def bench_gqa_step_form(lib, B, L, steps, Hq=16, Hkv=8, D=128, rows=None, n_rot=4):
@@ -305,7 +353,7 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "gqa-paged", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -340,6 +388,10 @@ def main(argv=None):
         for Hq, Hkv, D in ((8, 8, 128), (32, 8, 128), (64, 8, 128), (32, 4, 128), (32, 8, 64), (16, 8, 64), (16, 8, 256)):
             for B, L in ((32, 8192), (16, 4160), (4, 8192), (1, 32768)):
                 bench_gqa(lib, B, L, min(args.steps, 50), Hq=Hq, Hkv=Hkv, D=D, tag=f"gqa_Hq{Hq}_Hkv{Hkv}_D{D}")
+    elif args.what == "gqa-paged":
+        for B, L in ((32, 8192), (16, 4160), (8, 8192), (64, 1024), (1, 32768)):
+            bench_gqa_paged(lib, B, L, min(args.steps, 100))
+        bench_gqa_paged(lib, 32, 32768, 20, np.random.default_rng(0).integers(512, 32769, 32))
     elif args.what == "gqa-step":
         bench_gqa_step_form(lib, args.B if args.B != 32 else 16, args.L if args.L != 8192 else 4160, args.steps,
                             rows=args.rows or None)

@@ -20,6 +20,8 @@
 // in the same launch; a second small merge kernel is kept behind the tuning hook for comparison.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace axhip {
 namespace {
 
@@ -241,6 +243,11 @@ struct DecodeArgs {
   const int64_t *pos;       // [3, B]
   const float *inv_freq;    // [D/2]
   int h_lim, w_lim, cache_rows;
+  // Paged cache (template parameter PAGED): a.k / a.v are pools [n_pages, Hkv, kPageKeys, D]; key s of
+  // sequence b is row s % kPageKeys of page page_table[b * max_pages + s / kPageKeys].
+  const int32_t *page_table;
+  int max_pages;
+  int64_t page_stride;  // elements per page: Hkv * kPageKeys * D
 };
 
 // Split partials travel between workgroups that may sit on different XCDs, whose L2 caches are not
@@ -340,17 +347,40 @@ __device__ __forceinline__ void norm_rope_row(const DecodeArgs &a, const float *
   }
 }
 
+// Where key row `row` of the workgroup's (sequence, kv head) starts, as an element offset from the
+// workgroup's base pointers.  Dense: rows lie stride_s elements apart.  Paged: the sequence's keys live in
+// pages of kPageKeys rows scattered over a pool [n_pages, Hkv, kPageKeys, D]; the page numbers of the
+// workgroup's key range sit in LDS (filled from the page table before the first tile).
+constexpr int kPageShift = 7;
+constexpr int kPageKeys = 1 << kPageShift;      // keys per page: one tile of the fp16 D=128 kernel
+constexpr int kMaxRangePages = 1025;            // page numbers a workgroup can hold: ranges of up to 131072 keys
+struct DenseRows {
+  int64_t stride_s;
+  __device__ __forceinline__ int64_t operator()(int row) const { return row * stride_s; }
+};
+typedef const int __attribute__((address_space(3))) *lds_cint_ptr;
+struct PagedRows {
+  lds_cint_ptr pages;   // page numbers of pages first_page, first_page + 1, ... of this sequence
+  int first_page;
+  int row_elems;        // D
+  int64_t page_stride;  // Hkv * kPageKeys * D
+  __device__ __forceinline__ int64_t operator()(int row) const {
+    return pages[(row >> kPageShift) - first_page] * page_stride + (row & (kPageKeys - 1)) * row_elems;
+  }
+};
+
 // One tile: U load instructions per lane for K and for V (U*RG key rows per workgroup).
-template <typename T, int D, int U, bool CHECK>
-__device__ __forceinline__ void tile_load(const T *kb, const T *vb, int64_t stride_s, int base, int rg, int s1,
+template <typename T, int D, int U, bool CHECK, typename ROWS>
+__device__ __forceinline__ void tile_load(const T *kb, const T *vb, const ROWS &rows, int base, int rg, int s1,
                                           Frag8<T> (&kr)[U], Frag8<T> (&vr)[U]) {
   constexpr int RG = kThreads / (D / 8);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int row = base + u * RG + rg;
     if (!CHECK || row < s1) {
-      kr[u].template load_stream<FragMap<T, D>::kSecond>(kb + row * stride_s);  // read once: streaming loads
-      vr[u].template load_stream<FragMap<T, D>::kSecond>(vb + row * stride_s);
+      const int64_t off = rows(row);
+      kr[u].template load_stream<FragMap<T, D>::kSecond>(kb + off);  // read once: streaming loads
+      vr[u].template load_stream<FragMap<T, D>::kSecond>(vb + off);
     } else {
       kr[u].zero();
       vr[u].zero();
@@ -395,13 +425,13 @@ __device__ __forceinline__ void tile_update(const Frag8<T> (&kr)[U], const Frag8
   }
 }
 
-template <typename T, int D, int G, int U, bool CHECK>
-__device__ __forceinline__ void decode_tile(const T *kb, const T *vb, int64_t stride_s, int base,
+template <typename T, int D, int G, int U, bool CHECK, typename ROWS>
+__device__ __forceinline__ void decode_tile(const T *kb, const T *vb, const ROWS &rows, int base,
                                             int rg, int s1, float scale_log2e,
                                             const Frag8<T> (&qf)[G], float (&m)[G], float (&l)[G],
                                             float (&acc)[G][8]) {
   Frag8<T> kr[U], vr[U];
-  tile_load<T, D, U, CHECK>(kb, vb, stride_s, base, rg, s1, kr, vr);
+  tile_load<T, D, U, CHECK>(kb, vb, rows, base, rg, s1, kr, vr);
   tile_update<T, D, G, U, CHECK>(kr, vr, base, rg, s1, scale_log2e, qf, m, l, acc);
 }
 
@@ -422,9 +452,10 @@ __device__ __forceinline__ void write_zero_rows(const DecodeArgs &a, int b, int 
 // writes the result itself when `direct_ok`; otherwise the range leaves a partial state and (fused
 // merge) the workgroup that finishes last combines them.  A workgroup may call this several times:
 // the caller puts a barrier between two calls, because the LDS arrays are the same.
-template <typename T, int D, int G, int U, bool QKV, bool HOIST>
+template <typename T, int D, int G, int U, bool QKV, bool HOIST, bool PAGED = false>
 __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg, int split, int n_valid,
                                               bool direct_ok, int s0, int s1) {
+  static_assert(!(QKV && PAGED), "the decode-step form reads a dense cache");
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
   int tid = threadIdx.x;
@@ -438,9 +469,30 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
 
   constexpr int SEC = FragMap<T, D>::kSecond;
   const int lane_el = dl * FragMap<T, D>::kLane;  // this lane's first element of a row
-  const int64_t kv_off = b * a.stride_b + hk * a.stride_h + lane_el;
+  // paged: the pool is [page, kv head, key in page, D], so only the head and the lane are fixed here
+  const int64_t kv_off = PAGED ? static_cast<int64_t>(hk) * (kPageKeys * D) + lane_el
+                               : b * a.stride_b + hk * a.stride_h + lane_el;
   const T *kb = static_cast<const T *>(a.k) + kv_off;
   const T *vb = static_cast<const T *>(a.v) + kv_off;
+  // the page numbers of keys [s0, s1) of this sequence, from the page table into LDS
+  __shared__ int s_pages[PAGED ? kMaxRangePages : 1];
+  const int first_page = s0 >> kPageShift;
+  if constexpr (PAGED) {
+    const int n_pages = ((s1 - 1) >> kPageShift) - first_page + 1;
+    const int32_t *tbl = a.page_table + static_cast<int64_t>(b) * a.max_pages + first_page;
+    for (int i = tid; i < n_pages; i += kThreads) s_pages[i] = tbl[i];
+    __syncthreads();
+  }
+  using Rows = typename std::conditional<PAGED, PagedRows, DenseRows>::type;
+  Rows rows;
+  if constexpr (PAGED) {
+    rows.pages = (lds_cint_ptr)s_pages;
+    rows.first_page = first_page;
+    rows.row_elems = D;
+    rows.page_stride = a.page_stride;
+  } else {
+    rows.stride_s = a.stride_s;
+  }
 
   Frag8<T> qf[G];
   // Decode-step form: the token being decoded sits at row p_new; the workgroup whose key range holds
@@ -458,7 +510,7 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
     mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
     if (mine) kv_end = p_new;
     // the first tile of cached keys is requested before q is prepared: those loads do not need it
-    if constexpr (HOIST) tile_load<T, D, U, true>(kb, vb, a.stride_s, s0, rg, kv_end, kr0, vr0);
+    if constexpr (HOIST) tile_load<T, D, U, true>(kb, vb, rows, s0, rg, kv_end, kr0, vr0);
     const int wave = tid >> 6, lane = tid & 63;
     const int B = a.B;
     const bool writer = mine && (h0 % a.group == 0);
@@ -506,9 +558,9 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
     base += U * RG;
   }
   for (; base + U * RG <= kv_end; base += U * RG)
-    decode_tile<T, D, G, U, false>(kb, vb, a.stride_s, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
+    decode_tile<T, D, G, U, false>(kb, vb, rows, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
   for (; base < kv_end; base += U * RG)
-    decode_tile<T, D, G, U, true>(kb, vb, a.stride_s, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
+    decode_tile<T, D, G, U, true>(kb, vb, rows, base, rg, kv_end, a.scale_log2e, qf, m, l, acc);
   if constexpr (QKV) {
     if (mine) {  // the new token's key and value: one more row, taken by row group 0
       Frag8<T> kn, vn;
@@ -960,8 +1012,9 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
 //       sequences they belong to: a workgroup then works through a piece of each sequence its range
 //       touches, and every slot streams the same number of keys.  A sequence without keys gets its
 //       zeros from the slot that holds its place on the line.
-template <typename T, int D, int G, int U, bool QKV, bool MFMA = false>
+template <typename T, int D, int G, int U, bool QKV, bool MFMA = false, bool PAGED = false>
 __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kernel(DecodeArgs a) {
+  static_assert(!(MFMA && PAGED), "paged caches run on the vector path");
   // the piece to work on: keys [s0, s1) of sequence b, range `split` of its n_valid ranges
   int b, hg, split, n_valid, s0, s1;
   bool direct_ok = true;
@@ -1028,8 +1081,8 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
           process_range_mfma<D, QKV>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true, max(g0 - start_b, 0),
                                 min(g1 - start_b, len_b));
         else
-          process_range<T, D, G, U, QKV, false>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
-                                                max(g0 - start_b, 0), min(g1 - start_b, len_b));
+          process_range<T, D, G, U, QKV, false, PAGED>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
+                                                       max(g0 - start_b, 0), min(g1 - start_b, len_b));
       }
       while (empty) {
         const int e = uni(__ffsll(empty) - 1);
@@ -1058,7 +1111,7 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
   if constexpr (MFMA)
     process_range_mfma<D, QKV>(a, b, hg, split, n_valid, direct_ok, s0, s1);
   else
-    process_range<T, D, G, U, QKV, true>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+    process_range<T, D, G, U, QKV, true, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1);
 }
 
 // Cross-split merge: one workgroup of D threads per (sequence, query head).
@@ -1092,7 +1145,9 @@ int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   constexpr int U = (sizeof(T) == 2 ? 8 : 4) / (G >= 4 ? 2 : 1);
   // static plan: (split, head group, sequence); length-dealt plan: one dimension, slot index slowest
   const dim3 grid(a.dynamic ? a.active * (a.Hq / G) : a.n_splits, a.dynamic ? 1 : a.Hq / G, a.dynamic ? 1 : B);
-  if (a.len_add)
+  if (a.page_table)
+    hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, false, false, true>), grid, dim3(kThreads), 0, st, a);
+  else if (a.len_add)
     hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, true>), grid, dim3(kThreads), 0, st, a);
   else
     hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, false>), grid, dim3(kThreads), 0, st, a);
@@ -1183,7 +1238,7 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
                     int D, int max_len, axhip_stream stream, bool static_ws = false) {
   const int group = Hq / Hkv;
   // four or more heads per kv head, fp16: the heads of a kv head become the columns of an MFMA tile
-  const bool mfma = g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) &&
+  const bool mfma = !a.page_table && g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) &&
                     a.stride_s % 8 == 0 && a.stride_h % 8 == 0 && a.stride_b % 8 == 0;
   const int G = mfma ? mfma_heads_per_workgroup(group) : heads_per_workgroup(group);
   a.wg_heads = G;
@@ -1305,6 +1360,37 @@ AXHIP_API int axhip_gqa_decode_static(const void *q, const void *k, const void *
                                       axhip_stream stream) {
   return gqa_decode_entry(q, k, v, seq_lens, out, nullptr, 0, dtype, B, Hq, Hkv, D, max_len, stride_b,
                           stride_h, stride_s, stream, true);
+}
+
+// Paged cache: the same kernels, plan and merge as axhip_gqa_decode; only the address of a key row differs
+// (looked up through the page table), so the result has the bits of the dense call on the same keys.
+AXHIP_API int axhip_gqa_decode_paged(const void *q, const void *k_pool, const void *v_pool, const int32_t *page_table,
+                                     const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,
+                                     int dtype, int B, int Hq, int Hkv, int D, int max_len, int max_pages, int n_pages,
+                                     axhip_stream stream) {
+  if (dtype != AXHIP_FLOAT16 && dtype != AXHIP_FLOAT32) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || Hq <= 0 || Hkv <= 0 || max_len <= 0 || max_pages <= 0 || n_pages <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (Hq % Hkv != 0) return AXHIP_SHAPE_MISMATCH;
+  if (D != 64 && D != 128 && D != 256) return AXHIP_INVALID_ARGUMENT;
+  // every key up to max_len needs a table entry; a workgroup holds the page numbers of its range in LDS
+  if (static_cast<int64_t>(max_pages) * kPageKeys < max_len || max_len > (kMaxRangePages - 1) * kPageKeys)
+    return AXHIP_INVALID_ARGUMENT;
+  if (B == 0) return AXHIP_OK;
+  if (B > 65535) return AXHIP_INVALID_ARGUMENT;
+  if (!q || !k_pool || !v_pool || !page_table || !out) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool)) & 15)
+    return AXHIP_INVALID_PTR;
+  DecodeArgs a{};
+  a.q = q;
+  a.k = k_pool;
+  a.v = v_pool;
+  a.seq_lens = seq_lens;
+  a.out = out;
+  a.page_table = page_table;
+  a.max_pages = max_pages;
+  a.page_stride = static_cast<int64_t>(Hkv) * kPageKeys * D;
+  a.stride_s = D;  // (unused by the paged addressing; kept sane for the alignment rule of the MFMA test)
+  return plan_and_launch(a, workspace, workspace_bytes, dtype, B, Hq, Hkv, D, max_len, stream);
 }
 
 AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float *k, int64_t k_stride,

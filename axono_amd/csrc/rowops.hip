@@ -563,6 +563,35 @@ __global__ __launch_bounds__(kBlock) void kv_append_kernel(const uint8_t *__rest
   st16(v_cache + dst, ld16(v_new + src));
 }
 
+// Paged form: token t of sequence b (rows [B, S, Hkv, row_bytes], token-major) goes to key position
+// start[b] + t, i.e. row (position % 128) of page page_table[b, position / 128] of pools
+// [n_pages, Hkv, 128, row_bytes].  Positions past the table and page numbers outside the pool are skipped.
+template <typename P>
+__global__ __launch_bounds__(kBlock) void kv_append_paged_kernel(const uint8_t *__restrict__ k_new,
+                                                                 const uint8_t *__restrict__ v_new,
+                                                                 uint8_t *__restrict__ k_pool, uint8_t *__restrict__ v_pool,
+                                                                 const int32_t *__restrict__ page_table,
+                                                                 const P *__restrict__ start, int B, int S, int Hkv,
+                                                                 int row_bytes, int max_pages, int n_pages) {
+  const int vec_per_row = row_bytes / 16;
+  const int64_t total = static_cast<int64_t>(B) * S * Hkv * vec_per_row;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (t >= total) return;
+  const int vi = static_cast<int>(t % vec_per_row);
+  const int64_t th = t / vec_per_row;       // (b, token, head)
+  const int hk = static_cast<int>(th % Hkv);
+  const int64_t bt = th / Hkv;
+  const int b = static_cast<int>(bt / S);
+  const int64_t p = (start ? static_cast<int64_t>(start[b]) : 0) + (bt - static_cast<int64_t>(b) * S);
+  if (p < 0 || (p >> 7) >= max_pages) return;
+  const int pid = page_table[static_cast<int64_t>(b) * max_pages + (p >> 7)];
+  if (pid < 0 || pid >= n_pages) return;
+  const int64_t src = th * row_bytes + vi * 16;
+  const int64_t dst = ((static_cast<int64_t>(pid) * Hkv + hk) * 128 + (p & 127)) * row_bytes + vi * 16;
+  st16(k_pool + dst, ld16(k_new + src));
+  st16(v_pool + dst, ld16(v_new + src));
+}
+
 // ------------------------------------------------------------------------------------------------
 // Embedding gather and argmax.
 // ------------------------------------------------------------------------------------------------
@@ -955,6 +984,31 @@ AXHIP_API int axhip_kv_append(const void *k_new, const void *v_new, void *k_cach
   else
     hipLaunchKernelGGL((kv_append_kernel<int64_t>), grid, dim3(kBlock), 0, st, kn, vn, kc, vc,
                        static_cast<const int64_t *>(pos), B, Hkv, Lmax, row_bytes);
+  return launch_status();
+}
+
+AXHIP_API int axhip_kv_append_paged(const void *k_new, const void *v_new, void *k_pool, void *v_pool,
+                                    const int32_t *page_table, const void *start, int start_dtype, int elem_bytes, int B,
+                                    int S, int Hkv, int D, int max_pages, int n_pages, axhip_stream stream) {
+  if (start && start_dtype != AXHIP_INT32 && start_dtype != AXHIP_INT64) return AXHIP_UNSUPPORTED_TYPE;
+  if (elem_bytes != 2 && elem_bytes != 4) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || S < 0 || Hkv <= 0 || D <= 0 || max_pages <= 0 || n_pages <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (B == 0 || S == 0) return AXHIP_OK;
+  if (!k_new || !v_new || !k_pool || !v_pool || !page_table) return AXHIP_INVALID_PTR;
+  const int row_bytes = D * elem_bytes;
+  if (row_bytes % 16 != 0 || !aligned16(k_new) || !aligned16(v_new) || !aligned16(k_pool) || !aligned16(v_pool))
+    return AXHIP_INVALID_ARGUMENT;
+  const int64_t total = static_cast<int64_t>(B) * S * Hkv * (row_bytes / 16);
+  const dim3 grid(blocks_for(total, kBlock));
+  hipStream_t st = as_stream(stream);
+  const uint8_t *kn = static_cast<const uint8_t *>(k_new), *vn = static_cast<const uint8_t *>(v_new);
+  uint8_t *kp = static_cast<uint8_t *>(k_pool), *vp = static_cast<uint8_t *>(v_pool);
+  if (start && start_dtype == AXHIP_INT64)
+    hipLaunchKernelGGL((kv_append_paged_kernel<int64_t>), grid, dim3(kBlock), 0, st, kn, vn, kp, vp, page_table,
+                       static_cast<const int64_t *>(start), B, S, Hkv, row_bytes, max_pages, n_pages);
+  else
+    hipLaunchKernelGGL((kv_append_paged_kernel<int32_t>), grid, dim3(kBlock), 0, st, kn, vn, kp, vp, page_table,
+                       static_cast<const int32_t *>(start), B, S, Hkv, row_bytes, max_pages, n_pages);
   return launch_status();
 }
 

@@ -123,6 +123,70 @@ def gqa_decode_attention_cache(q: Tensor, k_cache: Tensor, v_cache: Tensor, seq_
     return out
 
 
+PAGE_KEYS = 128  # keys per page of a paged KV cache (AXHIP_PAGE_KEYS)
+
+
+def gqa_decode_attention_paged(q: Tensor, k_pool: Tensor, v_pool: Tensor, page_table: Tensor, seq_lens: Tensor | None,
+                               max_len: int, out: Tensor | None = None, workspace: Tensor | None = None) -> Tensor:
+    """Decode attention over a paged cache: q (B,Hq,D), pools (n_pages,Hkv,128,D), page_table INT32
+    (B,max_pages), seq_lens INT32 (B,), both on the device; max_len bounds every length.  Same result, bit
+    for bit, as gqa_decode_attention_cache on a dense cache holding the same keys."""
+    op = "gqa_decode_attention_paged"
+    _need_hip(op, q, k_pool, v_pool, page_table, seq_lens)
+    if q.ndim != 3 or k_pool.ndim != 4 or q.dtype not in _FLOATS or k_pool.dtype != q.dtype or v_pool.dtype != q.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    B, hq, d = q.shape
+    n_pages, hkv, pk, dk = k_pool.shape
+    if pk != PAGE_KEYS or dk != d or v_pool.shape != k_pool.shape or hkv == 0 or hq % hkv != 0:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if page_table.dtype != DataType.INT32 or page_table.ndim != 2 or page_table.shape[0] != B:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if seq_lens is not None and (seq_lens.dtype != DataType.INT32 or seq_lens.num_elements != B):
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    max_pages = page_table.shape[1]
+    max_len = int(max_len)
+    if out is None:
+        out = _new(q.dtype, [B, hq, d], q)
+    lib = _lib_()
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, hq, hkv, d, max(max_len, 1))
+    ws = workspace if workspace is not None else _workspace(wsb, q)
+    check(lib.axhip_gqa_decode_paged(q.data_ptr, k_pool.data_ptr, v_pool.data_ptr, page_table.data_ptr,
+                                     seq_lens.data_ptr if seq_lens is not None else None, out.data_ptr, ws.data_ptr,
+                                     ws.num_bytes, int(q.dtype), B, hq, hkv, d, max_len, max_pages, n_pages,
+                                     current_stream()), op)
+    return out
+
+
+def kv_append_paged(k_new: Tensor, v_new: Tensor, k_pool: Tensor, v_pool: Tensor, page_table: Tensor,
+                    start: Tensor | None, tokens_per_sequence: int = 1, table_row: int | None = None) -> None:
+    """In place: token t of sequence b (rows [B, S, Hkv, D], S = tokens_per_sequence) is written at key
+    position start[b] + t of the paged cache.  table_row: treat the rows as ONE sequence, the one of that
+    row of the page table (start is then that sequence's entry of a per-sequence tensor)."""
+    op = "kv_append_paged"
+    _need_hip(op, k_new, v_new, k_pool, v_pool, page_table, start)
+    if k_pool.ndim != 4 or k_new.dtype != k_pool.dtype or v_new.dtype != v_pool.dtype or k_pool.dtype != v_pool.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    n_pages, hkv, pk, d = k_pool.shape
+    B, max_pages = page_table.shape
+    S = int(tokens_per_sequence)
+    tbl, st_ptr = page_table.data_ptr, (start.data_ptr if start is not None else None)
+    if table_row is not None:
+        if not 0 <= table_row < B:
+            raise AxhipError(op, Status.INVALID_ARGUMENT)
+        tbl += table_row * max_pages * 4
+        if start is not None:
+            st_ptr += table_row * (4 if start.dtype == DataType.INT32 else 8)
+        B = 1
+    if pk != PAGE_KEYS or v_pool.shape != k_pool.shape or k_new.num_elements != B * S * hkv * d or v_new.num_elements != k_new.num_elements:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if start is not None and start.dtype not in (DataType.INT32, DataType.INT64):
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    check(_lib_().axhip_kv_append_paged(k_new.data_ptr, v_new.data_ptr, k_pool.data_ptr, v_pool.data_ptr, tbl, st_ptr,
+                                        int(start.dtype) if start is not None else int(DataType.INT32),
+                                        k_pool.num_bytes // max(k_pool.num_elements, 1), B, S, hkv, d, max_pages, n_pages,
+                                        current_stream()), op)
+
+
 def scaled_dot_product_attention(q: Tensor, k: Tensor, v: Tensor, is_causal: bool = False) -> Tensor:
     """q (Sq,Hq,D), k/v (Skv,Hkv,D).  nanobind_module.cpp:1107-1135."""
     op = "scaled_dot_product_attention"

@@ -2,6 +2,7 @@
 
 `KVCache` is the abstract interface; `DynamicKVCache` is the default component (per layer, the
 full k / v tensors, layout (seq, n_kv_head, d_head), grown along axis 0 by byte copies).
+`PagedKVCache` grows by pages of 128 keys through a page table (memory follows the tokens that exist).
 `StaticKVCache` is this build's cache for the captured decode step: one pre-allocated
 [B, n_kv_head, max_len, d_head] tensor pair per layer, device-resident lengths, and an append that
 writes one row per (sequence, head) instead of re-copying the cache.
@@ -172,3 +173,125 @@ class StaticKVCache(KVCache):
     def __len__(self) -> int:
         """Host-side view of the longest sequence (kept in step with advance/set_lengths)."""
         return self._host_len
+
+
+class PagedKVCache(KVCache):
+    """KV cache of a batch of sequences that grows by pages of 128 keys instead of being allocated for
+    batch x max_len rows up front.
+
+    Per layer two pools [n_pages, n_kv_head, 128, d_head]; ONE page table INT32 [batch, max_pages] shared by
+    all layers (page p of a sequence has the same page number in every layer's pool) and the lengths INT32
+    [batch], both on the device (the attention kernel reads them) with host mirrors for the allocator.  Pages
+    come from a free list; `free_sequence` returns a finished sequence's pages, so memory follows the tokens
+    that exist.  `update` (one new token per sequence) and `update_rows` (many tokens of one sequence: its
+    prefill) write through the page table; `attend` is decode attention over the pages, bit-identical to the
+    dense cache's.  The lengths advance once per step, after the last layer (`advance`), as in
+    StaticKVCache.  Page allocation uploads the page table, so inside a captured step call
+    `reserve(tokens)` before capturing."""
+
+    PAGE = _l.PAGE_KEYS
+
+    def __init__(self, n_layers: int, batch: int, n_kv_head: int, d_head: int, n_pages: int, max_len: int,
+                 dtype: DataType = DataType.FLOAT16, device: str = "hip", page_order=None):
+        self.n_layers, self.batch, self.n_kv_head, self.d_head = int(n_layers), int(batch), int(n_kv_head), int(d_head)
+        self.n_pages, self.max_len = int(n_pages), int(max_len)
+        self.max_pages = (self.max_len + self.PAGE - 1) // self.PAGE
+        self.dtype, self.device = DataType(dtype), device
+        shape = [self.n_pages, self.n_kv_head, self.PAGE, self.d_head]
+        self._k = [Tensor(dtype, shape, device) for _ in range(self.n_layers)]
+        self._v = [Tensor(dtype, shape, device) for _ in range(self.n_layers)]
+        self.page_table = Tensor(DataType.INT32, [self.batch, self.max_pages], device)
+        self.seq_lens = Tensor(DataType.INT32, [self.batch], device)
+        # page_order: the order in which physical pages are handed out (default 0, 1, 2, ...)
+        order = list(range(self.n_pages)) if page_order is None else [int(p) for p in page_order]
+        if sorted(order) != list(range(self.n_pages)):
+            raise ValueError("page_order must be a permutation of range(n_pages)")
+        self._order = order
+        self.reset()
+
+    # ---- page allocator (host) -----------------------------------------------------------------
+    def reset(self) -> None:
+        self._free = list(reversed(self._order))        # pop() hands out self._order[0] first
+        self._table = np.full((self.batch, self.max_pages), -1, np.int32)
+        self._lens = np.zeros(self.batch, np.int64)
+        self._owned = np.zeros(self.batch, np.int64)     # pages each sequence holds
+        self.page_table.copy_from_numpy(self._table)
+        self.seq_lens.fill_zero()
+
+    @property
+    def pages_in_use(self) -> int:
+        return self.n_pages - len(self._free)
+
+    def reserve(self, new_tokens=1) -> None:
+        """Makes sure every sequence has pages for its length + new_tokens (an int, or one int per
+        sequence).  Raises MemoryError when the pool runs out (nothing is changed then)."""
+        want = self._lens + np.broadcast_to(np.asarray(new_tokens, np.int64), (self.batch,))
+        if np.any(want > self.max_len):
+            raise ValueError(f"PagedKVCache: a sequence would exceed max_len = {self.max_len}")
+        need = (want + self.PAGE - 1) // self.PAGE - self._owned
+        need = np.maximum(need, 0)
+        if int(need.sum()) == 0:
+            return
+        if int(need.sum()) > len(self._free):
+            raise MemoryError(f"PagedKVCache: {int(need.sum())} pages needed, {len(self._free)} free of {self.n_pages}")
+        for b in np.nonzero(need)[0]:
+            for _ in range(int(need[b])):
+                self._table[b, self._owned[b]] = self._free.pop()
+                self._owned[b] += 1
+        self.page_table.copy_from_numpy(self._table)
+
+    def free_sequence(self, b: int) -> None:
+        """Returns sequence b's pages to the free list and empties it."""
+        n = int(self._owned[b])
+        self._free.extend(int(p) for p in self._table[b, :n][::-1])
+        self._table[b, :n] = -1
+        self._owned[b] = 0
+        self._lens[b] = 0
+        self.page_table.copy_from_numpy(self._table)
+        self.seq_lens.copy_from_numpy(self._lens.astype(np.int32))
+
+    # ---- KVCache interface ---------------------------------------------------------------------
+    def update(self, layer_idx: int, k_new, v_new) -> None:
+        """One new token per sequence: k_new / v_new [batch, n_kv_head, d_head], written at each
+        sequence's current length."""
+        self.reserve(1)
+        _l.kv_append_paged(k_new, v_new, self._k[layer_idx], self._v[layer_idx], self.page_table, self.seq_lens)
+
+    def update_rows(self, layer_idx: int, b: int, k_rows, v_rows) -> None:
+        """Many tokens of ONE sequence (its prefill): k_rows / v_rows [tokens, n_kv_head, d_head] - the
+        reference cache's own layout - written from sequence b's current length on."""
+        n = int(k_rows.shape[0])
+        grow = np.zeros(self.batch, np.int64)
+        grow[b] = n
+        self.reserve(grow)
+        _l.kv_append_paged(k_rows, v_rows, self._k[layer_idx], self._v[layer_idx], self.page_table, self.seq_lens,
+                           tokens_per_sequence=n, table_row=b)
+
+    def advance(self, n: int = 1) -> None:
+        """Every sequence grew by n tokens (call once per step, after the last layer's update)."""
+        self.reserve(max(int(n), 0))
+        _l.index_add(self.seq_lens, n)
+        self._lens += n
+
+    def advance_rows(self, b: int, n: int) -> None:
+        self._lens[b] += n
+        self.seq_lens.copy_from_numpy(self._lens.astype(np.int32))
+
+    def get(self, layer_idx: int):
+        """(k_pool, v_pool) of the layer; together with `page_table` and `seq_lens` they are what
+        gqa_decode_attention_paged takes."""
+        return self._k[layer_idx], self._v[layer_idx]
+
+    def attend(self, layer_idx: int, q, extra_tokens: int = 0):
+        """Decode attention of q [batch, n_q_head, d_head] over the layer's cached keys (+ extra_tokens
+        rows already written by `update` in this step but not yet counted by `advance`)."""
+        lens = self.seq_lens
+        if extra_tokens:
+            lens = Tensor(DataType.INT32, [self.batch], self.device, _zero=False)
+            lens.copy_from_numpy((self._lens + extra_tokens).astype(np.int32))
+        bound = int(self._lens.max()) + int(extra_tokens)
+        return _l.gqa_decode_attention_paged(q, self._k[layer_idx], self._v[layer_idx], self.page_table, lens,
+                                             max(bound, 1))
+
+    def __len__(self) -> int:
+        return int(self._lens.max()) if self.batch else 0

@@ -199,6 +199,24 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
                                int max_len, int64_t stride_b, int64_t stride_h, int64_t stride_s,
                                axhip_stream stream);
 
+/* axhip_gqa_decode over a paged KV cache.  Keys and values live in pools
+ *   k_pool, v_pool  [n_pages, Hkv, 128, D]   (pages of AXHIP_PAGE_KEYS = 128 consecutive keys of one sequence)
+ * and key s of sequence b is row s % 128 of page  page_table[b * max_pages + s / 128]  (device int32
+ * [B, max_pages]; entries behind a sequence's last page are never read).  Everything else - q, out, seq_lens,
+ * max_len, workspace, the split plan, the in-kernel merge - is as in axhip_gqa_decode, and so is the
+ * result, bit for bit, for the same keys in the same order: only the address of a key row differs (each
+ * workgroup copies the page numbers of its key range from the table into LDS before its first tile).
+ * max_pages * 128 >= max_len; max_len <= 131072; head groups of four and more query heads run on the vector
+ * ALUs here (the matrix-core variant reads a dense cache).  A cache that grows by pages allocates
+ * memory for the tokens that exist instead of B * Lmax rows; the reference's cache grows by re-copying
+ * (axono/python/axono/nn/kv_cache.py:96-102) and has no paged form. */
+#define AXHIP_PAGE_KEYS 128
+AXHIP_API int axhip_gqa_decode_paged(const void *q, const void *k_pool, const void *v_pool,
+                                     const int32_t *page_table, const int32_t *seq_lens, void *out,
+                                     void *workspace, size_t workspace_bytes, int dtype, int B, int Hq,
+                                     int Hkv, int D, int max_len, int max_pages, int n_pages,
+                                     axhip_stream stream);
+
 /* axhip_gqa_decode for callers that cannot allocate (code under hipGraph capture, tight serving loops,
  * harnesses that forbid hipMalloc) and therefore have no workspace to pass: the split partials go to a
  * static device array inside the library, AXHIP_GQA_DECODE_STATIC_SCRATCH_BYTES per device, held until
@@ -254,6 +272,17 @@ AXHIP_API int axhip_sdpa(const void *q, const void *k, const void *v, void *out,
 AXHIP_API int axhip_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache,
                               const void *pos, int pos_dtype, int elem_bytes, int B, int Hkv,
                               int Lmax, int D, axhip_stream stream);
+
+/* KV append into a paged cache (pools and page table as for axhip_gqa_decode_paged): token t of sequence
+ * b, rows k_new / v_new [B, S, Hkv, D] (token-major: the (seq, n_kv_head, d_head) layout of the
+ * reference's cache with a batch axis in front), goes to key position start[b] + t (start: device int32 or
+ * int64 [B], or NULL for 0).  A byte copy (bit exact).  Positions behind the table and page numbers
+ * outside [0, n_pages) are skipped.  Counterpart of DynamicKVCache.update
+ * (axono/python/axono/nn/kv_cache.py:96-102). */
+AXHIP_API int axhip_kv_append_paged(const void *k_new, const void *v_new, void *k_pool, void *v_pool,
+                                    const int32_t *page_table, const void *start, int start_dtype,
+                                    int elem_bytes, int B, int S, int Hkv, int D, int max_pages,
+                                    int n_pages, axhip_stream stream);
 
 /* out = [a ; b] along an axis: `outer` blocks of a_bytes then b_bytes each (axis 0: outer = 1).
  * Replaces ops::cuda::Concat, src/ops/cuda/sequence.cu:474-521. */

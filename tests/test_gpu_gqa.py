@@ -548,3 +548,133 @@ def test_prefill_attention_random_configurations(seed):
     S = int(rng.choice([1, 17, 64, 100, 200, 333]))
     start = [int(s) for s in rng.choice([0, 1, 63, 64, 150], int(rng.integers(1, 4)))]
     test_prefill_attention_matches_causal_oracle(hkv * group, hkv, d, S, start)
+
+
+# ---- paged KV cache ------------------------------------------------------------------------------
+def _paged_from_dense(k, v, lens, perm_seed, extra_pages=3):
+    """Scatters a dense cache [B,Hkv,Lmax,D] into pools [n_pages,Hkv,128,D] through a random page table."""
+    B, Hkv, Lmax, D = k.shape
+    P = 128
+    max_pages = -(-Lmax // P)
+    need = [-(-int(n) // P) for n in lens]
+    n_pages = sum(need) + extra_pages
+    rng = np.random.default_rng(perm_seed)
+    order = rng.permutation(n_pages)
+    table = np.full((B, max_pages), -1, np.int32)
+    kp = rng.standard_normal((n_pages, Hkv, P, D)).astype(k.dtype)   # unused rows hold noise, not zeros
+    vp = rng.standard_normal((n_pages, Hkv, P, D)).astype(k.dtype)
+    nxt = 0
+    for b in range(B):
+        for p in range(need[b]):
+            pid = int(order[nxt]); nxt += 1
+            table[b, p] = pid
+            rows = min(P, Lmax - p * P)
+            kp[pid, :, :rows] = k[b, :, p * P:p * P + rows]
+            vp[pid, :, :rows] = v[b, :, p * P:p * P + rows]
+    return kp, vp, table, n_pages, max_pages
+
+
+def _gqa_paged(q, kp, vp, table, lens, max_len):
+    l = lib()
+    B, Hq, D = q.shape
+    n_pages, Hkv = kp.shape[:2]
+    dq, dk, dv, dt_, dl = (gu.dev(a) for a in (q, kp, vp, table, np.asarray(lens, np.int32)))
+    out = gu.DeviceBuffer(q.nbytes)
+    wsb = l.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, max_len)
+    ws = gu.DeviceBuffer(max(wsb, 256))
+    gu.check(l.axhip_gqa_decode_paged(dq.ptr, dk.ptr, dv.ptr, dt_.ptr, dl.ptr, out.ptr, ws.ptr, wsb, gu.dt(q), B, Hq, Hkv,
+                                      D, max_len, table.shape[1], n_pages, None), "gqa_decode_paged")
+    gu.synchronize()
+    return out.download(q.dtype, q.shape)
+
+
+@pytest.mark.parametrize("dtype,hq,hkv,d", [(np.float16, 16, 8, 128), (np.float32, 16, 8, 128), (np.float16, 8, 8, 64),
+                                             (np.float16, 16, 4, 128), (np.float32, 4, 2, 256)])
+def test_paged_cache_has_the_bits_of_the_dense_cache(dtype, hq, hkv, d):
+    """Pages handed out in a random order: the result equals the dense kernel's on the same keys bit for
+    bit (same plan, same summation order) and the oracle's within tolerance.  Ragged lengths incl. empty,
+    one key, a page boundary, one past it; default plan, a forced split count (static plan) and the
+    two-kernel merge."""
+    rng = np.random.default_rng(hq * 13 + d)
+    lens = np.array([3000, 0, 1, 128, 129, 2047, 777], np.int32)
+    B, Lmax = len(lens), 3000
+    q = rng.standard_normal((B, hq, d)).astype(np.float32).astype(dtype)
+    k = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(dtype)
+    v = rng.standard_normal((B, hkv, Lmax, d)).astype(np.float32).astype(dtype)
+    kp, vp, table, n_pages, max_pages = _paged_from_dense(k, v, lens, 5)
+    want = port.gqa_decode_cache_native(q, k, v, lens)
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    tol = TOL16 if dtype == np.float16 else TOL32
+    l = lib()
+    try:
+        for tune in ((0, 0), (0, 3), (-1, 3), (0, 1)):
+            l.axhip_gqa_decode_tune(*tune)
+            if hq // hkv >= 4:
+                l.axhip_gqa_decode_tune(tune[0], tune[1] + 1000)   # dense on the vector path too: same arithmetic
+            dense = gqa_decode(q, k, v, lens)
+            paged = _gqa_paged(q, kp, vp, table, lens, Lmax)
+            np.testing.assert_array_equal(paged.view(bits), dense.view(bits), err_msg=str(tune))
+            assert np.abs(paged.astype(np.float32) - want).max() <= tol, tune
+            assert np.all(paged[1] == 0)
+    finally:
+        l.axhip_gqa_decode_tune(0, 0)
+
+
+def test_paged_cache_headline_shape_random_pages():
+    """B=32, L=8192 fp16 through a random page permutation (2048 pages of 32 KB per kv head): equal to the
+    dense kernel bit for bit; sequence 0 against the oracle."""
+    rng = np.random.default_rng(808)
+    B, Hq, Hkv, D, L = 32, 16, 8, 128, 8192
+    lens = np.full(B, L, np.int32)
+    q = rng.standard_normal((B, Hq, D)).astype(np.float32).astype(np.float16)
+    blk = rng.standard_normal((4, Hkv, L, D)).astype(np.float32).astype(np.float16)
+    k = np.concatenate([np.roll(blk, s, axis=2) for s in range(0, 8)], 0)       # 32 distinct sequences from 4 blocks
+    v = np.concatenate([np.roll(blk, 64 + s, axis=3) for s in range(0, 8)], 0)
+    kp, vp, table, n_pages, _ = _paged_from_dense(k, v, lens, 9, extra_pages=7)
+    dense = gqa_decode(q, k, v, lens)
+    paged = _gqa_paged(q, kp, vp, table, lens, L)
+    np.testing.assert_array_equal(paged.view(np.uint16), dense.view(np.uint16))
+    want0 = port.gqa_decode_cache_native(q[:1], k[:1], v[:1])
+    assert np.abs(paged[:1].astype(np.float32) - want0).max() <= TOL16
+
+
+def test_paged_append_is_a_byte_copy_through_the_table():
+    rng = np.random.default_rng(77)
+    B, S, Hkv, D, P = 3, 5, 2, 64, 128
+    n_pages, max_pages = 9, 3
+    table = np.array([[4, 0, -1], [7, 2, 8], [1, -1, -1]], np.int32)
+    start = np.array([126, 250, 0], np.int32)            # crosses a page boundary; crosses two; stays inside
+    kn = rng.integers(0, 65536, (B, S, Hkv, D)).astype(np.uint16).view(np.float16)
+    vn = rng.integers(0, 65536, (B, S, Hkv, D)).astype(np.uint16).view(np.float16)
+    kp0 = rng.integers(0, 65536, (n_pages, Hkv, P, D)).astype(np.uint16)
+    vp0 = rng.integers(0, 65536, (n_pages, Hkv, P, D)).astype(np.uint16)
+    dk, dv, dkn, dvn, dtb, dst = (gu.dev(a) for a in (kp0, vp0, kn, vn, table, start))
+    gu._run("axhip_kv_append_paged", dkn.ptr, dvn.ptr, dk.ptr, dv.ptr, dtb.ptr, dst.ptr, gu.I32, 2, B, S, Hkv, D,
+            max_pages, n_pages, None)
+    gu.synchronize()
+    wk, wv = kp0.copy(), vp0.copy()
+    for b in range(B):
+        for t in range(S):
+            pos = start[b] + t
+            pid = table[b, pos // P]
+            wk[pid, :, pos % P] = kn[b, t].view(np.uint16)
+            wv[pid, :, pos % P] = vn[b, t].view(np.uint16)
+    np.testing.assert_array_equal(dk.download(np.uint16, kp0.shape), wk)
+    np.testing.assert_array_equal(dv.download(np.uint16, vp0.shape), wv)
+    # a position behind the table and a page number outside the pool are skipped, nothing else is touched
+    bad_table = np.array([[4, 0, 99], [7, 2, 8], [1, -1, -1]], np.int32)
+    dtb2, dst2 = gu.dev(bad_table), gu.dev(np.array([254, 382, 126], np.int32))
+    gu._run("axhip_kv_append_paged", dkn.ptr, dvn.ptr, dk.ptr, dv.ptr, dtb2.ptr, dst2.ptr, gu.I32, 2, B, S, Hkv, D,
+            max_pages, n_pages, None)
+    gu.synchronize()
+    got = dk.download(np.uint16, kp0.shape)
+    for t in range(2):                                   # sequence 0: positions 254, 255 land in page 0; 256.. hit page 99
+        wk[0, :, 126 + t] = kn[0, t].view(np.uint16)
+    for t in range(2):                                   # sequence 1: positions 382, 383 in page 8; 384.. are behind the table
+        wk[8, :, 126 + t] = kn[1, t].view(np.uint16)
+    for t in range(2):                                   # sequence 2: positions 126, 127 in page 1; 128.. have page -1
+        wk[1, :, 126 + t] = kn[2, t].view(np.uint16)
+    np.testing.assert_array_equal(got, wk)
+    l = lib()
+    assert l.axhip_gqa_decode_paged(None, None, None, None, None, None, None, 0, 4, 1, 16, 8, 128, 300, 2, 4, None) == 1  # table too short
+    assert l.axhip_gqa_decode_paged(None, None, None, None, None, None, None, 0, 4, 1, 16, 8, 128, 256, 2, 4, None) == 7

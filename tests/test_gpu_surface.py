@@ -505,3 +505,55 @@ def test_axm_weights_go_straight_to_the_device(tmp_path):
     assert set(dev16) == {"w", "ids"}
     np.testing.assert_array_equal(dev16["w"].numpy(), sd["w"].astype(np.float16))
     np.testing.assert_array_equal(dev16["ids"].numpy(), sd["ids"])
+
+
+def test_paged_kv_cache_component():
+    """nn.PagedKVCache: prefill rows per sequence, one-token updates, attention through the page table
+    equal to the static cache's bit for bit, page accounting, freeing a sequence, running out of pages."""
+    rng = np.random.default_rng(41)
+    B, hq, hkv, d, lmax = 3, 4, 2, 64, 512
+    order = rng.permutation(10)
+    pg = nn.PagedKVCache(2, B, hkv, d, n_pages=10, max_len=lmax, dtype=DataType.FLOAT16, device=DEV, page_order=order)
+    st = nn.StaticKVCache(2, B, hkv, lmax, d, DataType.FLOAT16, DEV)
+    assert len(pg) == 0 and pg.pages_in_use == 0
+    prompt = [130, 5, 256]
+    for layer in range(2):
+        for b, n in enumerate(prompt):
+            kr = rng.standard_normal((n, hkv, d)).astype(np.float16)
+            vr = rng.standard_normal((n, hkv, d)).astype(np.float16)
+            pg.update_rows(layer, b, t(kr), t(vr))
+            # the static cache row by row (its layout is [B, hkv, L, d])
+            kc, vc = st.get(layer)
+            kh, vh = kc.numpy(), vc.numpy()
+            kh[b, :, :n], vh[b, :, :n] = np.transpose(kr, (1, 0, 2)), np.transpose(vr, (1, 0, 2))
+            kc.copy_from_numpy(kh)
+            vc.copy_from_numpy(vh)
+    for b, n in enumerate(prompt):
+        pg.advance_rows(b, n)
+    st.set_lengths(prompt)
+    assert pg.pages_in_use == 2 + 1 + 2 and len(pg) == 256
+    np.testing.assert_array_equal(pg.seq_lens.to_numpy(), prompt)
+    for step in range(3):
+        q = rng.standard_normal((B, hq, d)).astype(np.float16)
+        for layer in range(2):
+            kn = rng.standard_normal((B, hkv, d)).astype(np.float16)
+            vn = rng.standard_normal((B, hkv, d)).astype(np.float16)
+            pg.update(layer, t(kn), t(vn))
+            st.update(layer, t(kn), t(vn))
+            got = pg.attend(layer, t(q), extra_tokens=1).numpy()
+            lens1 = Tensor(DataType.INT32, [B], DEV)
+            lens1.copy_from_numpy((np.array(prompt) + step + 1).astype(np.int32))
+            want = axono.gqa_decode_attention_cache(t(q), *st.get(layer), lens1, max_len=int(max(prompt)) + step + 1).numpy()
+            np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+        pg.advance()
+        st.advance()
+    assert pg.pages_in_use == 2 + 1 + 3                  # sequence 2 crossed into its third page at 257 tokens
+    pg.free_sequence(0)
+    assert pg.pages_in_use == 4 and int(pg.seq_lens.to_numpy()[0]) == 0
+    with pytest.raises(MemoryError):
+        pg.reserve([512, 0, 0])                          # 4 pages for sequence 0, then 512 more tokens for it: 6 free
+        pg.reserve([0, 512 - 8, 512 - 259])
+    with pytest.raises(ValueError):
+        pg.reserve([0, 0, 300])                          # past max_len
+    pg.reset()
+    assert pg.pages_in_use == 0 and len(pg) == 0

@@ -111,7 +111,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
 
 
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
-        cpu_step_hook=None, cfg: TextConfig | None = None) -> dict:
+        cpu_step_hook=None, cfg: TextConfig | None = None, kernel_table: bool = True) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
     after the prefill with the model positioned at the first decode step (the benchmark passes a
     hook that times and compares a CPU restatement of one step); its dict is merged into the result."""
@@ -162,7 +162,7 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     assert toks.shape == (decode_steps, batch) and toks.min() >= 0 and toks.max() < cfg.vocab_size
     log(f"[decode] {decode_steps} replays: {ms_step:.3f} ms/step, {tok_s:.0f} tok/s "
         f"({100 * tok_s / ceiling:.1f}% of the {ceiling:.0f} tok/s HBM ceiling)")
-    table = per_kernel_table(model, context + decode_steps)
+    table = per_kernel_table(model, context + decode_steps) if kernel_table else []
     in_kernels = sum(r["us_per_step"] for r in table)
     for r in table:
         log(f"[decode]   {r['kernel']:<68s} {r['calls_per_step']:3d} x {r['us_per_call']:7.2f} us = {r['us_per_step']:7.1f} us"
@@ -192,11 +192,14 @@ def main(argv=None):
     ap.add_argument("--gqa-two-kernels", type=int, default=0, metavar="SPLITS",
                     help="attention with a fixed split count and a second merge kernel (the default deals "
                          "workgroups by length and merges in the last workgroup)")
+    ap.add_argument("--no-kernel-table", action="store_true",
+                    help="skip the per-kernel table (its extra launches would mix into a profiler's kernel statistics)")
     args = ap.parse_args(argv)
     if args.gqa_two_kernels:
         from .. import _lib
         _lib.load().axhip_gqa_decode_tune(-1, args.gqa_two_kernels)
-    res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True))
+    res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
+              kernel_table=not args.no_kernel_table)
     print(json.dumps(res), flush=True)
 
 

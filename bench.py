@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the headline split kernel, from the rocprofv3 --pmc runs recorded in
 # profiles/gqa_decode_split_B32_L8192_f16.md (a measured constant, not computed in this process)
-MEASURED_TRAFFIC_BYTES = 1074176614
+MEASURED_TRAFFIC_BYTES = 1074196367
 
 F16 = 4
 

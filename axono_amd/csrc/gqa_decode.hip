@@ -246,7 +246,7 @@ struct DecodeArgs {
   // Paged cache (template parameter PAGED): a.k / a.v are pools [n_pages, Hkv, kPageKeys, D]; key s of
   // sequence b is row s % kPageKeys of page page_table[b * max_pages + s / kPageKeys].
   const int32_t *page_table;
-  int max_pages;
+  int max_pages, n_pages;
   int64_t page_stride;  // elements per page: Hkv * kPageKeys * D
 };
 
@@ -478,9 +478,10 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   __shared__ int s_pages[PAGED ? kMaxRangePages : 1];
   const int first_page = s0 >> kPageShift;
   if constexpr (PAGED) {
-    const int n_pages = ((s1 - 1) >> kPageShift) - first_page + 1;
+    const int range_pages = ((s1 - 1) >> kPageShift) - first_page + 1;
     const int32_t *tbl = a.page_table + static_cast<int64_t>(b) * a.max_pages + first_page;
-    for (int i = tid; i < n_pages; i += kThreads) s_pages[i] = tbl[i];
+    // page numbers are clamped into the pool: a corrupt table gives wrong values, never an access outside it
+    for (int i = tid; i < range_pages; i += kThreads) s_pages[i] = min(max(tbl[i], 0), a.n_pages - 1);
     __syncthreads();
   }
   using Rows = typename std::conditional<PAGED, PagedRows, DenseRows>::type;
@@ -1388,6 +1389,7 @@ AXHIP_API int axhip_gqa_decode_paged(const void *q, const void *k_pool, const vo
   a.out = out;
   a.page_table = page_table;
   a.max_pages = max_pages;
+  a.n_pages = n_pages;
   a.page_stride = static_cast<int64_t>(Hkv) * kPageKeys * D;
   a.stride_s = D;  // (unused by the paged addressing; kept sane for the alignment rule of the MFMA test)
   return plan_and_launch(a, workspace, workspace_bytes, dtype, B, Hq, Hkv, D, max_len, stream);

@@ -282,16 +282,25 @@ class PagedKVCache(KVCache):
         gqa_decode_attention_paged takes."""
         return self._k[layer_idx], self._v[layer_idx]
 
-    def attend(self, layer_idx: int, q, extra_tokens: int = 0):
+    def attend(self, layer_idx: int, q, extra_tokens: int = 0, max_len: int | None = None):
         """Decode attention of q [batch, n_q_head, d_head] over the layer's cached keys (+ extra_tokens
-        rows already written by `update` in this step but not yet counted by `advance`)."""
+        rows already written by `update` in this step but not yet counted by `advance`).  Everything
+        runs on the device, so the call can be captured; a captured step passes `max_len`, the longest
+        sequence any replay will see (the split plan is made from it), and reserves the pages for those
+        tokens before capturing."""
         lens = self.seq_lens
         if extra_tokens:
             lens = Tensor(DataType.INT32, [self.batch], self.device, _zero=False)
-            lens.copy_from_numpy((self._lens + extra_tokens).astype(np.int32))
-        bound = int(self._lens.max()) + int(extra_tokens)
+            _l.copy_bytes(lens, 0, self.seq_lens, 0, 4 * self.batch)
+            _l.index_add(lens, int(extra_tokens))
+        bound = int(max_len) if max_len is not None else int(self._lens.max()) + int(extra_tokens)
         return _l.gqa_decode_attention_paged(q, self._k[layer_idx], self._v[layer_idx], self.page_table, lens,
-                                             max(bound, 1))
+                                             max(min(bound, self.max_len), 1))
+
+    def sync_from_device(self) -> None:
+        """Refreshes the host mirror of the lengths from the device tensor (after replays of a captured
+        step, whose `advance` ran on the device only)."""
+        self._lens = self.seq_lens.to_numpy().astype(np.int64)
 
     def __len__(self) -> int:
         return int(self._lens.max()) if self.batch else 0

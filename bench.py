@@ -6,7 +6,8 @@
 Prints ONE JSON line.  The metric is BASELINE.json's: "GQA decode HBM GB/s (% of peak) B=32 L=8k
 fp16; decode tok/s 2B-shape B=16".  `value` is the first half: achieved algorithmic GB/s of the
 split-K GQA decode attention at B=32, Hq=16, Hkv=8, D=128, L=8192, fp16 KV cache resident in HBM.
-A "step" is one pass of that operator over one batch (split kernel + merge kernel).  The second half
+A "step" is one pass of that operator over one batch (one launch: at this shape every sequence is one key
+range of one workgroup, so nothing is merged).  The second half
 (tokens/s of the Qwen3-VL-2B-shaped text decode step, B=16, 128 hipGraph replays) is reported in
 `decode_step` on the same line.
 
@@ -318,6 +319,11 @@ def config_tables(lib, with_cpu=True):
             rec["cpu_us_one_sequence"] = cpu_seq_us[L]
         c3.append(rec)
     out["config3_gqa_decode_sweep"] = c3
+    # the headline shape through a paged cache whose pages were handed out in a random order (and the dense cache
+    # of the same buffers beside it)
+    out["config3_paged_cache_random_pages"] = [
+        {"form": r["op"], "B": r["B"], "L": r["L"], "pages": r["pages"], "us": r["us"], "bytes": r["bytes"], "GBps": r["GBps"],
+         "frac_hbm": round(r["GBps"] / HBM_PEAK_GBS, 4)} for r in mb.collect(mb.bench_gqa_paged, lib, 32, 8192, 100)]
 
     # ---- config 4: the fp16 Linear ---------------------------------------------------------------------
     c4 = []
@@ -418,9 +424,9 @@ def main():
                    "B": 32, "Hq": 16, "Hkv": 8, "D": 128, "L": 8192, "plan": wl.plan(),
                    "kv_buffers_rotated": len(wl.kv)},
         "pct_of_hbm_peak": round(100 * gbs_wall / HBM_PEAK_GBS, 2),
-        # achieved = algorithmic bytes per step / HIP-event time per step (split kernel + the 5 us merge
-        # kernel); traffic = HBM bytes per launch of the split kernel from rocprofv3 counters
-        # (FETCH_SIZE x 2.0000 + WRITE_SIZE x 1.0000, factors from a 1 GiB copy kernel), see profiles/
+        # achieved = algorithmic bytes per step / HIP-event time per step (one launch of the split kernel);
+        # traffic = HBM bytes per launch of that kernel from rocprofv3 counters (FETCH_SIZE x 2.0000 +
+        # WRITE_SIZE x 1.0000, factors from a 1 GiB copy kernel), see profiles/
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "gqa_decode_split_kernel<__half,128,2,8> (one range per sequence at this shape: no merge)",

@@ -202,7 +202,8 @@ AXHIP_API int axhip_gqa_decode(const void *q, const void *k, const void *v,
 /* axhip_gqa_decode over a paged KV cache.  Keys and values live in pools
  *   k_pool, v_pool  [n_pages, Hkv, 128, D]   (pages of AXHIP_PAGE_KEYS = 128 consecutive keys of one sequence)
  * and key s of sequence b is row s % 128 of page  page_table[b * max_pages + s / 128]  (device int32
- * [B, max_pages]; entries behind a sequence's last page are never read).  Everything else - q, out, seq_lens,
+ * [B, max_pages]; entries behind a sequence's last page are never read, and an entry outside [0, n_pages) is
+ * clamped into the pool: wrong values, never an access outside it).  Everything else - q, out, seq_lens,
  * max_len, workspace, the split plan, the in-kernel merge - is as in axhip_gqa_decode, and so is the
  * result, bit for bit, for the same keys in the same order: only the address of a key row differs (each
  * workgroup copies the page numbers of its key range from the table into LDS before its first tile).

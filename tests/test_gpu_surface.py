@@ -557,3 +557,59 @@ def test_paged_kv_cache_component():
         pg.reserve([0, 0, 300])                          # past max_len
     pg.reset()
     assert pg.pages_in_use == 0 and len(pg) == 0
+
+
+def test_paged_kv_cache_step_captured_in_a_graph():
+    """One decode step over a PagedKVCache (append through the page table, attention over the pages, length
+    advance) captured once and replayed: pages for all replays are reserved before the capture, so the body
+    has no host <-> device traffic.  Every replay equals the static cache driven eagerly with the same inputs."""
+    rng = np.random.default_rng(43)
+    B, hq, hkv, d, lmax, steps = 2, 4, 2, 64, 384, 5
+    pg = nn.PagedKVCache(1, B, hkv, d, n_pages=6, max_len=lmax, device=DEV, page_order=[5, 1, 4, 0, 3, 2])
+    st = nn.StaticKVCache(1, B, hkv, lmax, d, DataType.FLOAT16, DEV)
+    prompt = [126, 250]                         # both sequences cross a page boundary during the replays
+    for b, n in enumerate(prompt):
+        kr = rng.standard_normal((n, hkv, d)).astype(np.float16)
+        vr = rng.standard_normal((n, hkv, d)).astype(np.float16)
+        pg.update_rows(0, b, t(kr), t(vr))
+        pg.advance_rows(b, n)
+        kc, vc = st.get(0)
+        kh, vh = kc.numpy(), vc.numpy()
+        kh[b, :, :n], vh[b, :, :n] = np.transpose(kr, (1, 0, 2)), np.transpose(vr, (1, 0, 2))
+        kc.copy_from_numpy(kh)
+        vc.copy_from_numpy(vh)
+    st.set_lengths(prompt)
+    pg.reserve(steps + 2)                       # warm-up run + recorded run + replays never allocate a page
+    q_in = Tensor(DataType.FLOAT16, [B, hq, d], DEV)
+    k_in = Tensor(DataType.FLOAT16, [B, hkv, d], DEV)
+    v_in = Tensor(DataType.FLOAT16, [B, hkv, d], DEV)
+    bound = max(prompt) + steps + 2
+
+    def step():
+        pg.update(0, k_in, v_in)
+        out = pg.attend(0, q_in, extra_tokens=1, max_len=bound)
+        pg.advance()
+        return out
+
+    lens0 = pg.seq_lens.to_numpy().copy()
+    g = axono.HIPGraph().capture(step)          # runs the body twice
+    pg.seq_lens.copy_from_numpy(lens0)
+    pg.sync_from_device()
+    for s_ in range(steps):
+        qn = rng.standard_normal((B, hq, d)).astype(np.float16)
+        kn = rng.standard_normal((B, hkv, d)).astype(np.float16)
+        vn = rng.standard_normal((B, hkv, d)).astype(np.float16)
+        q_in.copy_from_numpy(qn)
+        k_in.copy_from_numpy(kn)
+        v_in.copy_from_numpy(vn)
+        g.replay()
+        got = g.output.numpy().copy()
+        st.update(0, t(kn), t(vn))
+        lens1 = Tensor(DataType.INT32, [B], DEV)
+        lens1.copy_from_numpy((np.array(prompt) + s_ + 1).astype(np.int32))
+        want = axono.gqa_decode_attention_cache(t(qn), *st.get(0), lens1, max_len=bound).numpy()
+        st.advance()
+        np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+    pg.sync_from_device()
+    assert len(pg) == max(prompt) + steps
+    np.testing.assert_array_equal(pg.seq_lens.to_numpy(), np.array(prompt) + steps)

@@ -70,7 +70,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
     kinds = [
         ("qkv Linear 2048->4096", nl, lin_bytes(H, (nq + 2 * nkv) * D, 4),
          layers(lambda p, i: model._linear(xn, p + "self_attn.qkv_proj.weight"))),
-        ("attention (q/k norm + M-RoPE + KV append + split-K decode + merge)", nl,
+        ("attention (qk-norm + M-RoPE + KV append + split-K decode + merge)", nl,
          2 * nkv * D * 2 * B * (context + 1) + B * (nq + 2 * nkv) * D * 4 + B * nq * D * 2,
          layers(lambda p, i: L.gqa_decode_attention_qkv(
              qkv, W(p + "self_attn.q_norm.weight"), W(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, model._pos,
@@ -171,7 +171,10 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     result.update({
         "per_kernel": {"how": "each kind of launch captured for all layers (own weights / caches) and replayed back to "
                               "back; host clock around 10 replays; bytes are algorithmic",
-                       "rows": table, "sum_us_per_step": round(in_kernels, 1)},
+                       "cols": ["kernel", "calls_per_step", "us_per_call", "us_per_step", "bytes_per_call", "frac_hbm_peak"],
+                       "rows": [[r["kernel"], r["calls_per_step"], r["us_per_call"], r["us_per_step"], r["bytes_per_call"],
+                                 r["frac_hbm_peak"]] for r in table],
+                       "sum_us_per_step": round(in_kernels, 1)},
         "metric": "decode tok/s 2B-shape B=16", "value": round(tok_s, 1), "unit": "tok/s",
         "ms_per_step": round(ms_step, 4), "steps": decode_steps, "batch": batch, "context": context,
         "graph_nodes": g.num_nodes, "bytes_per_step": int(avg_bytes),

@@ -231,18 +231,14 @@ def cpu_decode_step_hook(cfg, weights, model, first, pos, batch, max_len, log):
            "greedy_tokens_agree": agree, "greedy_tokens_equal": f"{same_tok}/{batch}",
            "restatement_logit_gap_of_device_choice": tie_gap,
            "float64_yardstick": {
-               "what": "the same op sequence in float64 (NumPy) with the same fp16 storage points, from the same cache",
-               "logits_free_running_device_vs_f64": d_gpu, "logits_free_running_restatement_vs_f64": d_cpu,
-               "per_layer_identical_inputs_device_vs_f64": layer_gpu,
-               "per_layer_identical_inputs_restatement_vs_f64": layer_cpu,
-               "logits_identical_final_state_device_vs_f64": tf_gpu,
-               "logits_identical_final_state_restatement_vs_f64": tf_cpu,
+               "logits_free_running": {"device_vs_f64": d_gpu, "restatement_vs_f64": d_cpu},
+               "per_layer_identical_inputs": {"device_vs_f64": layer_gpu, "restatement_vs_f64": layer_cpu},
+               "logits_identical_final_state": {"device_vs_f64": tf_gpu, "restatement_vs_f64": tf_cpu},
                "device_within_1p5x_of_restatement": bool(d_gpu <= max(1.5 * d_cpu, 1e-3)),
                "per_layer_within_2e-3": bool(layer_gpu <= 2e-3)},
-           "note": "fp16 storage points (activation entering each Linear, q, KV cache) round on different "
-                   "sides of an fp16 boundary for a few elements when two correct pipelines differ by 1e-7; "
-                   "free-running, these flips compound over 28 layers, layer-wise they cannot"}
-    return {"cpu_baseline": base, "parity": par}
+           "note": "fp16 storage points let two correct fp32 pipelines drift apart over 28 layers; f64 = the same op "
+                   "sequence in float64 with the same storage points"}
+    return {"cpu_baseline": base, "parity": _sig4(par)}
 
 
 
@@ -265,7 +261,8 @@ def config_tables(lib, with_cpu=True):
     from axono_amd.benchmarks import microbench as mb
 
     out = {"peaks": {"hbm_GBps": HBM_PEAK_GBS, "mfma_f16_dense_TFLOPs": mb.MFMA_F16_PEAK},
-           "timing": "HIP events around back-to-back launches on the stream the kernels run on; us per launch"}
+           "how": "HIP events around back-to-back launches, us per launch, buffers rotated; config 4: bytes = 2KN+2MK+4MN, "
+                  "flops = 2MKN, weights packed; frac = of the bound's peak; cpu_us = the CPU restatement on the same shape"}
     port = None
     if with_cpu:
         import oracle
@@ -314,7 +311,7 @@ def config_tables(lib, with_cpu=True):
         r = mb.collect(mb.bench_gqa, lib, B, L, steps, lens)[0]
         rec = {"B": B, "L": L, "ragged_512_32768": lens is not None, "us": r["us"], "bytes": r["bytes"],
                "GBps": r["GBps"], "frac_hbm": round(r["GBps"] / HBM_PEAK_GBS, 4),
-               "plan": {"ranges_per_sequence": r["splits"], "keys_per_range": r["chunk"]}, "kv_buffers": r["kv_buffers"]}
+               "ranges_per_seq": r["splits"], "keys_per_range": r["chunk"]}
         if lens is None and L in cpu_seq_us:
             rec["cpu_us_one_sequence"] = cpu_seq_us[L]
         c3.append(rec)
@@ -330,18 +327,37 @@ def config_tables(lib, with_cpu=True):
     shapes = [(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)]
     for r in mb.collect(mb.bench_linear, lib, 40, shapes, (1, 16, 32, 512), True, 0):
         M, K, N = r["M"], r["K"], r["N"]
-        rec = {"M": M, "K": K, "N": N, "us": r["us"], "weight_copies_rotated": r["weight_copies"]}
+        rec = {"M": M, "K": K, "N": N, "us": r["us"]}
         if M <= 32:
-            rec.update({"bound": "hbm", "bytes": r["bytes"], "GBps": r["GBps"], "frac_hbm": round(r["GBps"] / HBM_PEAK_GBS, 4)})
+            rec.update({"bound": "hbm", "GBps": r["GBps"], "TFLOPs": None, "frac": round(r["GBps"] / HBM_PEAK_GBS, 4)})
         else:
-            rec.update({"bound": "mfma", "flops": 2 * M * K * N, "TFLOPs": r["TFLOPs"],
-                        "frac_mfma": round(r["TFLOPs"] / mb.MFMA_F16_PEAK, 4)})
+            rec.update({"bound": "mfma", "GBps": None, "TFLOPs": r["TFLOPs"], "frac": round(r["TFLOPs"] / mb.MFMA_F16_PEAK, 4)})
         if port is not None and 2.0 * M * K * N <= 2.1e9:
             xw, ww = h16(M, K), h16(N, K, scale=0.02)
             rec["cpu_us"] = _cpu_min_us(lambda: port.linear(xw, ww), budget_s=0.5, max_runs=5)
         c4.append(rec)
     out["config4_linear_f16_packed"] = c4
-    return out
+    return {k: (_compact(v) if isinstance(v, list) else v) for k, v in out.items()}
+
+
+def _sig4(x):
+    """Floats of a nested dict rounded to four significant digits (distances are quoted, not compared)."""
+    if isinstance(x, dict):
+        return {k: _sig4(v) for k, v in x.items()}
+    if isinstance(x, float):
+        return float(f"{x:.4g}")
+    return x
+
+
+def _compact(rows):
+    """A list of flat records as {"cols": [...], "rows": [[...], ...]} (the JSON line stays short); nested
+    values and missing keys are kept (None where a record lacks a column)."""
+    cols = []
+    for r in rows:
+        for k in r:
+            if k not in cols:
+                cols.append(k)
+    return {"cols": cols, "rows": [[r.get(c) for c in cols] for r in rows]}
 
 
 def smoke_parity(lib):

@@ -54,3 +54,14 @@ def test_argument_checks_run_without_a_device():
     assert lib.axhip_gqa_decode(None, None, None, None, None, None, 0, 5, 1, 16, 5, 128, 16, 0, 0, 0, None) == 4
     assert lib.axhip_kv_append(None, None, None, None, None, 5, 2, 1, 1, 1, 8, None) == 3  # pos dtype
     assert lib.axhip_gqa_decode_workspace_bytes(32, 16, 8, 128, 8192) > 0
+    # entry points added for paged caches, callers that cannot allocate, one-launch RoPE and transpose
+    assert lib.axhip_gqa_decode_static(None, None, None, None, None, 5, 1, 16, 5, 128, 16, 0, 0, 0, None) == 4
+    assert lib.axhip_gqa_decode_static(None, None, None, None, None, 5, 1, 16, 8, 128, 16, 0, 128, 1024, None) == 7
+    assert lib.axhip_gqa_decode_paged(None, None, None, None, None, None, None, 0, 4, 1, 16, 8, 128, 300, 2, 4, None) == 1
+    assert lib.axhip_gqa_decode_paged(None, None, None, None, None, None, None, 0, 4, 1, 16, 8, 128, 256, 2, 4, None) == 7
+    assert lib.axhip_kv_append_paged(None, None, None, None, None, None, 2, 3, 1, 1, 1, 8, 1, 1, None) == 3   # 3-byte elements
+    assert lib.axhip_kv_append_paged(None, None, None, None, None, None, 2, 2, 0, 1, 1, 8, 1, 1, None) == 0   # no sequences
+    assert lib.axhip_rope_qk(None, None, None, 1e6, None, None, 5, 4, 2, 1, 7, None) == 1                      # odd head size
+    assert lib.axhip_transpose(None, None, 3, 1, 2, 1, 2, 1, None) == 3
+    assert lib.axhip_transpose(None, None, 4, 1, 2, 1, 0, 1, None) == 0                                        # no elements
+    assert lib.axhip_reset_tickets() == 0                                                                      # no device: nothing to reset

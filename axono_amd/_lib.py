@@ -67,6 +67,7 @@ PROTOTYPES = {
     "axhip_gqa_decode_paged": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_i,
                                      c_vp]),
     "axhip_kv_append_paged": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "axhip_kv_dense_to_paged": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_sdpa": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_kv_append": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_concat": (c_i, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
@@ -94,6 +95,8 @@ PROTOTYPES = {
     "axhip_prefill_attention": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_gqa_decode_qkv": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i, c_i, c_vp,
                                    c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
+    "axhip_gqa_decode_qkv_paged": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i, c_i, c_vp,
+                                         c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_qkv_norm_rope_append": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp,
                                          c_i, c_i, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_silu_mul_fused": (c_i, [c_vp, c_vp, c_i, c_i, c_i64, c_i64, c_vp]),

@@ -455,7 +455,6 @@ __device__ __forceinline__ void write_zero_rows(const DecodeArgs &a, int b, int 
 template <typename T, int D, int G, int U, bool QKV, bool HOIST, bool PAGED = false>
 __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg, int split, int n_valid,
                                               bool direct_ok, int s0, int s1) {
-  static_assert(!(QKV && PAGED), "the decode-step form reads a dense cache");
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
   int tid = threadIdx.x;
@@ -520,8 +519,14 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
         norm_rope_row<T, D>(a, a.pq + b * a.pq_stride + static_cast<int64_t>(h0 + job) * D, a.qw, b, B, lane, s_q[job],
                             static_cast<T *>(nullptr));
       } else {
-        T *crow = const_cast<T *>(static_cast<const T *>(job == G ? a.k : a.v)) + b * a.stride_b + hk * a.stride_h +
-                  static_cast<int64_t>(p_new) * a.stride_s;
+        // the cache row of the new token: through the page numbers of this range when the cache is paged
+        // (p_new lies in [s0, s1), so its page is among them)
+        T *crow = const_cast<T *>(static_cast<const T *>(job == G ? a.k : a.v));
+        if constexpr (PAGED)
+          crow += s_pages[(p_new >> kPageShift) - first_page] * a.page_stride + static_cast<int64_t>(hk) * (kPageKeys * D) +
+                  (p_new & (kPageKeys - 1)) * D;
+        else
+          crow += b * a.stride_b + hk * a.stride_h + static_cast<int64_t>(p_new) * a.stride_s;
         if (job == G) {
           norm_rope_row<T, D>(a, a.pk + b * a.pk_stride + static_cast<int64_t>(hk) * D, a.kw, b, B, lane, s_kv[0],
                               writer ? crow : static_cast<T *>(nullptr));
@@ -1146,7 +1151,12 @@ int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   constexpr int U = (sizeof(T) == 2 ? 8 : 4) / (G >= 4 ? 2 : 1);
   // static plan: (split, head group, sequence); length-dealt plan: one dimension, slot index slowest
   const dim3 grid(a.dynamic ? a.active * (a.Hq / G) : a.n_splits, a.dynamic ? 1 : a.Hq / G, a.dynamic ? 1 : B);
-  if (a.page_table)
+  if (a.page_table && a.len_add) {
+    if constexpr (sizeof(T) == 2)  // the decode-step form over a paged cache: fp16 caches
+      hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, true, false, true>), grid, dim3(kThreads), 0, st, a);
+    else
+      return AXHIP_UNSUPPORTED_TYPE;
+  } else if (a.page_table)
     hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, false, false, true>), grid, dim3(kThreads), 0, st, a);
   else if (a.len_add)
     hipLaunchKernelGGL((gqa_decode_split_kernel<T, D, G, U, true>), grid, dim3(kThreads), 0, st, a);
@@ -1436,6 +1446,55 @@ AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float
   a.h_lim = h_sec * 3;
   a.w_lim = w_sec * 3;
   a.cache_rows = cache_rows;
+  return plan_and_launch(a, workspace, workspace_bytes, cache_dtype, B, Hq, Hkv, D, max_len, stream);
+}
+
+// axhip_gqa_decode_qkv over a paged cache: the new token's k / v row goes to row seq_lens[b] % 128 of page
+// page_table[b, seq_lens[b] / 128] (the page must have been reserved), the keys are read through the table.
+AXHIP_API int axhip_gqa_decode_qkv_paged(const float *q, int64_t q_stride, const float *k, int64_t k_stride,
+                                         const float *v, int64_t v_stride, const void *q_weight, const void *k_weight,
+                                         int w_dtype, float eps, const int64_t *pos, const float *inv_freq, int h_sec,
+                                         int w_sec, const int32_t *seq_lens, void *k_pool, void *v_pool,
+                                         const int32_t *page_table, void *out, void *workspace, size_t workspace_bytes,
+                                         int cache_dtype, int B, int Hq, int Hkv, int D, int max_len, int max_pages,
+                                         int n_pages, axhip_stream stream) {
+  if (cache_dtype != AXHIP_FLOAT16) return AXHIP_UNSUPPORTED_TYPE;
+  if ((q_weight || k_weight) && !is_float_dtype(w_dtype)) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || Hq <= 0 || Hkv <= 0 || max_len <= 0 || max_pages <= 0 || n_pages <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (Hq % Hkv != 0) return AXHIP_SHAPE_MISMATCH;
+  if (D != 64 && D != 128 && D != 256) return AXHIP_INVALID_ARGUMENT;
+  if (static_cast<int64_t>(max_pages) * kPageKeys < max_len || max_len > (kMaxRangePages - 1) * kPageKeys)
+    return AXHIP_INVALID_ARGUMENT;
+  if (B == 0) return AXHIP_OK;
+  if (B > 65535) return AXHIP_INVALID_ARGUMENT;
+  if (!q || !k || !v || !pos || !inv_freq || !seq_lens || !k_pool || !v_pool || !page_table || !out) return AXHIP_INVALID_PTR;
+  if ((reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool)) & 15) return AXHIP_INVALID_PTR;
+  DecodeArgs a{};
+  a.k = k_pool;
+  a.v = v_pool;
+  a.seq_lens = seq_lens;
+  a.out = out;
+  a.page_table = page_table;
+  a.max_pages = max_pages;
+  a.n_pages = n_pages;
+  a.page_stride = static_cast<int64_t>(Hkv) * kPageKeys * D;
+  a.stride_s = D;
+  a.len_add = 1;
+  a.pq = q;
+  a.pk = k;
+  a.pv = v;
+  a.pq_stride = q_stride;
+  a.pk_stride = k_stride;
+  a.pv_stride = v_stride;
+  a.qw = q_weight;
+  a.kw = k_weight;
+  a.w_f16 = w_dtype == AXHIP_FLOAT16;
+  a.eps = eps;
+  a.pos = pos;
+  a.inv_freq = inv_freq;
+  a.h_lim = h_sec * 3;
+  a.w_lim = w_sec * 3;
+  a.cache_rows = max_pages * kPageKeys;
   return plan_and_launch(a, workspace, workspace_bytes, cache_dtype, B, Hq, Hkv, D, max_len, stream);
 }
 

@@ -592,6 +592,34 @@ __global__ __launch_bounds__(kBlock) void kv_append_paged_kernel(const uint8_t *
   st16(v_pool + dst, ld16(v_new + src));
 }
 
+// Dense cache [B, Hkv, rows, row_bytes] -> pages: key positions 0 .. lens[b]-1 (all `rows` when lens is null) of
+// every sequence are copied to row (position % 128) of page page_table[b, position / 128].
+__global__ __launch_bounds__(kBlock) void kv_dense_to_paged_kernel(const uint8_t *__restrict__ k_dense,
+                                                                   const uint8_t *__restrict__ v_dense,
+                                                                   uint8_t *__restrict__ k_pool, uint8_t *__restrict__ v_pool,
+                                                                   const int32_t *__restrict__ page_table,
+                                                                   const int32_t *__restrict__ lens, int B, int Hkv, int rows,
+                                                                   int row_bytes, int max_pages, int n_pages) {
+  const int vec_per_row = row_bytes / 16;
+  const int64_t total = static_cast<int64_t>(B) * Hkv * rows * vec_per_row;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; t < total; t += stride) {
+    const int vi = static_cast<int>(t % vec_per_row);
+    const int64_t r = t / vec_per_row;                 // (b, head, position)
+    const int p = static_cast<int>(r % rows);
+    const int64_t bh = r / rows;
+    const int hk = static_cast<int>(bh % Hkv), b = static_cast<int>(bh / Hkv);
+    if (lens && p >= lens[b]) continue;
+    if ((p >> 7) >= max_pages) continue;
+    const int pid = page_table[static_cast<int64_t>(b) * max_pages + (p >> 7)];
+    if (pid < 0 || pid >= n_pages) continue;
+    const int64_t src = r * row_bytes + vi * 16;
+    const int64_t dst = ((static_cast<int64_t>(pid) * Hkv + hk) * 128 + (p & 127)) * row_bytes + vi * 16;
+    st16(k_pool + dst, ld16(k_dense + src));
+    st16(v_pool + dst, ld16(v_dense + src));
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Embedding gather and argmax.
 // ------------------------------------------------------------------------------------------------
@@ -1009,6 +1037,26 @@ AXHIP_API int axhip_kv_append_paged(const void *k_new, const void *v_new, void *
   else
     hipLaunchKernelGGL((kv_append_paged_kernel<int32_t>), grid, dim3(kBlock), 0, st, kn, vn, kp, vp, page_table,
                        static_cast<const int32_t *>(start), B, S, Hkv, row_bytes, max_pages, n_pages);
+  return launch_status();
+}
+
+AXHIP_API int axhip_kv_dense_to_paged(const void *k_dense, const void *v_dense, void *k_pool, void *v_pool,
+                                      const int32_t *page_table, const int32_t *lens, int elem_bytes, int B, int Hkv,
+                                      int rows, int D, int max_pages, int n_pages, axhip_stream stream) {
+  if (elem_bytes != 2 && elem_bytes != 4) return AXHIP_UNSUPPORTED_TYPE;
+  if (B < 0 || Hkv <= 0 || rows < 0 || D <= 0 || max_pages <= 0 || n_pages <= 0) return AXHIP_INVALID_ARGUMENT;
+  if (B == 0 || rows == 0) return AXHIP_OK;
+  if (!k_dense || !v_dense || !k_pool || !v_pool || !page_table) return AXHIP_INVALID_PTR;
+  const int row_bytes = D * elem_bytes;
+  if (row_bytes % 16 != 0 || !aligned16(k_dense) || !aligned16(v_dense) || !aligned16(k_pool) || !aligned16(v_pool))
+    return AXHIP_INVALID_ARGUMENT;
+  const int64_t total = static_cast<int64_t>(B) * Hkv * rows * (row_bytes / 16);
+  unsigned grid = blocks_for(total, kBlock);
+  if (grid > 256u * 32u) grid = 256u * 32u;
+  hipLaunchKernelGGL(kv_dense_to_paged_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream),
+                     static_cast<const uint8_t *>(k_dense), static_cast<const uint8_t *>(v_dense),
+                     static_cast<uint8_t *>(k_pool), static_cast<uint8_t *>(v_pool), page_table, lens, B, Hkv, rows, row_bytes,
+                     max_pages, n_pages);
   return launch_status();
 }
 

@@ -141,7 +141,12 @@ def _dev(arr, device):
 
 
 class Qwen3VLTextDecoder(nn.Module):
-    def __init__(self, cfg: TextConfig, weights: dict, batch: int, max_len: int, device: str = "hip"):
+    """paged=True keeps the KV cache in pages of 128 keys (nn.PagedKVCache, `n_pages` per layer pool; default:
+    enough for every sequence to reach max_len) instead of one [B, n_kv, max_len, d_head] block per layer; the
+    prefill of a sequence then runs over one dense scratch block and is copied into the sequence's pages."""
+
+    def __init__(self, cfg: TextConfig, weights: dict, batch: int, max_len: int, device: str = "hip", paged: bool = False,
+                 n_pages: int | None = None):
         super().__init__()
         self._cfg = cfg
         self._device = device
@@ -155,8 +160,18 @@ class Qwen3VLTextDecoder(nn.Module):
                         for name, t in self._parameters.items()
                         if name.endswith("_proj.weight") or name == "embed_tokens.weight"}
         self._inv_freq = _dev(inv_freq_table(cfg.rope_theta, cfg.head_dim), device)
-        self._cache = nn.StaticKVCache(cfg.num_hidden_layers, batch, cfg.num_key_value_heads, max_len, cfg.head_dim,
-                                       DataType.FLOAT16, device)
+        self._paged = bool(paged)
+        if self._paged:
+            per_seq = (max_len + nn.PagedKVCache.PAGE - 1) // nn.PagedKVCache.PAGE
+            self._cache = nn.PagedKVCache(cfg.num_hidden_layers, batch, cfg.num_key_value_heads, cfg.head_dim,
+                                          n_pages if n_pages is not None else batch * per_seq, max_len,
+                                          DataType.FLOAT16, device)
+            # prefill works on one sequence and one layer at a time over this dense block
+            shape = [1, cfg.num_key_value_heads, per_seq * nn.PagedKVCache.PAGE, cfg.head_dim]
+            self._scratch_kv = (Tensor(DataType.FLOAT16, shape, device), Tensor(DataType.FLOAT16, shape, device))
+        else:
+            self._cache = nn.StaticKVCache(cfg.num_hidden_layers, batch, cfg.num_key_value_heads, max_len, cfg.head_dim,
+                                           DataType.FLOAT16, device)
         # static state of the captured step
         self._ids = Tensor(DataType.INT64, [batch], device)
         self._pos = Tensor(DataType.INT64, [3, batch], device)
@@ -171,8 +186,18 @@ class Qwen3VLTextDecoder(nn.Module):
         return self._parameters[name]
 
     @property
-    def cache(self) -> nn.StaticKVCache:
+    def cache(self):
         return self._cache
+
+    def _attention_step(self, qkv, p, i, pos, max_len):
+        """q/k RMSNorm + M-RoPE + KV append + attention over seq_lens + 1 keys: one launch (+ the merge)."""
+        cfg, cache = self._cfg, self._cache
+        args = (qkv, self._w(p + "self_attn.q_norm.weight"), self._w(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, pos,
+                self._inv_freq, cfg.mrope_section, cache.seq_lens, *cache.get(i))
+        if self._paged:
+            return L.gqa_decode_attention_qkv_paged(*args, cache.page_table, cfg.num_attention_heads, max_len,
+                                                    workspace=self._attn_ws)
+        return L.gqa_decode_attention_qkv(*args, cfg.num_attention_heads, max_len, workspace=self._attn_ws)
 
     def _linear(self, x, name):
         """x @ W^T over the packed copy of the weight (skinny kernels in decode, MFMA GEMM in prefill)."""
@@ -212,12 +237,7 @@ class Qwen3VLTextDecoder(nn.Module):
             if trace is not None:
                 trace.append(h)
             qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")
-            kc, vc = cache.get(i)
-            # q/k RMSNorm + M-RoPE + KV append + attention over seq_lens + 1 keys: one launch (+ the merge)
-            attn = L.gqa_decode_attention_qkv(qkv, self._w(p + "self_attn.q_norm.weight"),
-                                              self._w(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, pos,
-                                              self._inv_freq, cfg.mrope_section, cache.seq_lens, kc, vc,
-                                              cfg.num_attention_heads, max_len, workspace=self._attn_ws)
+            attn = self._attention_step(qkv, p, i, pos, max_len)
             attn_out = self._linear(attn.reshape([B, nqd]), p + "self_attn.o_proj.weight")
             h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                     DataType.FLOAT16)
@@ -250,14 +270,22 @@ class Qwen3VLTextDecoder(nn.Module):
         ws = Tensor(DataType.INT8, [max(wsb, 256)], dev, _zero=False)
         last_h = Tensor(DataType.FLOAT16, [B, H], dev)  # normalised hidden state of each sequence's last token
         esz = 2
+        if self._paged:
+            self._cache.reserve(S)
+            lmax = self._scratch_kv[0].shape[2]
+            s_lens = _dev(np.full(B, S, np.int32), dev)
         for b in range(B):
             h = L.embedding(_dev(ids[b].astype(np.int64), dev), self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)
             xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
             for i in range(cfg.num_hidden_layers):
                 p = f"layers.{i}."
                 qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")  # [S, width] fp32
-                kc, vc = self._cache.get(i)
-                seq_off = b * nkv * lmax * D * esz
+                if self._paged:
+                    kc, vc = self._scratch_kv   # this sequence's rows of this layer, dense; copied to its pages below
+                    seq_off = 0
+                else:
+                    kc, vc = self._cache.get(i)
+                    seq_off = b * nkv * lmax * D * esz
                 q = Tensor(DataType.FLOAT16, [S, nq, D], dev, _zero=False)
                 base = qkv.data_ptr
                 check(lib.axhip_qkv_norm_rope_append(
@@ -278,6 +306,8 @@ class Qwen3VLTextDecoder(nn.Module):
                     check(lib.axhip_gqa_decode(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, vis.data_ptr,
                                                attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq,
                                                nkv, D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
+                if self._paged:
+                    L.kv_dense_to_paged(kc, vc, *self._cache.get(i), self._cache.page_table, lens=s_lens, table_row=b)
                 attn_out = self._linear(attn, p + "self_attn.o_proj.weight")
                 h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                     DataType.FLOAT16)
@@ -298,6 +328,10 @@ class Qwen3VLTextDecoder(nn.Module):
         self._ids.copy_from_numpy(np.ascontiguousarray(first_ids, dtype=np.int64).reshape(B))
         self._pos.copy_from_numpy(np.ascontiguousarray(first_pos, dtype=np.int64).reshape(3, B))
         bound = min(self._cache.max_len, len(self._cache) + max_new_tokens + 1)
+        if self._paged:
+            # pages for every token the loop (and the two runs of a capture) can write: allocated now, so
+            # that the captured step never touches the page table
+            self._cache.reserve(bound - len(self._cache))
         # the captured attention launches attend to at most `bound` keys and append only below it:
         # generate() refuses to run past it (it would silently drop tokens from the cache otherwise)
         self._decode_bound = bound
@@ -356,5 +390,5 @@ class Qwen3VLTextDecoder(nn.Module):
         if use_graph:
             self._graph.sync()
         L.synchronize()
-        self._cache._host_len += max_new_tokens
+        self._cache.note_advanced(max_new_tokens)   # the steps advanced the lengths on the device
         return self._log.numpy()[:max_new_tokens].copy()

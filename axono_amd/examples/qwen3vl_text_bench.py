@@ -72,10 +72,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
          layers(lambda p, i: model._linear(xn, p + "self_attn.qkv_proj.weight"))),
         ("attention (qk-norm + M-RoPE + KV append + split-K decode + merge)", nl,
          2 * nkv * D * 2 * B * (context + 1) + B * (nq + 2 * nkv) * D * 4 + B * nq * D * 2,
-         layers(lambda p, i: L.gqa_decode_attention_qkv(
-             qkv, W(p + "self_attn.q_norm.weight"), W(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, model._pos,
-             model._inv_freq, cfg.mrope_section, lens, *model.cache.get(i), nq, model._decode_bound,
-             workspace=model._attn_ws))),
+         layers(lambda p, i: model._attention_step(qkv, p, i, model._pos, model._decode_bound))),
         ("o_proj Linear 2048->2048", nl, lin_bytes(nq * D, H, 4),
          layers(lambda p, i: model._linear(attn, p + "self_attn.o_proj.weight"))),
         ("add + RMSNorm (fp32 residual, fp16 out)", 2 * nl, B * H * (4 + 4 + 4 + 2) + 4 * H,
@@ -111,7 +108,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
 
 
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
-        cpu_step_hook=None, cfg: TextConfig | None = None, kernel_table: bool = True) -> dict:
+        cpu_step_hook=None, cfg: TextConfig | None = None, kernel_table: bool = True, paged: bool = False) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
     after the prefill with the model positioned at the first decode step (the benchmark passes a
     hook that times and compares a CPU restatement of one step); its dict is merged into the result."""
@@ -121,7 +118,7 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     log(f"[decode] random weights: {sum(w.size for w in weights.values()) / 1e9:.2f} G params in {time.perf_counter() - t0:.1f} s")
     max_len = context + decode_steps + 1
     max_len = (max_len + 127) // 128 * 128
-    model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0")
+    model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0", paged=paged)
     rng = np.random.default_rng(seed + 1)
     ids = rng.integers(0, cfg.vocab_size, (batch, context)).astype(np.int64)
 
@@ -147,8 +144,7 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
         g.replay()
     model._ids.copy_from_numpy(state[0])
     model._pos.copy_from_numpy(state[1])
-    model.cache.seq_lens.copy_from_numpy(state[2])
-    model.cache._host_len = context
+    model.cache.set_lengths(state[2])
     L.synchronize()
     t0 = time.perf_counter()
     toks = model.generate(decode_steps, use_graph=True)  # ends with a device synchronisation
@@ -195,6 +191,7 @@ def main(argv=None):
     ap.add_argument("--gqa-two-kernels", type=int, default=0, metavar="SPLITS",
                     help="attention with a fixed split count and a second merge kernel (the default deals "
                          "workgroups by length and merges in the last workgroup)")
+    ap.add_argument("--paged", action="store_true", help="keep the KV cache in pages of 128 keys (nn.PagedKVCache)")
     ap.add_argument("--no-kernel-table", action="store_true",
                     help="skip the per-kernel table (its extra launches would mix into a profiler's kernel statistics)")
     args = ap.parse_args(argv)
@@ -202,7 +199,7 @@ def main(argv=None):
         from .. import _lib
         _lib.load().axhip_gqa_decode_tune(-1, args.gqa_two_kernels)
     res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
-              kernel_table=not args.no_kernel_table)
+              kernel_table=not args.no_kernel_table, paged=args.paged)
     print(json.dumps(res), flush=True)
 
 

@@ -722,6 +722,81 @@ def gqa_decode_attention_qkv(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, ep
     return out
 
 
+def gqa_decode_attention_qkv_paged(qkv: Tensor, q_weight: Tensor, k_weight: Tensor, eps: float, pos: Tensor, inv_freq: Tensor,
+                                   mrope_section, seq_lens: Tensor, k_pool: Tensor, v_pool: Tensor, page_table: Tensor,
+                                   n_q_heads: int, max_len: int, workspace: Tensor | None = None) -> Tensor:
+    """gqa_decode_attention_qkv over a paged cache (pools (n_pages,Hkv,128,D) FLOAT16, page_table INT32
+    (B,max_pages)): the new token's k / v row is written through the table at position seq_lens[b] (its page
+    must be reserved) and the query attends over seq_lens[b] + 1 keys.  Same bits as the dense form."""
+    op = "gqa_decode_attention"
+    _need_hip(op, qkv, q_weight, k_weight, pos, inv_freq, seq_lens, k_pool, v_pool, page_table, workspace)
+    if qkv.dtype != DataType.FLOAT32 or k_pool.ndim != 4 or k_pool.dtype != DataType.FLOAT16 or v_pool.dtype != k_pool.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    n_pages, hkv, pk, d = k_pool.shape
+    B = seq_lens.num_elements
+    hq = int(n_q_heads)
+    width = (hq + 2 * hkv) * d
+    if pk != PAGE_KEYS or qkv.num_elements != B * width or v_pool.shape != k_pool.shape:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if pos.dtype != DataType.INT64 or pos.shape != [3, B] or seq_lens.dtype != DataType.INT32:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if page_table.dtype != DataType.INT32 or page_table.ndim != 2 or page_table.shape[0] != B:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if inv_freq.dtype != DataType.FLOAT32 or inv_freq.num_elements != d // 2:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    for w in (q_weight, k_weight):
+        if w is not None and (w.num_elements != d or w.dtype not in _FLOATS):
+            raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    _, h_sec, w_sec = (list(mrope_section) + [0, 0, 0])[:3]
+    bound = int(max_len)
+    lib = _lib_()
+    wsb = lib.axhip_gqa_decode_workspace_bytes(B, hq, hkv, d, bound)
+    if workspace is None:
+        workspace = _new(DataType.INT8, [max(wsb, 256)], qkv)
+    out = _new(k_pool.dtype, [B, hq, d], qkv)
+    base = qkv.data_ptr
+    wdt = int(q_weight.dtype) if q_weight is not None else int(DataType.FLOAT32)
+    check(lib.axhip_gqa_decode_qkv_paged(
+        base, width, base + hq * d * 4, width, base + (hq + hkv) * d * 4, width,
+        q_weight.data_ptr if q_weight is not None else None, k_weight.data_ptr if k_weight is not None else None,
+        wdt, float(eps), pos.data_ptr, inv_freq.data_ptr, int(h_sec), int(w_sec), seq_lens.data_ptr,
+        k_pool.data_ptr, v_pool.data_ptr, page_table.data_ptr, out.data_ptr, workspace.data_ptr, workspace.num_bytes,
+        int(k_pool.dtype), B, hq, hkv, d, bound, page_table.shape[1], n_pages, current_stream()), op)
+    return out
+
+
+def kv_dense_to_paged(k_dense: Tensor, v_dense: Tensor, k_pool: Tensor, v_pool: Tensor, page_table: Tensor,
+                      lens: Tensor | None = None, table_row: int | None = None) -> None:
+    """Copies the first lens[b] key positions (all rows when lens is None) of dense caches [B,Hkv,rows,D] into
+    the pages the table names.  table_row: the dense caches hold ONE sequence, the one of that table row."""
+    op = "kv_dense_to_paged"
+    _need_hip(op, k_dense, v_dense, k_pool, v_pool, page_table, lens)
+    if k_dense.ndim != 4 or k_pool.ndim != 4 or k_dense.dtype != k_pool.dtype or v_dense.dtype != k_pool.dtype or v_pool.dtype != k_pool.dtype:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    B, hkv, rows, d = k_dense.shape
+    n_pages, hkv_p, pk, d_p = k_pool.shape
+    tb, max_pages = page_table.shape
+    tbl = page_table.data_ptr
+    lens_ptr = lens.data_ptr if lens is not None else None
+    if table_row is not None:
+        if B != 1 or not 0 <= table_row < tb:
+            raise AxhipError(op, Status.INVALID_ARGUMENT)
+        tbl += table_row * max_pages * 4
+        if lens is not None:
+            lens_ptr += table_row * 4
+    elif tb != B:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if pk != PAGE_KEYS or hkv_p != hkv or d_p != d or v_dense.shape != k_dense.shape or v_pool.shape != k_pool.shape:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if lens is not None and lens.dtype != DataType.INT32:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    check(_lib_().axhip_kv_dense_to_paged(k_dense.data_ptr, v_dense.data_ptr, k_pool.data_ptr, v_pool.data_ptr, tbl, lens_ptr,
+                                          k_pool.num_bytes // max(k_pool.num_elements, 1), B, hkv, rows, d, max_pages, n_pages,
+                                          current_stream()), op)
+
+
 # ---- graph capture -------------------------------------------------------------------------------
 def set_ticket_lane(lane: int) -> None:
     """Attention and wide argmax launches issued (or captured) from now on by this thread use the

@@ -166,6 +166,11 @@ class StaticKVCache(KVCache):
         self.seq_lens.copy_from_numpy(lens)
         self._host_len = int(lens.max()) if lens.size else 0
 
+    def note_advanced(self, n: int) -> None:
+        """The device-side lengths were advanced by n outside `advance` (replays of a captured step): keeps the
+        host-side view in step."""
+        self._host_len += int(n)
+
     def reset(self) -> None:
         self.seq_lens.fill_zero()
         self._host_len = 0
@@ -296,6 +301,18 @@ class PagedKVCache(KVCache):
         bound = int(max_len) if max_len is not None else int(self._lens.max()) + int(extra_tokens)
         return _l.gqa_decode_attention_paged(q, self._k[layer_idx], self._v[layer_idx], self.page_table, lens,
                                              max(min(bound, self.max_len), 1))
+
+    def set_lengths(self, lens) -> None:
+        """Sets every sequence's length (pages for them must exist: `reserve` / `update_rows` first)."""
+        lens = np.ascontiguousarray(lens, dtype=np.int64).reshape(self.batch)
+        if np.any((lens + self.PAGE - 1) // self.PAGE > self._owned):
+            raise ValueError("PagedKVCache.set_lengths: a sequence has fewer pages than its length needs")
+        self._lens = lens.copy()
+        self.seq_lens.copy_from_numpy(lens.astype(np.int32))
+
+    def note_advanced(self, n: int) -> None:
+        """The device-side lengths were advanced by n outside `advance` (replays of a captured step)."""
+        self._lens += int(n)
 
     def sync_from_device(self) -> None:
         """Refreshes the host mirror of the lengths from the device tensor (after replays of a captured

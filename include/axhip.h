@@ -285,6 +285,15 @@ AXHIP_API int axhip_kv_append_paged(const void *k_new, const void *v_new, void *
                                     int elem_bytes, int B, int S, int Hkv, int D, int max_pages,
                                     int n_pages, axhip_stream stream);
 
+/* Copies sequences from a dense cache into a paged one (after a prefill that filled dense rows): key positions
+ * 0 .. lens[b]-1 (device int32 [B]; NULL: all `rows`) of k_dense / v_dense [B, Hkv, rows, D] go to row
+ * (position % 128) of page page_table[b, position / 128].  A byte copy; positions behind the table and page
+ * numbers outside [0, n_pages) are skipped.  No reference counterpart. */
+AXHIP_API int axhip_kv_dense_to_paged(const void *k_dense, const void *v_dense, void *k_pool, void *v_pool,
+                                      const int32_t *page_table, const int32_t *lens, int elem_bytes, int B,
+                                      int Hkv, int rows, int D, int max_pages, int n_pages,
+                                      axhip_stream stream);
+
 /* out = [a ; b] along an axis: `outer` blocks of a_bytes then b_bytes each (axis 0: outer = 1).
  * Replaces ops::cuda::Concat, src/ops/cuda/sequence.cu:474-521. */
 AXHIP_API int axhip_concat(const void *a, const void *b, void *out, int64_t outer, int64_t a_bytes,
@@ -475,6 +484,20 @@ AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float
                                    void *k_cache, void *v_cache, void *out, void *workspace,
                                    size_t workspace_bytes, int cache_dtype, int B, int Hq, int Hkv, int D,
                                    int cache_rows, int max_len, axhip_stream stream);
+
+/* axhip_gqa_decode_qkv over a paged cache (pools, page table, max_pages, n_pages as for
+ * axhip_gqa_decode_paged; FLOAT16 caches): the new token's k / v row goes to row seq_lens[b] % 128 of page
+ * page_table[b, seq_lens[b] / 128] - that page must already be in the table - when seq_lens[b] < max_len, and
+ * the keys are read through the table.  Same bits as axhip_gqa_decode_qkv on a dense cache holding the same rows.
+ * No reference counterpart. */
+AXHIP_API int axhip_gqa_decode_qkv_paged(const float *q, int64_t q_stride, const float *k, int64_t k_stride,
+                                         const float *v, int64_t v_stride, const void *q_weight,
+                                         const void *k_weight, int w_dtype, float eps, const int64_t *pos,
+                                         const float *inv_freq, int h_sec, int w_sec, const int32_t *seq_lens,
+                                         void *k_pool, void *v_pool, const int32_t *page_table, void *out,
+                                         void *workspace, size_t workspace_bytes, int cache_dtype, int B, int Hq,
+                                         int Hkv, int D, int max_len, int max_pages, int n_pages,
+                                         axhip_stream stream);
 
 /* y[r, c] = silu(gate_up[r, c]) * gate_up[r, cols + c] for a fused [gate | up] projection output
  * [rows, 2*cols] -> [rows, cols].  Same arithmetic as axhip_silu_mul.  cols % 8 == 0.  out_dtype

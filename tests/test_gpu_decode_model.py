@@ -229,3 +229,46 @@ def test_device_is_no_farther_from_the_float64_evaluation_than_the_fp32_restatem
     assert d_gpu <= max(1.5 * d_cpu, 1e-3), (d_gpu, d_cpu)
     assert layer_gpu <= 2e-3 and layer_cpu <= 2e-3, (layer_gpu, layer_cpu)
     assert layer_gpu <= max(1.5 * layer_cpu, 1e-3), (layer_gpu, layer_cpu)
+
+
+def test_paged_decoder_gives_the_tokens_and_logits_of_the_dense_one():
+    """The decoder over a PagedKVCache (prefill through a dense scratch block copied into pages, decode step
+    with the paged attention launch, captured and replayed) against the same decoder over the static cache:
+    same prefill logits, same tokens, same logits of the last replay, bit for bit; pages in use follow the
+    tokens; and against the oracle like the dense one."""
+    n_steps = 6
+    dense, cpu, ids = _setup(seed=23, S=125, max_len=160)      # the steps cross the first page boundary
+    B, S = ids.shape
+    w = cpu.w
+    paged = Qwen3VLTextDecoder(CFG, w, B, 160, "hip:0", paged=True)
+    outs = {}
+    for name, m in (("dense", dense), ("paged", paged)):
+        logits, nxt = m.prefill(ids)
+        first = nxt.to_numpy().copy()
+        m.start_decode(first, np.full((3, B), S, np.int64), n_steps)
+        m.capture()
+        toks = m.generate(n_steps)
+        outs[name] = (logits.to_numpy().copy(), first, toks, m._graph_out[0].to_numpy().copy())
+    for a, b in zip(outs["dense"], outs["paged"]):
+        np.testing.assert_array_equal(a, b)
+    assert paged.cache.pages_in_use == B * 2 and len(paged.cache) == S + n_steps
+    np.testing.assert_array_equal(paged.cache.seq_lens.to_numpy(), [S + n_steps] * B)
+    # the cached rows, read back through the page table, are the dense cache's rows
+    table = paged.cache.page_table.to_numpy()
+    for i in range(CFG.num_hidden_layers):
+        kd = dense.cache.get(i)[0].numpy()
+        kp = paged.cache.get(i)[0].numpy()
+        for b in range(B):
+            for pg in range(2):
+                rows = min(128, S + n_steps - pg * 128)
+                np.testing.assert_array_equal(kp[table[b, pg], :, :rows].view(np.uint16),
+                                              kd[b, :, pg * 128:pg * 128 + rows].view(np.uint16))
+    # and the oracle accepts the tokens
+    c_logits, _ = cpu.prefill(ids)
+    assert np.abs(outs["paged"][0] - c_logits).max() <= 2e-3
+    cur, pos = outs["paged"][1], np.full((3, B), S, np.int64)
+    for s in range(n_steps):
+        logits, _ = cpu.decode_step(cur, pos + s)
+        chosen = logits[np.arange(B), outs["paged"][2][s]]
+        assert np.all(chosen >= logits.max(-1) - 4e-3)
+        cur = outs["paged"][2][s]

@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the headline split kernel, from the rocprofv3 --pmc runs recorded in
-# profiles/gqa_decode_split_B32_L8192_f16.md (a measured constant, not computed in this process)
+# profiles/gqa_decode_split_B32_L8192_f16.md: reported when the counters cannot be read live (measure_traffic)
 MEASURED_TRAFFIC_BYTES = 1074196367
 
 F16 = 4
@@ -360,6 +360,52 @@ def _compact(rows):
     return {"cols": cols, "rows": [[r.get(c) for c in cols] for r in rows]}
 
 
+def measure_traffic(log, timeout_s=90):
+    """HBM bytes per launch of the headline kernel, read from the hardware counters in child processes: four short
+    `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE, for the attention microbenchmark and for a plain copy
+    kernel of 1 GiB each way, which gives each counter's scale factor).  Returns (bytes, details) or None when
+    the profiler is not usable here (the recorded constant is reported then)."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+
+    exe = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(exe):
+        return None
+    env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""), TMPDIR="/tmp")
+    base = tempfile.mkdtemp(prefix="axhip_pmc_", dir="/tmp")
+    readings = {}
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            for what, kernel in (("gqa", "gqa_decode_split_kernel"), ("copy", "copy_bytes_kernel")):
+                out = os.path.join(base, f"{counter}_{what}")
+                cmd = [exe, "--pmc", counter, "-d", out, "-o", "p", "--output-format", "csv", "--", sys.executable, "-m",
+                       "axono_amd.benchmarks.microbench", what, "--steps", "3"]
+                r = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                                   timeout=timeout_s)
+                files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
+                if r.returncode != 0 or not files:
+                    return None
+                vals = [float(row["Counter_Value"]) for row in csv.DictReader(open(files[0]))
+                        if kernel in row["Kernel_Name"] and row["Counter_Name"] == counter]
+                if not vals:
+                    return None
+                readings[(counter, what)] = sum(vals) / len(vals)   # KiB per dispatch
+        gib_kib = float(1 << 20)  # the copy kernel moves 1 GiB each way
+        f_fetch, f_write = gib_kib / readings[("FETCH_SIZE", "copy")], gib_kib / readings[("WRITE_SIZE", "copy")]
+        kib = readings[("FETCH_SIZE", "gqa")] * f_fetch + readings[("WRITE_SIZE", "gqa")] * f_write
+        return int(round(kib * 1024)), {"FETCH_SIZE_KiB": round(readings[("FETCH_SIZE", "gqa")], 2),
+                                        "WRITE_SIZE_KiB": round(readings[("WRITE_SIZE", "gqa")], 2),
+                                        "fetch_factor": round(f_fetch, 5), "write_factor": round(f_write, 5)}
+    except (subprocess.TimeoutExpired, OSError, KeyError, ValueError, ZeroDivisionError) as e:
+        log(f"traffic counters not read ({type(e).__name__}): the recorded constant is reported")
+        return None
+    finally:
+        shutil.rmtree(base, ignore_errors=True)
+
+
 def smoke_parity(lib):
     """Small invocation checked against the oracle; raises on mismatch."""
     import oracle
@@ -394,6 +440,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode-step", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-point tables of configurations 2-4")
+    ap.add_argument("--no-traffic-counters", action="store_true",
+                    help="do not read FETCH_SIZE / WRITE_SIZE through rocprofv3 child processes (report the recorded constant)")
     ap.add_argument("--decode-steps", type=int, default=128)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -449,6 +497,16 @@ def main():
                      "avg_launch_us": round(ev_ms * 1e3, 2), "algorithmic_bytes": wl.bytes_per_step},
     }
     del wl
+    if not args.no_traffic_counters:
+        # read here, before the decode model takes its memory: the child processes allocate 2 x 1 GiB themselves
+        t = measure_traffic(log)
+        if t is not None:
+            result["roofline"]["traffic"] = t[0]
+            result["roofline"]["traffic_source"] = {"how": "rocprofv3 --pmc in child processes of this run, scaled by a "
+                                                           "1 GiB copy kernel", **t[1]}
+            log(f"HBM traffic per launch by counters: {t[0]} B = {t[0] / result['roofline']['algorithmic_bytes']:.5f} x algorithmic")
+        else:
+            result["roofline"]["traffic_source"] = "recorded constant (profiles/gqa_decode_split_B32_L8192_f16.md)"
 
     if not args.no_decode_step:
         try:

@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Prints ONE JSON line.  The metric is BASELINE.json's: "GQA decode HBM GB/s (% of peak) B=32 L=8k
+Prints ONE JSON line.  The metric is the headline one of this build: "GQA decode HBM GB/s (% of peak) B=32 L=8k
 fp16; decode tok/s 2B-shape B=16".  `value` is the first half: achieved algorithmic GB/s of the
 split-K GQA decode attention at B=32, Hq=16, Hkv=8, D=128, L=8192, fp16 KV cache resident in HBM.
 A "step" is one pass of that operator over one batch (one launch: at this shape every sequence is one key
@@ -255,7 +255,8 @@ def _cpu_min_us(fn, budget_s=0.6, max_runs=50):
 
 
 def config_tables(lib, with_cpu=True):
-    """BASELINE's configurations 2, 3 and 4, every point timed with HIP events on the device (through the
+    """The benchmark configurations 2, 3 and 4 (fused elementwise operators at B = 32, the decode-attention sweep, the
+    fp16 Linear), every point timed with HIP events on the device (through the
     C ABI, buffers rotated so that nothing is served from the 256 MB memory-side cache) and, where it costs
     under about a second, the CPU restatement of the same operator on the same shape beside it."""
     from axono_amd.benchmarks import microbench as mb
@@ -360,7 +361,7 @@ def _compact(rows):
     return {"cols": cols, "rows": [[r.get(c) for c in cols] for r in rows]}
 
 
-def measure_traffic(log, timeout_s=90):
+def measure_traffic(log, timeout_s=60):
     """HBM bytes per launch of the headline kernel, read from the hardware counters in child processes: four short
     `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE, for the attention microbenchmark and for a plain copy
     kernel of 1 GiB each way, which gives each counter's scale factor).  Returns (bytes, details) or None when
@@ -383,10 +384,19 @@ def measure_traffic(log, timeout_s=90):
                 out = os.path.join(base, f"{counter}_{what}")
                 cmd = [exe, "--pmc", counter, "-d", out, "-o", "p", "--output-format", "csv", "--", sys.executable, "-m",
                        "axono_amd.benchmarks.microbench", what, "--steps", "3"]
-                r = subprocess.run(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
-                                   timeout=timeout_s)
+                # own process group: a run that outlives its time limit is ended together with its children
+                proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                                        start_new_session=True)
+                try:
+                    rc = proc.wait(timeout=timeout_s)
+                except subprocess.TimeoutExpired:
+                    import signal
+                    os.killpg(proc.pid, signal.SIGKILL)
+                    proc.wait()
+                    log("traffic counters: a profiler run exceeded its time limit; the recorded constant is reported")
+                    return None
                 files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
-                if r.returncode != 0 or not files:
+                if rc != 0 or not files:
                     return None
                 vals = [float(row["Counter_Value"]) for row in csv.DictReader(open(files[0]))
                         if kernel in row["Kernel_Name"] and row["Counter_Name"] == counter]
@@ -446,7 +456,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported "
-              "(the decode path shards by batch or kv-head with no exchange, see DESIGN.md)", file=sys.stderr)
+              "(the decode path shards by batch or kv-head with no exchange between devices)", file=sys.stderr)
         sys.exit(2)
 
     from axono_amd import _lib

@@ -529,7 +529,7 @@ def main():
 
     if not args.no_configs:
         result["configs"] = config_tables(lib, with_cpu=not args.no_cpu_baseline)
-        log(f"configs 2-4: {sum(len(v) for v in result['configs'].values() if isinstance(v, list))} points timed")
+        log(f"configs 2-4: {sum(len(v['rows']) for v in result['configs'].values() if isinstance(v, dict) and 'rows' in v)} points timed")
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_gqa()

@@ -948,6 +948,137 @@ __global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedAr
   }
 }
 
+// One workgroup per CU with eight wavefronts for the problems that give a CU only one tile of 64 TW weight
+// rows x 64 rows of x (M = 512 with N = 2048 or 4096).  The bytes a CU pulls through its vector memory path per
+// product fall with the tile's area, so the tile is the CU's whole share of the output; the second wavefront
+// per SIMD that hides the latency of a step then has to come from inside the workgroup: wavefronts 0-3 sum the
+// first half of K, wavefronts 4-7 the second half (each half with its own x double buffer in LDS and its own W
+// fragments, so no byte is fetched twice), and the halves are added through LDS at the end: out = S(first
+// half) + S(second half), each S accumulated in K order, the same for every launch.  fp16 x, K % 512 == 0.
+template <int TW>
+__global__ __launch_bounds__(512, 1) void linear_gemm_packed_khalves_kernel(PackedArgs a, int n_blocks, int m_blocks) {
+  constexpr int GM = 64, MT = GM / 16;
+  constexpr int XV = GM * 16 / 256;  // 16-byte x vectors per thread of a half and step
+  __shared__ __attribute__((aligned(16))) _Float16 xs[2][2][GM * kGK];  // [K half][buffer]: 64 KiB
+  const int tid = threadIdx.x, kh = tid >> 8, ht = tid & 255, wave = ht >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int id = blockIdx.x;
+  const int xcd = id % kXcds, slot = id / kXcds;
+  const int nb = (slot / m_blocks) * kXcds + xcd, mb = slot % m_blocks;
+  if (nb >= n_blocks) return;
+  const int n_tiles = (a.N + 15) / 16;
+  const int tile0 = (nb * 4 + wave) * TW;
+  const int m0 = mb * GM;
+  const __half *x = static_cast<const __half *>(a.x);
+  const int steps = a.KC / 8;    // steps of 128 K per half
+  const int step0 = kh * steps;  // first step of this half
+
+  const __half *wt[TW];
+#pragma unroll
+  for (int t = 0; t < TW; ++t)
+    wt[t] = a.wp + (static_cast<int64_t>(min(tile0 + t, n_tiles - 1)) * a.KC + step0 * 4) * 512 + lane * 8;
+  const __half *xp[XV];
+#pragma unroll
+  for (int p = 0; p < XV; ++p) {
+    const int v = p * 256 + ht;
+    xp[p] = x + static_cast<int64_t>(min(m0 + (v >> 4), a.M - 1)) * a.K + step0 * kGK + (v & 15) * 8;
+  }
+  auto load_x = [&](int step, half8_t (&xv)[XV]) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) xv[p] = load_h8(xp[p] + step * kGK);
+  };
+  auto store_x = [&](int buf, const half8_t (&xv)[XV]) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) {
+      const int v = p * 256 + ht;
+      const int row = v >> 4, unit = v & 15;
+      *reinterpret_cast<half8_t *>(&xs[kh][buf][row * kGK + ((unit ^ (row & 15)) * 8)]) = xv[p];
+    }
+  };
+
+  float4_t acc[TW][MT];
+#pragma unroll
+  for (int t = 0; t < TW; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  // W fragments wait two steps ahead of their products (a weight line comes from HBM, and a step of this
+  // tile is shorter than that trip); x, which every workgroup of a row block shares in L2, one step ahead.
+  // (Running the halves in opposite phases - one multiplies while the other fills LDS, two barriers per
+  // step - measured 3-5 % slower than letting them run side by side.)
+  half8_t wf[2][TW][4];  // [step parity][row tile][chunk]
+  half8_t xv[XV];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int t = 0; t < TW; ++t) wf[s][t][j] = load_h8(wt[t] + (s * 4 + j) * 512);
+  load_x(0, xv);
+  store_x(0, xv);
+  __syncthreads();
+
+  for (int i0 = 0; i0 < steps; i0 += 2) {  // steps is even
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int i = i0 + s;  // LDS buffer and fragment set s
+      // past the end the last step is fetched once more: no branch in the loop
+      load_x(min(i + 1, steps - 1), xv);
+      const int64_t w2 = static_cast<int64_t>(min(i + 2, steps - 1)) * 4 * 512;
+      __builtin_amdgcn_sched_barrier(0);
+      half8_t bf[2][MT];
+      auto load_bf = [&](int j, half8_t (&f)[MT]) {
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+          const int row = u * 16 + r, unit = j * 4 + g;
+          f[u] = *reinterpret_cast<const half8_t *>(&xs[kh][s][row * kGK + ((unit ^ (row & 15)) * 8)]);
+        }
+      };
+      load_bf(0, bf[0]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j + 1 < 4) load_bf(j + 1, bf[(j + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < TW; ++t)
+#pragma unroll
+          for (int u = 0; u < MT; ++u)
+            acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[s][t][j], bf[j & 1][u], acc[t][u], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < TW; ++t) wf[s][t][j] = load_h8(wt[t] + w2 + j * 512);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      store_x(s ^ 1, xv);
+      __syncthreads();
+    }
+  }
+
+  // the second half hands its sums over through LDS (every x fragment has been read: the loop ends on a barrier)
+  float4_t *red = reinterpret_cast<float4_t *>(&xs[0][0][0]);
+  if (kh == 1) {
+#pragma unroll
+    for (int t = 0; t < TW; ++t)
+#pragma unroll
+      for (int u = 0; u < MT; ++u) red[((wave * TW + t) * MT + u) * 64 + lane] = acc[t][u];
+  }
+  __syncthreads();
+  if (kh == 1) return;
+  LinearArgs o;
+  o.bias = a.bias;
+  o.out = a.out;
+  o.M = a.M;
+  o.N = a.N;
+  o.out_f16 = a.out_f16;
+#pragma unroll
+  for (int u = 0; u < MT; ++u)
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+      const float4_t s = acc[t][u] + red[((wave * TW + t) * MT + u) * 64 + lane];
+      const float v[4] = {s[0], s[1], s[2], s[3]};
+      if (tile0 + t < n_tiles) store_out4(o, m0 + u * 16 + r, (tile0 + t) * 16 + 4 * g, v);
+    }
+}
+
 // Weight rows per workgroup: 256 (four row tiles per wavefront), or 128 / 64 when 256 would leave CUs
 // without a workgroup (M = 512, N = 2048: 64 workgroups of 256 x 64, 256 of 64 x 64).
 int gemm_tiles_per_wave(const PackedArgs &a, int gm) {
@@ -996,6 +1127,28 @@ void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
       return;
     }
   }
+  if constexpr (sizeof(XT) == 2) {
+    // the CU's whole share of the output as one tile, K in two halves inside the workgroup
+    if (!a.glu && a.K % (4 * kGK) == 0 && (g_gemm_rows == 512 || (g_gemm_rows == 0 && g_gemm_tiles == 0))) {
+      const int64_t mb64 = (a.M + 63) / 64;
+      const int64_t t2 = static_cast<int64_t>((a.N + 127) / 128) * mb64, t1 = static_cast<int64_t>((a.N + 63) / 64) * mb64;
+      const int cus = device_cu_count();
+      int tw = 0;
+      if (g_gemm_rows == 512) tw = g_gemm_tiles == 2 ? 2 : 1;
+      else if (t2 <= cus && 2 * t2 > cus) tw = 2;
+      else if (t1 <= cus && 2 * t1 > cus) tw = 1;
+      if (tw) {
+        const int n_blocks = (a.N + 64 * tw - 1) / (64 * tw), m_blocks = static_cast<int>(mb64);
+        const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
+        const dim3 grid(static_cast<unsigned>(nb_pad) * m_blocks);
+        if (tw == 2)
+          hipLaunchKernelGGL((linear_gemm_packed_khalves_kernel<2>), grid, dim3(512), 0, st, a, n_blocks, m_blocks);
+        else
+          hipLaunchKernelGGL((linear_gemm_packed_khalves_kernel<1>), grid, dim3(512), 0, st, a, n_blocks, m_blocks);
+        return;
+      }
+    }
+  }
   int gm = (g_gemm_rows == 32 || g_gemm_rows == 64 || g_gemm_rows == 128) ? g_gemm_rows : 64;
   const int tw = gemm_tiles_per_wave(a, gm == 32 ? 64 : gm);
   // a problem that gives no CU a second workgroup even with the smallest weight tile is bounded by the
@@ -1038,7 +1191,7 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
   // gemm_rows: 64 or 128 rows of x per GEMM workgroup, plus 1000 t to force t = 1, 2, 4 row tiles of W per wavefront
   g_gemm_tiles = gemm_rows >= 1000 ? gemm_rows / 1000 : 0;
   gemm_rows %= 1000;
-  g_gemm_rows = (gemm_rows == 32 || gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256) ? gemm_rows : 0;
+  g_gemm_rows = (gemm_rows == 32 || gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256 || gemm_rows == 512) ? gemm_rows : 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : 0;
   g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;

@@ -186,7 +186,11 @@ def test_packed_gemm_256x128_tile(M, K, N):
     w = h16(0.02 * rng.standard_normal((N, K)))
     b = h16(0.05 * rng.standard_normal(N))
     l = gu.lib()
-    base = gu.linear_f16_packed(x, w, b)
+    l.axhip_linear_f16_tune(0, 0, 0, 64)
+    try:
+        base = gu.linear_f16_packed(x, w, b)
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
     l.axhip_linear_f16_tune(0, 0, 0, 256)
     try:
         out = gu.linear_f16_packed(x, w, b)
@@ -203,6 +207,39 @@ def test_packed_gemm_256x128_tile(M, K, N):
     gu_ = port.linear(x.astype(np.float32), w[:n2].astype(np.float32))
     wantg = port.silu_mul(np.ascontiguousarray(gu_[:, : n2 // 2]), np.ascontiguousarray(gu_[:, n2 // 2:]))
     np.testing.assert_allclose(glu, wantg, rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("tiles,M,K,N", [(1, 512, 2048, 2048), (1, 512, 6144, 2048), (2, 512, 2048, 4096), (1, 130, 512, 200),
+                                         (2, 333, 1024, 1000), (1, 65, 1536, 64)])
+def test_packed_gemm_k_in_two_halves(tiles, M, K, N):
+    """The tile for problems that give a CU one tile only (eight wavefronts, K summed in two halves that are
+    added at the end), forced on edge shapes and at its own sizes: against the oracle, fp16 output, twice the
+    same bits, and the halves really are S(first half) + S(second half) of the sequential kernel."""
+    rng = np.random.default_rng(M + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    b = h16(0.05 * rng.standard_normal(N))
+    l = gu.lib()
+    l.axhip_linear_f16_tune(0, 0, 0, 1000 * tiles + 512)
+    try:
+        out = gu.linear_f16_packed(x, w, b)
+        again = gu.linear_f16_packed(x, w, b)
+        out16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16)
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
+    np.testing.assert_array_equal(out, again)
+    want = port.linear(x.astype(np.float32), w.astype(np.float32), b.astype(np.float32))
+    mag = np.abs(x.astype(np.float32)) @ np.abs(w.astype(np.float32)).T
+    assert np.all(np.abs(out - want) <= 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag + 1e-3 * 2.0 ** -11)
+    assert np.abs(out16.astype(np.float32) - want).max() <= 2e-3 + 2.0 ** -11 * np.abs(want).max()
+    # the two halves, each from the sequential kernel (64-row tile), added in fp32 and then the bias
+    l.axhip_linear_f16_tune(0, 0, 0, 64)
+    try:
+        s0 = gu.linear_f16_packed(np.ascontiguousarray(x[:, : K // 2]), np.ascontiguousarray(w[:, : K // 2]))
+        s1 = gu.linear_f16_packed(np.ascontiguousarray(x[:, K // 2:]), np.ascontiguousarray(w[:, K // 2:]))
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
+    np.testing.assert_array_equal(out, (s0 + s1) + b.astype(np.float32))
 
 
 @pytest.mark.parametrize("seed", range(16))

@@ -252,8 +252,8 @@ class Qwen3VLTextDecoder(nn.Module):
 
     # ---- prefill -----------------------------------------------------------------------------
     def prefill(self, ids: np.ndarray, positions: np.ndarray | None = None):
-        """ids int64 [B, S] (host).  Fills the cache for every sequence (one sequence at a time, all
-        S tokens at once) and returns (last-position logits FLOAT32 [B,V] as a Tensor, next ids [B]).
+        """ids int64 [B, S] (host).  Fills the cache for every sequence (all S tokens of up to 65 536 / S
+        sequences per pass) and returns (last-position logits FLOAT32 [B,V] as a Tensor, next ids [B]).
         Text-only positions by default: T = H = W = token index."""
         cfg = self._cfg
         B, S = ids.shape
@@ -274,38 +274,47 @@ class Qwen3VLTextDecoder(nn.Module):
             self._cache.reserve(S)
             lmax = self._scratch_kv[0].shape[2]
             s_lens = _dev(np.full(B, S, np.int32), dev)
-        for b in range(B):
-            h = L.embedding(_dev(ids[b].astype(np.int64), dev), self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)
+        # several sequences per pass (their tokens are the rows of every GEMM and one attention launch covers
+        # them all): up to 65 536 tokens at a time; the paged cache fills one sequence's dense scratch block at a time
+        per_pass = 1 if self._paged else max(1, min(B, 65536 // max(S, 1)))
+        for b in range(0, B, per_pass):
+            nb = min(per_pass, B - b)
+            pos_c = pos_t if nb == 1 else _dev(np.ascontiguousarray(np.tile(positions, (1, nb)), dtype=np.int64), dev)
+            h = L.embedding(_dev(ids[b:b + nb].astype(np.int64).reshape(-1), dev),
+                            self._w("embed_tokens.weight")).cast_to(DataType.FLOAT32)
             xn = L.rms_norm(h, self._w("layers.0.input_layernorm.weight"), cfg.rms_norm_eps, DataType.FLOAT16)
             for i in range(cfg.num_hidden_layers):
                 p = f"layers.{i}."
-                qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")  # [S, width] fp32
+                qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")  # [nb*S, width] fp32
                 if self._paged:
                     kc, vc = self._scratch_kv   # this sequence's rows of this layer, dense; copied to its pages below
                     seq_off = 0
                 else:
                     kc, vc = self._cache.get(i)
                     seq_off = b * nkv * lmax * D * esz
-                q = Tensor(DataType.FLOAT16, [S, nq, D], dev, _zero=False)
+                q = Tensor(DataType.FLOAT16, [nb * S, nq, D], dev, _zero=False)
                 base = qkv.data_ptr
                 check(lib.axhip_qkv_norm_rope_append(
                     base, width, base + nq * D * 4, width, base + (nq + nkv) * D * 4, width,
                     self._w(p + "self_attn.q_norm.weight").data_ptr, self._w(p + "self_attn.k_norm.weight").data_ptr,
-                    int(DataType.FLOAT32), cfg.rms_norm_eps, pos_t.data_ptr, self._inv_freq.data_ptr,
+                    int(DataType.FLOAT32), cfg.rms_norm_eps, pos_c.data_ptr, self._inv_freq.data_ptr,
                     cfg.mrope_section[1], cfg.mrope_section[2], None, q.data_ptr, kc.data_ptr + seq_off,
-                    vc.data_ptr + seq_off, int(DataType.FLOAT16), 1, S, nq, nkv, D, lmax, current_stream()),
+                    vc.data_ptr + seq_off, int(DataType.FLOAT16), nb, S, nq, nkv, D, lmax, current_stream()),
                     "qkv_norm_rope_append")
-                attn = Tensor(DataType.FLOAT16, [S, nq * D], dev, _zero=False)
+                attn = Tensor(DataType.FLOAT16, [nb * S, nq * D], dev, _zero=False)
                 if D in (64, 128):
                     # causal attention over the rows just appended, on the matrix cores
                     check(lib.axhip_prefill_attention(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, None,
-                                                      attn.data_ptr, int(DataType.FLOAT16), 1, S, nq, nkv, D, lmax,
+                                                      attn.data_ptr, int(DataType.FLOAT16), nb, S, nq, nkv, D, lmax,
                                                       current_stream()), "prefill_attention")
                 else:
-                    # every query row is a "sequence" of the decode kernel over this sequence's cache rows
-                    check(lib.axhip_gqa_decode(q.data_ptr, kc.data_ptr + seq_off, vc.data_ptr + seq_off, vis.data_ptr,
-                                               attn.data_ptr, ws.data_ptr, ws.num_bytes, int(DataType.FLOAT16), S, nq,
-                                               nkv, D, S, 0, lmax * D, D, current_stream()), "gqa_decode")
+                    # every query row is a "sequence" of the decode kernel over its sequence's cache rows
+                    for j in range(nb):
+                        off = seq_off + j * nkv * lmax * D * esz
+                        check(lib.axhip_gqa_decode(q.data_ptr + j * S * nq * D * esz, kc.data_ptr + off, vc.data_ptr + off,
+                                                   vis.data_ptr, attn.data_ptr + j * S * nq * D * esz, ws.data_ptr,
+                                                   ws.num_bytes, int(DataType.FLOAT16), S, nq, nkv, D, S, 0, lmax * D, D,
+                                                   current_stream()), "gqa_decode")
                 if self._paged:
                     L.kv_dense_to_paged(kc, vc, *self._cache.get(i), self._cache.page_table, lens=s_lens, table_row=b)
                 attn_out = self._linear(attn, p + "self_attn.o_proj.weight")
@@ -314,8 +323,10 @@ class Qwen3VLTextDecoder(nn.Module):
                 mlp_out = self._mlp(xn2, p)
                 nxt = f"layers.{i + 1}.input_layernorm.weight" if i + 1 < cfg.num_hidden_layers else "norm.weight"
                 h, xn = L.add_rms_norm(mlp_out, h, self._w(nxt), cfg.rms_norm_eps, DataType.FLOAT16)
-            # keep the normalised hidden state of the last position for the lm_head
-            check(lib.axhip_memcpy_d2d(last_h.data_ptr + b * H * 2, xn.data_ptr + (S - 1) * H * 2, H * 2), "copy")
+            # keep the normalised hidden state of each sequence's last position for the lm_head
+            for j in range(nb):
+                check(lib.axhip_memcpy_d2d(last_h.data_ptr + (b + j) * H * 2, xn.data_ptr + (j * S + S - 1) * H * 2, H * 2),
+                      "copy")
         self._cache.set_lengths(np.full(B, S, np.int32))
         logits = self._linear(last_h, "embed_tokens.weight")
         return logits, L.argmax(logits)

@@ -27,7 +27,7 @@ constexpr int kMaxWaves = 16;   // wavefronts per workgroup of the skinny kernel
 
 struct LinearTuning {
   int target_waves = 0;     // wavefronts to aim for in the skinny kernel; 0 = 8 per compute unit of the device
-  int force_nt = 0;         // > 0: rows-of-16 per wavefront (1, 2 or 4)
+  int force_nt = 0;         // > 0: rows-of-16 per wavefront (1 to 4)
   int force_waves = 0;      // > 0: wavefronts (K slices) per workgroup (4, 8 or 16)
 };
 LinearTuning g_lin;
@@ -556,6 +556,8 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
   if (p.mt == 1) {
     if (p.nt == 4)
       dispatch_packed_waves<4, 1, XT>(a, p.waves, half, st);
+    else if (p.nt == 3)
+      dispatch_packed_waves<3, 1, XT>(a, p.waves, half, st);
     else if (p.nt == 2)
       dispatch_packed_waves<2, 1, XT>(a, p.waves, half, st);
     else
@@ -1193,7 +1195,7 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
   gemm_rows %= 1000;
   g_gemm_rows = (gemm_rows == 32 || gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256 || gemm_rows == 512) ? gemm_rows : 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : 0;
-  g_lin.force_nt = (force_nt == 1 || force_nt == 2 || force_nt == 4) ? force_nt : 0;
+  g_lin.force_nt = (force_nt >= 1 && force_nt <= 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;
 }
 

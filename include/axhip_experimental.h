@@ -22,7 +22,7 @@ extern "C" {
 AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
 
 /* fp16 Linear plans (0 restores a default).  Skinny M: wavefronts to aim for, 16-row groups of W per
- * wavefront (1, 2 or 4), wavefronts (K slices) per workgroup (4, 8, 16).  M > 32 GEMM, gemm_rows: 64 or 128
+ * wavefront (1 to 4), wavefronts (K slices) per workgroup (4, 8, 16).  M > 32 GEMM, gemm_rows: 64 or 128
  * rows of x per workgroup (128: one workgroup per CU), 256 = the 256 x 128 tile at two workgroups per CU
  * (the default for large problems), 512 = the eight-wavefront workgroup that sums K in two halves (fp16 x,
  * K % 512 == 0, otherwise ignored; with 1000 t: t = 1 or 2 row tiles), plus 1000 t to force t = 1, 2 or 4 row

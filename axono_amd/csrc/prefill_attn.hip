@@ -25,6 +25,8 @@
 // [0, 1]); the row sum is kept per lane and reduced once at the end.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace axhip {
 namespace {
 
@@ -145,6 +147,85 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
   store_stage(0, 0);
   __syncthreads();
 
+  // One block of 32 keys for this wavefront.  DIAG: some key of the block may lie behind a query of the
+  // wavefront (the block touches the diagonal, or the end of the cache); every other block skips the
+  // masks, which are a third of the softmax instructions.  The scale is folded into the exponent's
+  // argument: p = exp2(s * scale - m) with m the running maximum of s * scale.
+  auto block = [&](int buf, int sub, int kb, auto diag_c) __attribute__((always_inline)) {
+    constexpr bool DIAG = decltype(diag_c)::value;
+    const _Float16 *kst_l = &ks[buf][sub * 32 * D];
+    // ---- S^T = K . Q^T for two tiles of 16 keys ----
+    float4_t sc[G][2];
+#pragma unroll
+    for (int t = 0; t < G; ++t) sc[t][0] = sc[t][1] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const int row = tk * 16 + c, unit = kk * 4 + g;  // row & 15 == c
+        const half8_t kf = lds_h8(kst_l + row * D + ((unit ^ (c & (UPR - 1))) << 3));
+#pragma unroll
+        for (int t = 0; t < G; ++t)
+          sc[t][tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][kk], sc[t][tk], 0, 0, 0);
+      }
+    // ---- mask, online softmax ----
+    half8_t pf[G];
+#pragma unroll
+    for (int t = 0; t < G; ++t) {
+      float x[8];
+#pragma unroll
+      for (int tk = 0; tk < 2; ++tk)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = sc[t][tk][e];
+          if constexpr (DIAG) {
+            const int key = kb + tk * 16 + 4 * g + e;
+            if (key > pos) v = kMasked;
+          }
+          x[tk * 4 + e] = v;
+        }
+      float mx = x[0];
+#pragma unroll
+      for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      // masked scores are -1e30 before the (positive) scale: they stay far below every real score
+      const float mn = fmaxf(m[t], mx * a.scale_log2e);
+      float ps = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(x[j], a.scale_log2e, -mn));
+        if constexpr (DIAG) {
+          // a fully masked row keeps m == kMasked * scale: exp2(0) would count
+          if (x[j] <= kMasked) p = 0.f;
+        }
+        ps += p;
+        pf[t][j] = static_cast<_Float16>(p);
+      }
+      // once the running maxima have settled, most blocks change none of them: the rescale of the
+      // 4 DT output registers is skipped when no query of the wavefront needs it
+      if (__any(mn != m[t])) {
+        const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
+        lsum[t] *= corr;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
+      }
+      m[t] = mn;
+      lsum[t] += ps;
+    }
+    // ---- O^T += V^T . P^T ----
+    const _Float16 *vst_l = &vs[buf][sub * 32 * D];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const half4_t lo = lds_v_tr<D>(vst_l, 4 * g, dt * 16, c);
+      const half4_t hi = lds_v_tr<D>(vst_l, 16 + 4 * g, dt * 16, c);
+      const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+      for (int t = 0; t < G; ++t)
+        o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][dt], 0, 0, 0);
+    }
+  };
+
   for (int s = 0; s < n_stages; ++s) {
     const int buf = s & 1;
     const int nxt = min(s + 1, n_stages - 1);  // the last stage fetches itself again: no branch
@@ -154,73 +235,10 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
     for (int sub = 0; sub < kStageKeys / 32; ++sub) {
       const int kb = s * kStageKeys + sub * 32;      // first key of this block of 32
       if (kb <= wave_last && kb < k_end) {           // wave-uniform: otherwise every key is masked
-        const _Float16 *kst_l = &ks[buf][sub * 32 * D];
-        // ---- S^T = K . Q^T for two tiles of 16 keys ----
-        float4_t sc[G][2];
-#pragma unroll
-        for (int t = 0; t < G; ++t) sc[t][0] = sc[t][1] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int tk = 0; tk < 2; ++tk)
-#pragma unroll
-          for (int kk = 0; kk < KK; ++kk) {
-            const int row = tk * 16 + c, unit = kk * 4 + g;  // row & 15 == c
-            const half8_t kf = lds_h8(kst_l + row * D + ((unit ^ (c & (UPR - 1))) << 3));
-#pragma unroll
-            for (int t = 0; t < G; ++t)
-              sc[t][tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][kk], sc[t][tk], 0, 0, 0);
-          }
-        // ---- mask, online softmax ----
-        const bool diag = kb + 31 > wave_first;  // some key of the block may be masked
-        half8_t pf[G];
-#pragma unroll
-        for (int t = 0; t < G; ++t) {
-          float x[8];
-#pragma unroll
-          for (int tk = 0; tk < 2; ++tk)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int key = kb + tk * 16 + 4 * g + e;
-              float v = sc[t][tk][e] * a.scale_log2e;
-              if (diag && key > pos) v = kMasked;
-              x[tk * 4 + e] = v;
-            }
-          float mx = x[0];
-#pragma unroll
-          for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
-          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-          const float mn = fmaxf(m[t], mx);
-          float ps = 0.f;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            float p = __builtin_amdgcn_exp2f(x[j] - mn);
-            // a fully masked row keeps m == kMasked: exp2(0) would count (masks occur in diagonal blocks only)
-            if (diag && x[j] <= kMasked) p = 0.f;
-            ps += p;
-            pf[t][j] = static_cast<_Float16>(p);
-          }
-          // once the running maxima have settled, most blocks change none of them: the rescale of the
-          // 4 DT output registers is skipped when no query of the wavefront needs it
-          if (__any(mn != m[t])) {
-            const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
-            lsum[t] *= corr;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
-          }
-          m[t] = mn;
-          lsum[t] += ps;
-        }
-        // ---- O^T += V^T . P^T ----
-        const _Float16 *vst_l = &vs[buf][sub * 32 * D];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const half4_t lo = lds_v_tr<D>(vst_l, 4 * g, dt * 16, c);
-          const half4_t hi = lds_v_tr<D>(vst_l, 16 + 4 * g, dt * 16, c);
-          const half8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-          for (int t = 0; t < G; ++t)
-            o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][dt], 0, 0, 0);
-        }
+        if (kb + 31 > wave_first)                    // wave-uniform too
+          block(buf, sub, kb, std::true_type{});
+        else
+          block(buf, sub, kb, std::false_type{});
       }
     }
     __builtin_amdgcn_sched_barrier(0);

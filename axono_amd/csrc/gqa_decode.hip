@@ -790,13 +790,14 @@ constexpr int kMfmaHeads = 16;   // columns of the MFMA tile: heads per workgrou
 // one more step after the cached keys, and writes the cache row.
 extern __shared__ __attribute__((aligned(16))) unsigned char mfma_smem[];
 
-template <int D>
+template <int D, bool PAGED = false>
 constexpr int mfma_lds_bytes() {
-  // one stage of K and of V (the per-wavefront states reuse it), two rows for a new token, the merge flag
-  return 2 * kMfmaStage * D * 2 + 2 * D * 2 + 16;
+  // one stage of K and of V (the per-wavefront states reuse it), two rows for a new token, the merge flag,
+  // and for a paged cache the page numbers of the workgroup's key range
+  return 2 * kMfmaStage * D * 2 + 2 * D * 2 + 16 + (PAGED ? (kMaxRangePages * 4 + 15) / 16 * 16 : 0);
 }
 
-template <int D, bool QKV>
+template <int D, bool QKV, bool PAGED = false>
 __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, int hg, int split, int n_valid,
                                                    bool direct_ok, int s0, int s1) {
   constexpr int KK = D / 32;   // MFMA steps over d for S^T
@@ -824,8 +825,25 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
     mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
     if (mine) kv_end = p_new;
   }
-  const __half *kbase = static_cast<const __half *>(a.k) + b * a.stride_b + hk * a.stride_h;
-  const __half *vbase = static_cast<const __half *>(a.v) + b * a.stride_b + hk * a.stride_h;
+  // paged: the pool is [page, kv head, key in page, D]; the page numbers of keys [s0, s1) come from the page
+  // table into LDS first (clamped into the pool: a corrupt table gives wrong values, never an access outside it)
+  const int64_t kv_off = PAGED ? static_cast<int64_t>(hk) * (kPageKeys * D) : b * a.stride_b + hk * a.stride_h;
+  const __half *kbase = static_cast<const __half *>(a.k) + kv_off;
+  const __half *vbase = static_cast<const __half *>(a.v) + kv_off;
+  int *s_pages = reinterpret_cast<int *>(smem + 2 * kStageHalves * 2 + 2 * D * 2 + 16);
+  const int first_page = s0 >> kPageShift;
+  if constexpr (PAGED) {
+    const int range_pages = ((s1 - 1) >> kPageShift) - first_page + 1;
+    const int32_t *tbl = a.page_table + static_cast<int64_t>(b) * a.max_pages + first_page;
+    for (int i = tid; i < range_pages; i += kThreads) s_pages[i] = min(max(tbl[i], 0), a.n_pages - 1);
+    __syncthreads();
+  }
+  auto row_offset = [&](int key) -> int64_t {
+    if constexpr (PAGED)
+      return s_pages[(key >> kPageShift) - first_page] * a.page_stride + static_cast<int64_t>(key & (kPageKeys - 1)) * D;
+    else
+      return static_cast<int64_t>(key) * a.stride_s;
+  };
   // one stage waits in registers while the previous one is used from LDS.  (Two stages in registers
   // measured no faster: at 255 registers the compiler parks loaded data in accumulator registers, which
   // makes it wait for the loads early.  Per stage the kernel takes about 0.35 us more than its bytes do.)
@@ -835,7 +853,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
     for (int p = 0; p < VEC; ++p) {
       const int vi = p * kThreads + tid;
       const int row = vi / UPR, unit = vi % UPR;
-      const int64_t off = static_cast<int64_t>(min(key0 + row, kv_end - 1)) * a.stride_s + unit * 8;  // rows past the range: its last key again
+      const int64_t off = row_offset(min(key0 + row, kv_end - 1)) + unit * 8;  // rows past the range: its last key again
       kr[p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(kbase + off));
       vr[p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(vbase + off));
     }
@@ -873,8 +891,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
         norm_rope_row<__half, D>(a, a.pq + b * a.pq_stride + static_cast<int64_t>(h0 + job) * D, a.qw, b, a.B, lane,
                                  reinterpret_cast<__half *>(s_q + job * D), static_cast<__half *>(nullptr));
       } else {
-        __half *crow = const_cast<__half *>(static_cast<const __half *>(job == heads ? a.k : a.v)) + b * a.stride_b +
-                       hk * a.stride_h + static_cast<int64_t>(p_new) * a.stride_s;
+        __half *crow = const_cast<__half *>(static_cast<const __half *>(job == heads ? a.k : a.v)) + kv_off + row_offset(p_new);
         if (job == heads) {
           norm_rope_row<__half, D>(a, a.pk + b * a.pk_stride + static_cast<int64_t>(hk) * D, a.kw, b, a.B, lane,
                                    reinterpret_cast<__half *>(s_new), writer ? crow : static_cast<__half *>(nullptr));
@@ -1020,7 +1037,6 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
 //       zeros from the slot that holds its place on the line.
 template <typename T, int D, int G, int U, bool QKV, bool MFMA = false, bool PAGED = false>
 __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kernel(DecodeArgs a) {
-  static_assert(!(MFMA && PAGED), "paged caches run on the vector path");
   // the piece to work on: keys [s0, s1) of sequence b, range `split` of its n_valid ranges
   int b, hg, split, n_valid, s0, s1;
   bool direct_ok = true;
@@ -1084,8 +1100,8 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
         const int first_slot = start_b / cc, last_slot = (start_b + len_b - 1) / cc;
         if (again) __syncthreads();  // the previous piece is done with the LDS arrays
         if constexpr (MFMA)
-          process_range_mfma<D, QKV>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true, max(g0 - start_b, 0),
-                                min(g1 - start_b, len_b));
+          process_range_mfma<D, QKV, PAGED>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
+                                            max(g0 - start_b, 0), min(g1 - start_b, len_b));
         else
           process_range<T, D, G, U, QKV, false, PAGED>(a, b, hg, j - first_slot, last_slot - first_slot + 1, true,
                                                        max(g0 - start_b, 0), min(g1 - start_b, len_b));
@@ -1115,7 +1131,7 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
     }
   }
   if constexpr (MFMA)
-    process_range_mfma<D, QKV>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+    process_range_mfma<D, QKV, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1);
   else
     process_range<T, D, G, U, QKV, true, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1);
 }
@@ -1167,12 +1183,12 @@ int launch_decode(const DecodeArgs &a, int B, hipStream_t st) {
   return launch_status();
 }
 
-template <int D, bool QKV>
+template <int D, bool QKV, bool PAGED>
 int launch_decode_mfma_form(const DecodeArgs &a, int B, hipStream_t st) {
   const int n_hg = a.n_hg;
   const dim3 grid(a.dynamic ? a.active * n_hg : a.n_splits, a.dynamic ? 1 : n_hg, a.dynamic ? 1 : B);
-  auto kernel = gqa_decode_split_kernel<__half, D, 1, 8, QKV, true>;
-  constexpr int lds = mfma_lds_bytes<D>();
+  auto kernel = gqa_decode_split_kernel<__half, D, 1, 8, QKV, true, PAGED>;
+  constexpr int lds = mfma_lds_bytes<D, PAGED>();
   if (lds > 64 * 1024) {  // more dynamic LDS than the default limit
     static std::atomic<uint64_t> lds_set{0};
     const int rc = raise_dynamic_lds(reinterpret_cast<const void *>(kernel), lds, lds_set);
@@ -1186,7 +1202,9 @@ int launch_decode_mfma_form(const DecodeArgs &a, int B, hipStream_t st) {
 
 template <int D>
 int launch_decode_mfma(const DecodeArgs &a, int B, hipStream_t st) {
-  return a.len_add ? launch_decode_mfma_form<D, true>(a, B, st) : launch_decode_mfma_form<D, false>(a, B, st);
+  if (a.page_table)
+    return a.len_add ? launch_decode_mfma_form<D, true, true>(a, B, st) : launch_decode_mfma_form<D, false, true>(a, B, st);
+  return a.len_add ? launch_decode_mfma_form<D, true, false>(a, B, st) : launch_decode_mfma_form<D, false, false>(a, B, st);
 }
 
 template <typename T, int D>
@@ -1249,7 +1267,7 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
                     int D, int max_len, axhip_stream stream, bool static_ws = false) {
   const int group = Hq / Hkv;
   // four or more heads per kv head, fp16: the heads of a kv head become the columns of an MFMA tile
-  const bool mfma = !a.page_table && g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) &&
+  const bool mfma = g_tuning.mfma_groups && dtype == AXHIP_FLOAT16 && group >= 4 && (D == 64 || D == 128) &&
                     a.stride_s % 8 == 0 && a.stride_h % 8 == 0 && a.stride_b % 8 == 0;
   const int G = mfma ? mfma_heads_per_workgroup(group) : heads_per_workgroup(group);
   a.wg_heads = G;

@@ -620,10 +620,55 @@ def test_paged_cache_has_the_bits_of_the_dense_cache(dtype, hq, hkv, d):
         l.axhip_gqa_decode_tune(0, 0)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (16, 4, 128), (8, 1, 64), (32, 2, 128)])
+def test_decode_step_form_over_pages_has_the_bits_of_the_dense_cache(Hq, Hkv, D):
+    """axhip_gqa_decode_qkv_paged against axhip_gqa_decode_qkv on the same keys (two query heads per kv head: the
+    vector kernel; four and more: the matrix-core kernel): same output bits, the new token's row lands in its page
+    with the bits the dense cache gets, every other byte of the pools stays as it was."""
+    rng = np.random.default_rng(Hq * 1000 + Hkv * 10 + D)
+    lens = np.array([0, 1, 127, 128, 129, 700, 1279, 300], np.int32)
+    B, rows = len(lens), 1280
+    width = (Hq + 2 * Hkv) * D
+    qkv = rng.standard_normal((B, width)).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    pos = rng.integers(0, 8192, (3, B)).astype(np.int64)
+    inv = port.rope_inv_freq(1e6, D)
+    hw = 10 if D == 64 else 20
+    kc = (0.5 * rng.standard_normal((B, Hkv, rows, D))).astype(np.float16)
+    vc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
+    kp, vp, table, n_pages, max_pages = _paged_from_dense(kc, vc, lens + 1, 31)  # a page for the new row too
+    l = gu.lib()
+    dq, dqw, dkw, dp, di, dl = (gu.dev(a) for a in (qkv, qw, kw, pos, inv, lens))
+    dkc, dvc, dkp, dvp, dtb = (gu.dev(a) for a in (kc, vc, kp, vp, table))
+    out_d, out_p = gu.DeviceBuffer(B * Hq * D * 2), gu.DeviceBuffer(B * Hq * D * 2)
+    wsb = l.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, rows)
+    ws = gu.DeviceBuffer(max(wsb, 256))
+    common = (dq.ptr, width, dq.ptr + Hq * D * 4, width, dq.ptr + (Hq + Hkv) * D * 4, width, dqw.ptr, dkw.ptr, gu.F32,
+              1e-6, dp.ptr, di.ptr, hw, hw, dl.ptr)
+    gu._run("axhip_gqa_decode_qkv", *common, dkc.ptr, dvc.ptr, out_d.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows, rows,
+            None)
+    gu.synchronize()
+    gu._run("axhip_gqa_decode_qkv_paged", *common, dkp.ptr, dvp.ptr, dtb.ptr, out_p.ptr, ws.ptr, wsb, gu.F16, B, Hq, Hkv,
+            D, rows, max_pages, n_pages, None)
+    gu.synchronize()
+    np.testing.assert_array_equal(out_p.download(np.uint16, (B, Hq, D)), out_d.download(np.uint16, (B, Hq, D)))
+    gk, gv = dkc.download(np.float16, kc.shape), dvc.download(np.float16, vc.shape)
+    gkp, gvp = dkp.download(np.float16, kp.shape), dvp.download(np.float16, vp.shape)
+    touched = np.zeros(kp.shape, bool)
+    for b in range(B):
+        pid, r = int(table[b, lens[b] >> 7]), int(lens[b] & 127)
+        np.testing.assert_array_equal(gkp[pid, :, r].view(np.uint16), gk[b, :, lens[b]].view(np.uint16))
+        np.testing.assert_array_equal(gvp[pid, :, r].view(np.uint16), gv[b, :, lens[b]].view(np.uint16))
+        touched[pid, :, r] = True
+    np.testing.assert_array_equal(gkp[~touched].view(np.uint16), kp[~touched].view(np.uint16))
+    np.testing.assert_array_equal(gvp[~touched].view(np.uint16), vp[~touched].view(np.uint16))
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_paged_cache_random_configurations(seed):
     """Batch, head counts, head size, capacity, lengths (zeros included), dtype and page order at random: the paged
-    kernel against the oracle, and against the dense kernel bit for bit wherever both run on the vector ALUs."""
+    kernel against the oracle, and against the dense kernel bit for bit (vector kernel and matrix-core kernel)."""
     rng = np.random.default_rng(77000 + seed)
     B = int(rng.integers(1, 10))
     hkv = int(rng.integers(1, 4))
@@ -641,8 +686,7 @@ def test_paged_cache_random_configurations(seed):
     tol = TOL16 if dtype == np.float16 else TOL32
     assert np.abs(got - want).max() <= tol, (B, hkv, group, d, lmax, dtype, lens)
     assert np.all(got[lens == 0] == 0)
-    if not (group >= 4 and dtype == np.float16 and d <= 128):  # there the dense cache is read on the matrix cores
-        np.testing.assert_array_equal(got, gqa_decode(q, k, v, seq_lens=lens).astype(np.float32))
+    np.testing.assert_array_equal(got, gqa_decode(q, k, v, seq_lens=lens).astype(np.float32))
 
 
 def test_paged_cache_headline_shape_random_pages():

@@ -190,6 +190,41 @@ __device__ __forceinline__ float dpp_f32(float x) {
       float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
 }
 
+// Across the 16-lane rows of a wavefront: the value of lane l and that of lane l ^ 16 (l ^ 32), in an order
+// that depends on the lane - for sums, maxima and other symmetric operations.  One swap on the vector ALU
+// (v_permlane16_swap / v_permlane32_swap of gfx950: odd rows of the first operand change places with even
+// rows of the second, the upper half with the lower half) instead of a trip through the LDS crossbar.
+__device__ __forceinline__ void pair_xor16(unsigned x, unsigned &a, unsigned &b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  a = r[0];
+  b = r[1];
+}
+__device__ __forceinline__ void pair_xor32(unsigned x, unsigned &a, unsigned &b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  a = r[0];
+  b = r[1];
+}
+__device__ __forceinline__ float sum_xor16(float x) {
+  unsigned a, b;
+  pair_xor16(__builtin_bit_cast(unsigned, x), a, b);
+  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+__device__ __forceinline__ float sum_xor32(float x) {
+  unsigned a, b;
+  pair_xor32(__builtin_bit_cast(unsigned, x), a, b);
+  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
+__device__ __forceinline__ float max_xor16(float x) {
+  unsigned a, b;
+  pair_xor16(__builtin_bit_cast(unsigned, x), a, b);
+  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+__device__ __forceinline__ float max_xor32(float x) {
+  unsigned a, b;
+  pair_xor32(__builtin_bit_cast(unsigned, x), a, b);
+  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+
 // Sum over aligned groups of LANES consecutive lanes (LANES in {1,2,4,8,16,32,64}); every lane of a
 // group ends with the same bits because each step adds the same two partner values.
 template <int LANES>
@@ -198,8 +233,8 @@ __device__ __forceinline__ float group_sum(float x) {
   if constexpr (LANES >= 4) x += dpp_f32<0x4E>(x);   // quad_perm [2,3,0,1]
   if constexpr (LANES >= 8) x += dpp_f32<0x141>(x);  // row_half_mirror
   if constexpr (LANES >= 16) x += dpp_f32<0x140>(x); // row_mirror
-  if constexpr (LANES >= 32) x += __shfl_xor(x, 16, 64);
-  if constexpr (LANES >= 64) x += __shfl_xor(x, 32, 64);
+  if constexpr (LANES >= 32) x = sum_xor16(x);
+  if constexpr (LANES >= 64) x = sum_xor32(x);
   return x;
 }
 
@@ -209,9 +244,47 @@ __device__ __forceinline__ float group_max(float x) {
   if constexpr (LANES >= 4) x = fmaxf(x, dpp_f32<0x4E>(x));
   if constexpr (LANES >= 8) x = fmaxf(x, dpp_f32<0x141>(x));
   if constexpr (LANES >= 16) x = fmaxf(x, dpp_f32<0x140>(x));
-  if constexpr (LANES >= 32) x = fmaxf(x, __shfl_xor(x, 16, 64));
-  if constexpr (LANES >= 64) x = fmaxf(x, __shfl_xor(x, 32, 64));
+  if constexpr (LANES >= 32) x = max_xor16(x);
+  if constexpr (LANES >= 64) x = max_xor32(x);
   return x;
+}
+
+// The same for integers over the whole wavefront, and an inclusive prefix sum over its lanes (shifts within a
+// row, then the last lane of a row broadcast into the rows after it): a handful of vector instructions each.
+template <int CTRL, int ROW_MASK = 0xF, bool ZERO_FILL = true>
+__device__ __forceinline__ int dpp_i32(int x) {
+  return __builtin_amdgcn_update_dpp(0, x, CTRL, ROW_MASK, 0xF, ZERO_FILL);
+}
+__device__ __forceinline__ int wave_sum_i32(int v) {
+  v += dpp_i32<0xB1>(v);
+  v += dpp_i32<0x4E>(v);
+  v += dpp_i32<0x141>(v);
+  v += dpp_i32<0x140>(v);
+  unsigned a, b;
+  pair_xor16(static_cast<unsigned>(v), a, b);
+  v = static_cast<int>(a + b);
+  pair_xor32(static_cast<unsigned>(v), a, b);
+  return static_cast<int>(a + b);
+}
+__device__ __forceinline__ int wave_max_i32(int v) {
+  v = max(v, dpp_i32<0xB1>(v));
+  v = max(v, dpp_i32<0x4E>(v));
+  v = max(v, dpp_i32<0x141>(v));
+  v = max(v, dpp_i32<0x140>(v));
+  unsigned a, b;
+  pair_xor16(static_cast<unsigned>(v), a, b);
+  v = max(static_cast<int>(a), static_cast<int>(b));
+  pair_xor32(static_cast<unsigned>(v), a, b);
+  return max(static_cast<int>(a), static_cast<int>(b));
+}
+__device__ __forceinline__ int wave_prefix_i32(int v) {
+  v += dpp_i32<0x111>(v);  // row_shr:1 (lanes without a source add 0)
+  v += dpp_i32<0x112>(v);  // row_shr:2
+  v += dpp_i32<0x114>(v);  // row_shr:4
+  v += dpp_i32<0x118>(v);  // row_shr:8
+  v += dpp_i32<0x142, 0xA, false>(v);  // row_bcast:15 into rows 1 and 3: the total of the row before
+  v += dpp_i32<0x143, 0xC, false>(v);  // row_bcast:31 into rows 2 and 3: the total of rows 0 and 1
+  return v;
 }
 
 // Block-wide sum for blocks of NWAVES wavefronts; `smem` holds NWAVES floats.

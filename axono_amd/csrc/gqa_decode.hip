@@ -284,24 +284,9 @@ __device__ __forceinline__ int dyn_splits_of(int len, int c, int stride) {
   const int n = len > 0 ? (len + c - 1) / c : 1;
   return n < stride ? n : stride;
 }
-__device__ __forceinline__ int wave_sum_i(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
-__device__ __forceinline__ int wave_max_i(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
-  return v;
-}
-__device__ __forceinline__ int wave_prefix_i(int v, int lane) {  // inclusive prefix sum over the lanes
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const int up = __shfl_up(v, off, 64);
-    if (lane >= off) v += up;
-  }
-  return v;
-}
+__device__ __forceinline__ int wave_sum_i(int v) { return wave_sum_i32(v); }
+__device__ __forceinline__ int wave_max_i(int v) { return wave_max_i32(v); }
+__device__ __forceinline__ int wave_prefix_i(int v, int) { return wave_prefix_i32(v); }  // inclusive, over the lanes
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // One head row of the qkv projection -> RMSNorm over the head (weights optional) -> interleaved
@@ -945,8 +930,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
     float mx = x[0];
 #pragma unroll
     for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_xor32(max_xor16(mx));
     const float mn = fmaxf(m, mx);
     half8_t pf;
     float ps = 0.f;
@@ -1005,8 +989,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
   // the four per-wavefront states, [head][wavefront]: maximum, sum, output
   float *s_m = reinterpret_cast<float *>(smem), *s_l = s_m + kMfmaHeads * 4, *s_acc = s_l + kMfmaHeads * 4;
   int *s_flag = reinterpret_cast<int *>(smem + 2 * kStageHalves * 2 + 2 * D * 2);
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
+  lsum = sum_xor32(sum_xor16(lsum));
   if (g == 0) {
     s_m[c * 4 + wave] = m;
     s_l[c * 4 + wave] = lsum;
@@ -1080,7 +1063,7 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
     const bool end_to_end = a.active <= a.split_stride && total64 < (1 << 24) && longest - c_even > slack;
     if (end_to_end) {
       const int start = wave_prefix_i(len, lane) - len;  // where this lane's sequence begins on the line
-      const int total = uni(__shfl(start + len, 63, 64));
+      const int total = __builtin_amdgcn_readlane(start + len, 63);
       int cc = (total + a.active - 1) / a.active;
       cc = cc < kMinDevChunk ? kMinDevChunk : cc;
       cc = (cc + 15) & ~15;
@@ -1118,9 +1101,9 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kerne
     if (hit == 0ull) return;  // a slot the lengths of this launch leave unused
     // the same in every lane: say so, so that everything derived from it lives in scalar registers
     b = uni(__ffsll(hit) - 1);
-    split = uni(j - __shfl(first, b, 64));
-    const int n_b = uni(__shfl(n, b, 64));
-    const int len_b = uni(__shfl(len, b, 64));
+    split = j - __builtin_amdgcn_readlane(first, b);
+    const int n_b = __builtin_amdgcn_readlane(n, b);
+    const int len_b = __builtin_amdgcn_readlane(len, b);
     const int chunk = balanced_chunk(len_b, n_b);
     n_valid = (len_b + chunk - 1) / chunk;
     s0 = split * chunk;

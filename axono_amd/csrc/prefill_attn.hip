@@ -187,8 +187,7 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
       float mx = x[0];
 #pragma unroll
       for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_xor32(max_xor16(mx));
       // masked scores are -1e30 before the (positive) scale: they stay far below every real score
       const float mn = fmaxf(m[t], mx * a.scale_log2e);
       float ps = 0.f;
@@ -251,8 +250,7 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
 #pragma unroll
   for (int t = 0; t < G; ++t) {
     float l = lsum[t];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = sum_xor32(sum_xor16(l));
     const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {

@@ -107,28 +107,56 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
   const __half *kbase = a.k + kv_off;
   const __half *vbase = a.v + kv_off;
   half8_t kst[VEC], vst[VEC];
-  auto load_stage = [&](int key0) {
+  // A thread's VEC vectors of a stage: row and 16-byte unit are the same in every stage, so their element
+  // offsets and LDS positions are computed once; the stage's first row is the same for the whole workgroup and
+  // goes into the scalar base address.  Only a stage that reaches past the cache clamps rows, only a stage
+  // that reaches past the last visible key zeroes V rows (both tests are uniform).
+  unsigned voff[VEC];
+  int lds_o[VEC], vrow[VEC];
 #pragma unroll
-    for (int p = 0; p < VEC; ++p) {
-      const int vi = p * kPThreads + tid;
-      const int row = vi / UPR, unit = vi % UPR;
-      const int64_t off = static_cast<int64_t>(min(key0 + row, a.rows - 1)) * row_stride + unit * 8;
-      kst[p] = *reinterpret_cast<const half8_t *>(kbase + off);
-      vst[p] = *reinterpret_cast<const half8_t *>(vbase + off);
+  for (int p = 0; p < VEC; ++p) {
+    const int vi = p * kPThreads + tid;
+    const int row = vi / UPR, unit = vi % UPR;
+    vrow[p] = row;
+    voff[p] = static_cast<unsigned>(row) * static_cast<unsigned>(row_stride) + unit * 8;
+    lds_o[p] = row * D + ((unit ^ (row & (UPR - 1))) << 3);
+  }
+  auto load_stage = [&](int key0) {
+    if (key0 + kStageKeys <= a.rows) {
+      const __half *kb = kbase + static_cast<int64_t>(key0) * row_stride;
+      const __half *vb = vbase + static_cast<int64_t>(key0) * row_stride;
+#pragma unroll
+      for (int p = 0; p < VEC; ++p) {
+        kst[p] = *reinterpret_cast<const half8_t *>(kb + voff[p]);
+        vst[p] = *reinterpret_cast<const half8_t *>(vb + voff[p]);
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < VEC; ++p) {
+        const int unit = (p * kPThreads + tid) % UPR;
+        const int64_t off = static_cast<int64_t>(min(key0 + vrow[p], a.rows - 1)) * row_stride + unit * 8;
+        kst[p] = *reinterpret_cast<const half8_t *>(kbase + off);
+        vst[p] = *reinterpret_cast<const half8_t *>(vbase + off);
+      }
     }
   };
   // V rows past the last key any query of this workgroup may see are stored as zeros: their
   // probabilities are zero, but 0 * (whatever bits the unwritten cache holds) must stay 0
   auto store_stage = [&](int buf, int key0) {
+    if (key0 + kStageKeys <= k_end) {
 #pragma unroll
-    for (int p = 0; p < VEC; ++p) {
-      const int vi = p * kPThreads + tid;
-      const int row = vi / UPR, unit = vi % UPR;
-      const int o = row * D + ((unit ^ (row & (UPR - 1))) << 3);
-      *reinterpret_cast<half8_t *>(&ks[buf][o]) = kst[p];
-      half8_t vv = vst[p];
-      if (key0 + row >= k_end) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      *reinterpret_cast<half8_t *>(&vs[buf][o]) = vv;
+      for (int p = 0; p < VEC; ++p) {
+        *reinterpret_cast<half8_t *>(&ks[buf][lds_o[p]]) = kst[p];
+        *reinterpret_cast<half8_t *>(&vs[buf][lds_o[p]]) = vst[p];
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < VEC; ++p) {
+        *reinterpret_cast<half8_t *>(&ks[buf][lds_o[p]]) = kst[p];
+        half8_t vv = vst[p];
+        if (key0 + vrow[p] >= k_end) vv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        *reinterpret_cast<half8_t *>(&vs[buf][lds_o[p]]) = vv;
+      }
     }
   };
 
@@ -188,8 +216,14 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
 #pragma unroll
       for (int j = 1; j < 8; ++j) mx = fmaxf(mx, x[j]);
       mx = max_xor32(max_xor16(mx));
-      // masked scores are -1e30 before the (positive) scale: they stay far below every real score
-      const float mn = fmaxf(m[t], mx * a.scale_log2e);
+      // masked scores are -1e30 before the (positive) scale: they stay far below every real score.
+      // The running maximum moves only when a block exceeds it by more than 8 (a factor 256): until then
+      // the exponents stay <= 8, p <= 256 keeps its 11 bits in fp16 whatever its magnitude, and the block
+      // rescales nothing - with a maximum that follows every block, most blocks of a row's first few
+      // hundred keys pay 4 DT multiplications per query tile.
+      const float mxs = mx * a.scale_log2e;
+      const bool moved = __any(mxs > m[t] + 8.0f);
+      const float mn = moved ? fmaxf(m[t], mxs) : m[t];
       float ps = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -201,15 +235,13 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
         ps += p;
         pf[t][j] = static_cast<_Float16>(p);
       }
-      // once the running maxima have settled, most blocks change none of them: the rescale of the
-      // 4 DT output registers is skipped when no query of the wavefront needs it
-      if (__any(mn != m[t])) {
+      if (moved) {
         const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
         lsum[t] *= corr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
+        m[t] = mn;
       }
-      m[t] = mn;
       lsum[t] += ps;
     }
     // ---- O^T += V^T . P^T ----

@@ -2,7 +2,7 @@
 // already written to the static KV cache [B, Hkv, rows, D] (fp16), query i of sequence b sitting at
 // absolute position start[b] + i and seeing keys 0 .. start[b] + i.
 //
-// Work decomposition.  One workgroup (4 wavefronts) owns 64 consecutive positions of one sequence
+// Work decomposition.  One workgroup (4 or 8 wavefronts) owns 64 or 128 consecutive positions of one sequence
 // and the G query heads of one kv-head group; a wavefront owns 16 of those positions for all G
 // heads, i.e. G "query tiles" of 16 rows that share every K and V fragment it reads.  K and V
 // travel through LDS in stages of 64 keys (double-buffered, 16-byte units XOR-swizzled by key so
@@ -30,8 +30,6 @@
 namespace axhip {
 namespace {
 
-constexpr int kPThreads = 256;
-constexpr int kPosPerWg = 64;   // query positions per workgroup (16 per wavefront)
 constexpr int kStageKeys = 64;  // keys per LDS stage
 constexpr float kMasked = -1.0e30f;
 
@@ -57,8 +55,14 @@ struct PrefillArgs {
 // GEN = false is the cache form: K/V rows of a head are contiguous, the rule is causal and every query's
 // position lies inside the cache.  GEN = true takes any row/head/batch stride (token-major K/V), an
 // optional causal rule, and queries whose position is past the last key (they see every key).
-template <int D, int G, bool GEN>
-__global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel(PrefillArgs a) {
+// WAVES = 4: 64 positions per workgroup, two workgroups per CU (one's prologue and tail overlap the other's
+// blocks: best when a launch runs many workgroups per CU one after the other).  WAVES = 8: 128 positions, one
+// workgroup per CU, every K/V stage fetched and written to LDS once for eight wavefronts instead of four (best
+// when every workgroup has a long row of stages, or the launch is a single round of workgroups).
+template <int D, int G, bool GEN, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void prefill_attn_kernel(PrefillArgs a) {
+  constexpr int kPThreads = WAVES * 64;
+  constexpr int kPosPerWg = WAVES * 16;  // query positions per workgroup (16 per wavefront)
   constexpr int KK = D / 32;   // MFMA steps over d for S^T
   constexpr int DT = D / 16;   // d tiles of O^T
   constexpr int UPR = D / 8;   // 16-byte units per K/V row
@@ -298,11 +302,21 @@ __global__ __launch_bounds__(kPThreads, G <= 2 ? 2 : 1) void prefill_attn_kernel
 
 template <int D, bool GEN>
 int launch_prefill(const PrefillArgs &a, int B, int G, hipStream_t st) {
-  const dim3 grid((a.S + kPosPerWg - 1) / kPosPerWg, a.Hq / G, B);
+  // eight wavefronts per workgroup where every workgroup has all keys to go through (no causal rule), or where
+  // the launch is one round of workgroups anyway; G = 4 keeps four (its registers leave no room for eight)
+  const int64_t wgs8 = static_cast<int64_t>((a.S + 127) / 128) * (a.Hq / G) * B;
+  const bool eight = G <= 2 && ((GEN && !a.causal) || wgs8 <= device_cu_count());
+  const int pos = eight ? 128 : 64;
+  const dim3 grid((a.S + pos - 1) / pos, a.Hq / G, B);
+  if (eight) {
+    if (G == 2) hipLaunchKernelGGL((prefill_attn_kernel<D, 2, GEN, 8>), grid, dim3(512), 0, st, a);
+    else hipLaunchKernelGGL((prefill_attn_kernel<D, 1, GEN, 8>), grid, dim3(512), 0, st, a);
+    return launch_status();
+  }
   switch (G) {
-    case 4: hipLaunchKernelGGL((prefill_attn_kernel<D, 4, GEN>), grid, dim3(kPThreads), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((prefill_attn_kernel<D, 2, GEN>), grid, dim3(kPThreads), 0, st, a); break;
-    default: hipLaunchKernelGGL((prefill_attn_kernel<D, 1, GEN>), grid, dim3(kPThreads), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((prefill_attn_kernel<D, 4, GEN, 4>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((prefill_attn_kernel<D, 2, GEN, 4>), grid, dim3(256), 0, st, a); break;
+    default: hipLaunchKernelGGL((prefill_attn_kernel<D, 1, GEN, 4>), grid, dim3(256), 0, st, a); break;
   }
   return launch_status();
 }

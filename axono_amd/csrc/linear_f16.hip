@@ -142,6 +142,23 @@ __device__ __forceinline__ void store_out4(const LinearArgs &a, int m, int n, co
   }
 }
 
+// Gated epilogue of one 16-row tile that holds 8 gate rows (rows 0-7 of the tile) and their 8 up rows (rows
+// 8-15).  A lane owns rows 4g .. 4g+3 of the tile for x row m: the lower half of the wavefront (g = 0, 1) has
+// gate rows, fetches the up rows of the same columns from lane + 32 and stores silu(gate) * up for output
+// columns 8 tile + 4g ..; the upper half stores nothing.  `o.N` is the number of output columns (N / 2).
+__device__ __forceinline__ void store_glu_tile(const LinearArgs &o, int m, int tile, int g, const float4_t &acc) {
+  float v[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float own = acc[q];  // (a copy: bit-casting the vector element itself reads element 0)
+    unsigned lo, hi;
+    pair_xor32(__builtin_bit_cast(unsigned, own), lo, hi);  // lower half: lo = own value, hi = that of lane + 32
+    const float gt = __builtin_bit_cast(float, lo), up = __builtin_bit_cast(float, hi);
+    v[q] = gt / (1.0f + expf(-gt)) * up;
+  }
+  if (g < 2) store_out4(o, m, tile * 8 + 4 * g, v);
+}
+
 template <int NT, int MT, int WAVES, typename XT>
 __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(LinearArgs a) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -357,9 +374,10 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(const __half *__restri
   const int64_t blk = f >> 6;
   const int c = static_cast<int>(blk % KC);
   const int64_t t = blk / KC;
-  // glu: packed tile 2j takes rows [16j, 16j+16) of the first half of W (gate), tile 2j+1 the same
-  // rows of the second half (up)
-  const int64_t row = glu ? (t & 1) * (N / 2) + (t >> 1) * 16 + (lane & 15) : t * 16 + (lane & 15);
+  // glu: packed tile j takes rows [8j, 8j+8) of the first half of W (gate) as its rows 0-7 and the same rows of
+  // the second half (up) as its rows 8-15: every tile holds the gate and up rows of its own 8 output columns
+  const int r16 = lane & 15;
+  const int64_t row = glu ? (r16 >> 3) * (N / 2) + t * 8 + (r16 & 7) : t * 16 + r16;
   const int k = c * 32 + (lane >> 4) * 8;
   Vec16 v;
   v.w[0] = v.w[1] = v.w[2] = v.w[3] = 0u;
@@ -373,7 +391,7 @@ struct PackedArgs {
   const __half *bias;
   void *out;
   int M, K, N, KC, chunks_per_wave, out_f16;
-  int glu;  // rows come in tile pairs (gate tile, up tile): the epilogue stores silu(gate) * up, N/2 columns
+  int glu;  // every row tile holds 8 gate rows and their 8 up rows: the epilogue stores silu(gate) * up, N/2 columns
 };
 
 // x fragments.  Loading the MFMA "B" fragments straight from global memory is a 16-row gather (64
@@ -490,23 +508,12 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_packed_kernel(Packed
       tot[t][u] = s;
     }
   }
-  if constexpr (NT % 2 == 0) {
-    if (a.glu) {
-      // tile 2j holds gate rows, tile 2j+1 the up rows of the same 16 output columns
+  if (a.glu) {
 #pragma unroll
-      for (int t = 0; t < NT; t += 2)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int u = 0; u < MT; ++u) {
-          float v[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float gt = tot[t][u][q];
-            v[q] = gt / (1.0f + expf(-gt)) * tot[t + 1][u][q];
-          }
-          store_out4(o, m_base + u * 16 + r, ((tile0 + t) / 2) * 16 + 4 * g, v);
-        }
-      return;
-    }
+      for (int u = 0; u < MT; ++u) store_glu_tile(o, m_base + u * 16 + r, tile0 + t, g, tot[t][u]);
+    return;
   }
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -711,17 +718,9 @@ __global__ __launch_bounds__(256, GM == 128 ? 1 : (GM == 64 ? 2 : 4)) void linea
 #pragma unroll
   for (int u = 0; u < MT; ++u) {
     const int m = m0 + u * 16 + r;
-    if (TW % 2 == 0 && a.glu) {
+    if (a.glu) {
 #pragma unroll
-      for (int t = 0; t + 1 < TW; t += 2) {
-        float v[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float gt = acc[t][u][q];
-          v[q] = gt / (1.0f + expf(-gt)) * acc[t + 1][u][q];
-        }
-        store_out4(o, m, ((tile0 + t) / 2) * 16 + 4 * g, v);
-      }
+      for (int t = 0; t < TW; ++t) store_glu_tile(o, m, tile0 + t, g, acc[t][u]);
     } else {
 #pragma unroll
       for (int t = 0; t < TW; ++t) {
@@ -928,15 +927,7 @@ __global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedAr
 #pragma unroll
     for (int u = 0; u < MT; ++u) {
 #pragma unroll
-      for (int t = 0; t < TW; t += 2) {
-        float v[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float gt = acc[t][u][q];
-          v[q] = gt / (1.0f + expf(-gt)) * acc[t + 1][u][q];
-        }
-        store_out4(o, m0 + u * 16 + r, ((tile0 + t) / 2) * 16 + 4 * g, v);
-      }
+      for (int t = 0; t < TW; ++t) store_glu_tile(o, m0 + u * 16 + r, tile0 + t, g, acc[t][u]);
     }
   } else {
 #pragma unroll
@@ -1089,7 +1080,6 @@ int gemm_tiles_per_wave(const PackedArgs &a, int gm) {
   int tw = 4;
   const int cus = device_cu_count();
   while (tw > 1 && ((a.N + 64 * tw - 1) / (64 * tw)) * m_blocks < cus) tw /= 2;
-  if (a.glu && tw < 2) tw = 2;  // the gated epilogue needs a gate tile and its up tile in one wavefront
   return tw;
 }
 
@@ -1307,9 +1297,11 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
     return launch_status();
   }
   SkinnyPlan p = plan_skinny(M, K, N);
-  if (glu && p.nt % 2 != 0) {  // the gated epilogue needs gate and up tiles in the same wavefront
-    p.nt = 2;
-    if (p.waves > 8) p.waves = 8;
+  // two row tiles per workgroup that would put a second workgroup on half of the CUs only (gate+up 2048 -> 12288:
+  // 384 workgroups on 256 CUs): three tiles give every CU one (M = 16: 11.0 us against 12.0 us)
+  if (g_lin.force_nt == 0 && p.nt == 2 && p.mt == 1) {
+    const int64_t tiles = (N + 15) / 16, cus = device_cu_count();
+    if (tiles % 3 == 0 && tiles / 3 <= cus && (tiles + 1) / 2 > cus) p.nt = 3;
   }
   PackedArgs a;
   a.glu = glu ? 1 : 0;

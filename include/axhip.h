@@ -410,7 +410,7 @@ AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const 
  * Module.cast_linear_fp16 does to a Linear's weights (axono/python/axono/nn/module.py:158-184): a
  * one-off conversion into the resident format the inference kernels read.
  * glu != 0 (both calls): W is a fused [gate ; up] projection (N = 2*I rows, N % 32 == 0); the rows
- * are packed as alternating gate / up tiles and the kernel stores silu(gate) * up, an [M, N/2]
+ * are packed as tiles of 8 gate rows and their 8 up rows and the kernel stores silu(gate) * up, an [M, N/2]
  * result, instead of the [M, N] projection (same arithmetic as axhip_silu_mul on the two halves;
  * no bias). */
 AXHIP_API size_t axhip_linear_f16_packed_bytes(int64_t N, int64_t K);

@@ -572,6 +572,8 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
   } else {
     if (p.nt == 4)
       dispatch_packed_waves<4, 2, XT>(a, p.waves, half, st);
+    else if (p.nt == 3)
+      dispatch_packed_waves<3, 2, XT>(a, p.waves, half, st);
     else if (p.nt == 2)
       dispatch_packed_waves<2, 2, XT>(a, p.waves, half, st);
     else
@@ -1299,9 +1301,13 @@ AXHIP_API int axhip_linear_f16_packed(const void *x, int x_dtype, const void *pa
   SkinnyPlan p = plan_skinny(M, K, N);
   // two row tiles per workgroup that would put a second workgroup on half of the CUs only (gate+up 2048 -> 12288:
   // 384 workgroups on 256 CUs): three tiles give every CU one (M = 16: 11.0 us against 12.0 us)
-  if (g_lin.force_nt == 0 && p.nt == 2 && p.mt == 1) {
+  if (g_lin.force_nt == 0 && p.nt == 2) {
     const int64_t tiles = (N + 15) / 16, cus = device_cu_count();
-    if (tiles % 3 == 0 && tiles / 3 <= cus && (tiles + 1) / 2 > cus) p.nt = 3;
+    if (tiles % 3 == 0 && tiles / 3 <= cus && (tiles + 1) / 2 > cus) {
+      p.nt = 3;
+      // 32 rows of x: eight wavefronts again (M = 32: 13.0 us against 14.1 us with two tiles and four wavefronts)
+      if (p.mt == 2 && g_lin.force_waves == 0 && K / 8 >= 128) p.waves = 8;
+    }
   }
   PackedArgs a;
   a.glu = glu ? 1 : 0;

@@ -427,14 +427,14 @@ def test_decode_step_form_ragged_batch_with_one_workgroup_per_sequence_to_share(
 
 @pytest.mark.parametrize("Hq,Hkv,D,S,start", [(4, 2, 128, 200, [0, 37]), (2, 2, 128, 64, [0, 0]), (8, 2, 64, 130, [5, 300]),
                                                (16, 8, 128, 257, [0, 1])])
-def test_prefill_attention_matches_causal_oracle(Hq, Hkv, D, S, start):
+def test_prefill_attention_matches_causal_oracle(Hq, Hkv, D, S, start, q_scale=1.0):
     """axhip_prefill_attention (MFMA, fp16 probabilities) against the CPU operator with the causal
     mask, per sequence: query i at absolute position start + i sees cache rows 0 .. start + i.  Cache
     rows past the last visible key hold NaN bit patterns: they must not leak into the result."""
     rng = np.random.default_rng(11)
     B = len(start)
     rows = max(start) + S + 70
-    q = rng.standard_normal((B, S, Hq, D)).astype(np.float16)
+    q = (q_scale * rng.standard_normal((B, S, Hq, D))).astype(np.float16)
     kc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
     vc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
     for b in range(B):
@@ -466,6 +466,15 @@ def test_prefill_attention_matches_causal_oracle(Hq, Hkv, D, S, start):
     l = gu.lib()
     assert l.axhip_prefill_attention(dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F32, B, S, Hq, Hkv, D, rows, None) == 3
     assert l.axhip_prefill_attention(dq.ptr, dk.ptr, dv.ptr, ds.ptr, out.ptr, gu.F16, B, S, Hq, Hkv, 256, rows, None) == 1
+
+
+@pytest.mark.parametrize("Hq,Hkv,S,B", [(4, 2, 1100, 1), (16, 8, 600, 8)])
+def test_prefill_attention_both_workgroup_shapes_peaked_scores(Hq, Hkv, S, B):
+    """Long rows with peaked softmax (queries three times the usual size: the running maximum jumps by more than
+    the factor the kernel tolerates without rescaling, and stays put for long stretches) through both workgroup
+    shapes: one round of eight-wavefront workgroups (18 of them), and four-wavefront workgroups (more than one
+    eight-wavefront workgroup per CU would be needed)."""
+    test_prefill_attention_matches_causal_oracle(Hq, Hkv, 128, S, [0] * B, q_scale=3.0)
 
 
 def test_workgroups_are_dealt_by_length():

@@ -498,7 +498,16 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
     if constexpr (HOIST) tile_load<T, D, U, true>(kb, vb, rows, s0, rg, kv_end, kr0, vr0);
     const int wave = tid >> 6, lane = tid & 63;
     const int B = a.B;
-    const bool writer = mine && (h0 % a.group == 0);
+    bool writer = mine && (h0 % a.group == 0);
+    if constexpr (PAGED) {
+      // The clamp above protects reads only.  The page the new row is written to must be one the table
+      // really names: an entry outside the pool (a sequence whose pages were given back) skips the store,
+      // as kv_append_paged_kernel does, instead of landing in another sequence's page.
+      if (writer) {
+        const int raw = a.page_table[static_cast<int64_t>(b) * a.max_pages + (p_new >> kPageShift)];
+        writer = raw >= 0 && raw < a.n_pages;
+      }
+    }
     for (int job = wave; job < G + (mine ? 2 : 0); job += kThreads / 64) {
       if (job < G) {
         norm_rope_row<T, D>(a, a.pq + b * a.pq_stride + static_cast<int64_t>(h0 + job) * D, a.qw, b, B, lane, s_q[job],
@@ -870,7 +879,15 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
   half8_t qf[KK];
   if constexpr (QKV) {
     _Float16 *s_q = ks;  // [heads][D], gone once the first stage is stored
-    const bool writer = mine && (h0 % a.group == 0);
+    bool writer = mine && (h0 % a.group == 0);
+    if constexpr (PAGED) {
+      // reads are clamped into the pool, the store of the new row is not redirected: skipped when the
+      // table entry of its page lies outside the pool
+      if (writer) {
+        const int raw = a.page_table[static_cast<int64_t>(b) * a.max_pages + (p_new >> kPageShift)];
+        writer = raw >= 0 && raw < a.n_pages;
+      }
+    }
     for (int job = wave; job < heads + (mine ? 2 : 0); job += kThreads / 64) {
       if (job < heads) {
         norm_rope_row<__half, D>(a, a.pq + b * a.pq_stride + static_cast<int64_t>(h0 + job) * D, a.qw, b, a.B, lane,

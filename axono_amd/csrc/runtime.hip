@@ -291,14 +291,13 @@ AXHIP_API int axhip_reset_tickets(void) {
   return a != AXHIP_OK ? a : b;
 }
 
+// Gives every cached block back to the driver.  The ticket counters are not touched: they return to zero
+// at the end of every completed launch, and zeroing them here would race with a launch another thread has
+// in flight (axhip_reset_tickets is the explicit call for the recovery case).
 AXHIP_API int axhip_empty_cache(void) {
-  {
-    std::lock_guard<std::mutex> lk(g_mu);
-    evict_locked(0);
-  }
-  // the clean-up call of a process that recovers from a failed launch: counters a killed launch left
-  // behind go back to zero as well (not while capturing: it synchronises the device)
-  return t_capturing ? AXHIP_OK : axhip_reset_tickets();
+  std::lock_guard<std::mutex> lk(g_mu);
+  evict_locked(0);
+  return AXHIP_OK;
 }
 
 // ---- copies ------------------------------------------------------------------------------------

@@ -332,9 +332,13 @@ class Qwen3VLTextDecoder(nn.Module):
         return logits, L.argmax(logits)
 
     # ---- captured decode loop ------------------------------------------------------------------
-    def start_decode(self, first_ids: np.ndarray, first_pos: np.ndarray, max_new_tokens: int):
+    def start_decode(self, first_ids: np.ndarray, first_pos: np.ndarray, max_new_tokens: int,
+                     trace: list | None = None):
         """Sets the static step inputs (ids [B], positions [3,B]) and captures the step.  The
-        attention split plan is sized for the lengths the loop will reach."""
+        attention split plan is sized for the lengths the loop will reach.  `trace`, if given, holds
+        after every run of the step (eager, or a replay of the captured one) the residual stream entering
+        each layer and the one leaving the last, as decode_forward documents; inside a captured step these
+        are the graph's own buffers, refreshed by each replay."""
         B = self._batch
         self._ids.copy_from_numpy(np.ascontiguousarray(first_ids, dtype=np.int64).reshape(B))
         self._pos.copy_from_numpy(np.ascontiguousarray(first_pos, dtype=np.int64).reshape(3, B))
@@ -351,7 +355,9 @@ class Qwen3VLTextDecoder(nn.Module):
         self._counter = Tensor(DataType.INT64, [1], self._device)
 
         def step():
-            logits, nxt = self.decode_forward(self._ids, self._pos, bound)
+            if trace is not None:
+                del trace[:]
+            logits, nxt = self.decode_forward(self._ids, self._pos, bound, trace=trace)
             # the device-side state of the next step, and the token log: one launch
             L.decode_advance(nxt, self._ids, self._pos, self._cache.seq_lens, self._log, self._counter)
             return logits, nxt

@@ -146,7 +146,7 @@ def cpu_baseline_gqa(budget_s=12.0):
         t_total += dt
         n += 1
     gbs = gqa_bytes(1, L) / best / 1e9
-    return {"value": round(gbs, 3), "unit": "GB/s", "cores": cores, "kind": kind,
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": cores, "cpu_model": host_cpu_model(), "kind": kind,
             "sample": f"one sequence of the headline shape (B=1 of 32, L=8192, Hq16/Hkv8/D128), "
                       f"min of {n} runs, fp32 arithmetic on fp16-rounded data; bytes counted as fp16"}
 
@@ -223,7 +223,8 @@ def cpu_decode_step_hook(cfg, weights, model, first, pos, batch, max_len, log):
         f"(|h| max {h_abs:.1f}), logits from the same final state {tf_logit_err:.2e}; "
         f"free-running end to end: logits {err:.2e} (|logits| max {np.abs(c_logits).max():.2f}), greedy tokens agree: {agree}")
     cpu.drop_cache()
-    base = {"value": round(batch / cpu_s, 3), "unit": "tok/s", "cores": oracle.port.num_threads(), "kind": "port",
+    base = {"value": round(batch / cpu_s, 3), "unit": "tok/s", "cores": oracle.port.num_threads(),
+            "cpu_model": host_cpu_model(), "kind": "port",
             "sample": f"1 decode step (batch {batch}, context {ctx}) of the C restatement from the post-prefill cache"}
     par = {"per_layer_max_abs_err_identical_inputs": layer_err, "residual_abs_max": h_abs,
            "logits_max_abs_err_identical_final_state": tf_logit_err,
@@ -378,28 +379,45 @@ def measure_traffic(log, timeout_s=60):
     env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""), TMPDIR="/tmp")
     base = tempfile.mkdtemp(prefix="axhip_pmc_", dir="/tmp")
     readings = {}
+
+    def run_group(cmd):
+        """Runs cmd in a process group of its own and ends the whole group on every exit path (the profiler
+        starts helpers that can outlive it); returns its exit code, or None after the time limit."""
+        import signal
+        proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                                start_new_session=True)
+        try:
+            return proc.wait(timeout=timeout_s)
+        except subprocess.TimeoutExpired:
+            return None
+        finally:
+            try:
+                os.killpg(proc.pid, signal.SIGKILL)
+            except (ProcessLookupError, PermissionError):
+                pass
+            try:
+                proc.wait(timeout=10)
+            except subprocess.TimeoutExpired:
+                pass
+
     try:
         for counter in ("FETCH_SIZE", "WRITE_SIZE"):
             for what, kernel in (("gqa", "gqa_decode_split_kernel"), ("copy", "copy_bytes_kernel")):
                 out = os.path.join(base, f"{counter}_{what}")
                 cmd = [exe, "--pmc", counter, "-d", out, "-o", "p", "--output-format", "csv", "--", sys.executable, "-m",
                        "axono_amd.benchmarks.microbench", what, "--steps", "3"]
-                # own process group: a run that outlives its time limit is ended together with its children
-                proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
-                                        start_new_session=True)
-                try:
-                    rc = proc.wait(timeout=timeout_s)
-                except subprocess.TimeoutExpired:
-                    import signal
-                    os.killpg(proc.pid, signal.SIGKILL)
-                    proc.wait()
+                rc = run_group(cmd)
+                if rc is None:
                     log("traffic counters: a profiler run exceeded its time limit; the recorded constant is reported")
                     return None
                 files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
                 if rc != 0 or not files:
+                    log(f"traffic counters: profiler run ended with code {rc} and {len(files)} result files; "
+                        "the recorded constant is reported")
                     return None
-                vals = [float(row["Counter_Value"]) for row in csv.DictReader(open(files[0]))
-                        if kernel in row["Kernel_Name"] and row["Counter_Name"] == counter]
+                with open(files[0]) as fh:
+                    vals = [float(row["Counter_Value"]) for row in csv.DictReader(fh)
+                            if kernel in row["Kernel_Name"] and row["Counter_Name"] == counter]
                 if not vals:
                     return None
                 readings[(counter, what)] = sum(vals) / len(vals)   # KiB per dispatch
@@ -414,6 +432,38 @@ def measure_traffic(log, timeout_s=60):
         return None
     finally:
         shutil.rmtree(base, ignore_errors=True)
+
+
+def host_cpu_model():
+    """The CPU's model name as the kernel reports it (the CPU baselines are quoted with it)."""
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or platform.machine() or "unknown CPU"
+
+
+def device_label(reported):
+    """`name (arch)` from the runtime; some driver versions leave the name empty, then the marketing name that
+    rocminfo prints for the first GPU agent stands in."""
+    if reported.split("(")[0].strip():
+        return reported
+    import shutil
+    import subprocess
+    exe = shutil.which("rocminfo") or "/opt/rocm/bin/rocminfo"
+    try:
+        txt = subprocess.run([exe], capture_output=True, text=True, timeout=20).stdout
+        names = [l.split(":", 1)[1].strip() for l in txt.splitlines() if l.strip().startswith("Marketing Name")]
+        gpus = [n for n in names if n and "EPYC" not in n and "Xeon" not in n and "Ryzen" not in n and "CPU" not in n]
+        if gpus:
+            return f"{gpus[0]} {reported.strip()}"
+    except (OSError, subprocess.SubprocessError):
+        pass
+    return f"unnamed device {reported.strip()}"
 
 
 def smoke_parity(lib):
@@ -468,7 +518,8 @@ def main():
     name = C.create_string_buffer(256)
     gfx, tot, cus = C.c_int(0), C.c_size_t(0), C.c_int(0)
     lib.axhip_device_info(0, name, 256, C.byref(gfx), C.byref(tot), C.byref(cus))
-    log(f"device: {name.value.decode()} CUs={cus.value} mem={tot.value / 2**30:.0f} GiB")
+    log(f"device: {device_label(name.value.decode())} CUs={cus.value} mem={tot.value / 2**30:.0f} GiB")
+    log(f"host: {host_cpu_model()}, {os.cpu_count()} logical CPUs visible")
 
     err = smoke_parity(lib)
     log(f"parity (small case vs oracle): max abs err {err:.2e}")

@@ -117,7 +117,8 @@ AXHIP_API int axhip_ticket_lane(void);
  * ended abnormally (a device error reported by a later call) can leave counters non-zero, and every later
  * launch of the same slot would then merge early or never.  Synchronises the device; refused with
  * AXHIP_INVALID_ARGUMENT while the calling thread captures a graph; call it while no attention / argmax
- * launch is in flight.  axhip_empty_cache calls it as part of its clean-up.  No reference counterpart. */
+ * launch is in flight on any thread (counters of a launch in flight would be zeroed under it).  No other
+ * call resets the counters implicitly.  No reference counterpart. */
 AXHIP_API int axhip_reset_tickets(void);
 /* 1 while the calling thread is between axhip_graph_begin_capture and end/abort
  * (cuda::IsCapturing, include/axono/core/cuda/capture.h:19-33). */
@@ -488,7 +489,9 @@ AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float
 /* axhip_gqa_decode_qkv over a paged cache (pools, page table, max_pages, n_pages as for
  * axhip_gqa_decode_paged; FLOAT16 caches): the new token's k / v row goes to row seq_lens[b] % 128 of page
  * page_table[b, seq_lens[b] / 128] - that page must already be in the table - when seq_lens[b] < max_len, and
- * the keys are read through the table.  Same bits as axhip_gqa_decode_qkv on a dense cache holding the same rows.
+ * the keys are read through the table.  A table entry outside [0, n_pages) for that page (a sequence whose pages
+ * were given back and not reserved again) skips the store, as axhip_kv_append_paged does; reads clamp such
+ * entries into the pool.  Same bits as axhip_gqa_decode_qkv on a dense cache holding the same rows.
  * No reference counterpart. */
 AXHIP_API int axhip_gqa_decode_qkv_paged(const float *q, int64_t q_stride, const float *k, int64_t k_stride,
                                          const float *v, int64_t v_stride, const void *q_weight,

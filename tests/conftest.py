@@ -23,3 +23,17 @@ def rng():
 def f16(a):
     """fp32 -> fp16 with IEEE round-to-nearest-even (what the device conversion does)."""
     return np.asarray(a, dtype=np.float32).astype(np.float16)
+
+
+@pytest.fixture(autouse=True)
+def _default_tuning_after_gpu_tests(request):
+    """The tuning hooks of the library are process-global: whatever a GPU test forced (and however it
+    ended) the next test starts from the default plans."""
+    yield
+    if request.node.get_closest_marker("gpu") is None:
+        return
+    from axono_amd import _lib
+
+    l = _lib.load()
+    l.axhip_gqa_decode_tune(0, 0)
+    l.axhip_linear_f16_tune(0, 0, 0, 0)

@@ -1,4 +1,5 @@
 """Helpers for the GPU parity tests: every call goes through the C ABI of libaxhip.so."""
+import contextlib
 import ctypes as C
 
 import numpy as np
@@ -44,6 +45,25 @@ def gqa_decode(q, k, v, seq_lens=None, layout="cache", max_len=None):
                              B, Hq, Hkv, D, max_len, sb, sh, ss, None), "gqa_decode")
     synchronize()
     return dout.download(q.dtype, q.shape)
+
+
+@contextlib.contextmanager
+def gqa_tuned(target_workgroups, force_splits):
+    """Forces a split plan of the decode attention for the body; the defaults come back on every exit path."""
+    lib().axhip_gqa_decode_tune(target_workgroups, force_splits)
+    try:
+        yield
+    finally:
+        lib().axhip_gqa_decode_tune(0, 0)
+
+
+@contextlib.contextmanager
+def linear_tuned(target_waves=0, force_nt=0, force_waves=0, gemm_rows=0):
+    lib().axhip_linear_f16_tune(target_waves, force_nt, force_waves, gemm_rows)
+    try:
+        yield
+    finally:
+        lib().axhip_linear_f16_tune(0, 0, 0, 0)
 
 
 def _run(fn_name, *args):

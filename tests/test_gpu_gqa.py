@@ -147,9 +147,8 @@ def test_result_independent_of_split_count():
     q, k, v = _qkv_ref(rng, 5000)
     outs = []
     for splits in (1, 3, 16):
-        lib().axhip_gqa_decode_tune(0, splits)
-        outs.append(gqa_decode(q, k, v, layout="ref"))
-    lib().axhip_gqa_decode_tune(0, 0)
+        with gu.gqa_tuned(0, splits):
+            outs.append(gqa_decode(q, k, v, layout="ref"))
     want = port.gqa_decode(q, k, v)
     for o in outs:
         np.testing.assert_allclose(o, want, rtol=0, atol=TOL32)
@@ -322,19 +321,17 @@ def test_two_kernel_merge_mode_matches_fused_merge():
     for _ in range(3):
         again = gqa_decode(q, k, v, lens).astype(np.float32)
         np.testing.assert_array_equal(again, fused)
-    lib().axhip_gqa_decode_tune(0, 5)                          # 5 ranges per sequence, in-kernel merge
-    fixed = gqa_decode(q, k, v, lens).astype(np.float32)
-    lib().axhip_gqa_decode_tune(-1, 5)                         # 5 ranges per sequence, split kernel + merge kernel
-    two = gqa_decode(q, k, v, lens).astype(np.float32)
-    lib().axhip_gqa_decode_tune(0, 0)
+    with gu.gqa_tuned(0, 5):                                   # 5 ranges per sequence, in-kernel merge
+        fixed = gqa_decode(q, k, v, lens).astype(np.float32)
+    with gu.gqa_tuned(-1, 5):                                  # 5 ranges per sequence, split kernel + merge kernel
+        two = gqa_decode(q, k, v, lens).astype(np.float32)
     for o in (fused, fixed, two):
         assert np.abs(o - want).max() <= TOL16
         assert np.all(o[1] == 0)
     np.testing.assert_array_equal(fixed, two)                  # same ranges, same merge arithmetic
     # a single split and an empty sequence (the split-0 workgroup writes the zeros)
-    lib().axhip_gqa_decode_tune(0, 1)
-    one = gqa_decode(q, k, v, lens).astype(np.float32)
-    lib().axhip_gqa_decode_tune(0, 0)
+    with gu.gqa_tuned(0, 1):
+        one = gqa_decode(q, k, v, lens).astype(np.float32)
     assert np.abs(one - want).max() <= TOL16 and np.all(one[1] == 0)
 
 
@@ -672,6 +669,48 @@ def test_decode_step_form_over_pages_has_the_bits_of_the_dense_cache(Hq, Hkv, D)
         touched[pid, :, r] = True
     np.testing.assert_array_equal(gkp[~touched].view(np.uint16), kp[~touched].view(np.uint16))
     np.testing.assert_array_equal(gvp[~touched].view(np.uint16), vp[~touched].view(np.uint16))
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 2), (16, 2)])
+def test_decode_step_form_over_pages_skips_a_row_whose_page_is_not_in_the_table(Hq, Hkv):
+    """A sequence whose pages were given back (table entries -1, length 0) or whose table names a page outside the
+    pool, replayed without a new reservation: its new row is not stored anywhere (page 0 and every other byte of the
+    pools keep their bits), the other sequences' rows land where their tables say.  Vector and matrix-core kernels."""
+    rng = np.random.default_rng(Hq * 100 + Hkv)
+    D, rows = 128, 640
+    lens = np.array([0, 130, 255, 128, 17], np.int32)
+    B = len(lens)
+    width = (Hq + 2 * Hkv) * D
+    qkv = rng.standard_normal((B, width)).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    kw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    pos = rng.integers(0, 8192, (3, B)).astype(np.int64)
+    inv = port.rope_inv_freq(1e6, D)
+    kc = (0.5 * rng.standard_normal((B, Hkv, rows, D))).astype(np.float16)
+    vc = rng.standard_normal((B, Hkv, rows, D)).astype(np.float16)
+    kp, vp, table, n_pages, max_pages = _paged_from_dense(kc, vc, lens + 1, 3)
+    good = table.copy()
+    table[0, :] = -1                       # freed sequence: its row would have gone to page 0 under a clamp
+    table[3, 1] = n_pages + 5              # the page of row 128 lies outside the pool
+    table[4, 0] = -7
+    l = gu.lib()
+    dq, dqw, dkw, dp, di, dl = (gu.dev(a) for a in (qkv, qw, kw, pos, inv, lens))
+    dkp, dvp, dtb = (gu.dev(a) for a in (kp, vp, table))
+    out_p = gu.DeviceBuffer(B * Hq * D * 2)
+    wsb = l.axhip_gqa_decode_workspace_bytes(B, Hq, Hkv, D, rows)
+    ws = gu.DeviceBuffer(max(wsb, 256))
+    gu._run("axhip_gqa_decode_qkv_paged", dq.ptr, width, dq.ptr + Hq * D * 4, width, dq.ptr + (Hq + Hkv) * D * 4, width,
+            dqw.ptr, dkw.ptr, gu.F32, 1e-6, dp.ptr, di.ptr, 20, 20, dl.ptr, dkp.ptr, dvp.ptr, dtb.ptr, out_p.ptr, ws.ptr,
+            wsb, gu.F16, B, Hq, Hkv, D, rows, max_pages, n_pages, None)
+    gu.synchronize()
+    gkp, gvp = dkp.download(np.uint16, kp.shape), dvp.download(np.uint16, vp.shape)
+    written = np.zeros(kp.shape, bool)
+    for b in (1, 2):
+        written[int(good[b, lens[b] >> 7]), :, int(lens[b] & 127)] = True
+    np.testing.assert_array_equal(gkp[~written], kp.view(np.uint16)[~written])
+    np.testing.assert_array_equal(gvp[~written], vp.view(np.uint16)[~written])
+    assert np.any(gkp[written] != kp.view(np.uint16)[written])          # sequences 1 and 2 did append
+    assert np.all(np.isfinite(out_p.download(np.float16, (B, Hq, D)).astype(np.float32)))
 
 
 @pytest.mark.parametrize("seed", range(12))

@@ -88,6 +88,127 @@ def test_lm_head_every_row_count(M, lm_head_weight):
         assert np.abs(packed - out).max() <= 2 * float(bound.max())
 
 
+def _order_bound(x32, w32, K, b32=None):
+    mag = np.abs(x32) @ np.abs(w32).T + (0 if b32 is None else np.abs(b32))
+    return 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag
+
+
+@pytest.mark.parametrize("M", [1, 16, 32])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 4096)])
+def test_packed_weights_config4_shapes(M, K, N):
+    """The packed-weight (weight-streaming) kernels at the decode row counts of every narrow benchmark shape -
+    among them 2048 -> 12288 without the gate/up layout, which takes three row tiles per workgroup, at M = 32
+    with two x row tiles per wavefront - against the oracle, and close to the row-major path."""
+    rng = np.random.default_rng(M * 11 + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    out = gu.linear_f16_packed(x, w)
+    x32, w32 = x.astype(np.float32), w.astype(np.float32)
+    want = port.linear(x32, w32)
+    bound = _order_bound(x32, w32, K)
+    assert np.all(np.abs(out - want) <= bound), float(np.abs(out - want).max())
+    assert np.all(np.abs(out - gu.linear_f16(x, w)) <= 2 * bound)
+    # fp32 activations are rounded to fp16 on load: the same bits
+    np.testing.assert_array_equal(gu.linear_f16_packed(x32, w), out)
+
+
+@pytest.mark.parametrize("M,K,N", [(33, 2048, 2048), (64, 6144, 2048), (50, 520, 130), (64, 2048, 2064), (65, 2048, 2048),
+                                   (200, 6144, 2048), (100, 1024, 1000), (130, 1536, 4096)])
+def test_packed_weights_33_to_64_rows(M, K, N):
+    """Narrow matrices keep the weight-streaming kernels up to 64 rows (two blocks of rows); one column
+    tile more, or one row more, and the tiled GEMM takes over - for problems this small its form whose
+    loads run four K steps ahead (K a multiple of 512).  Same oracle either side of each switch."""
+    rng = np.random.default_rng(M + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    out = gu.linear_f16_packed(x, w)
+    x32, w32 = x.astype(np.float32), w.astype(np.float32)
+    want = port.linear(x32, w32)
+    assert np.all(np.abs(out - want) <= _order_bound(x32, w32, K))
+    np.testing.assert_array_equal(gu.linear_f16_packed(x32, w), out)
+
+
+@pytest.mark.parametrize("nt", [1, 2, 3, 4])
+@pytest.mark.parametrize("M,K,N,glu", [(16, 2048, 1232, False), (32, 1024, 800, False), (7, 520, 130, False),
+                                       (32, 2048, 1216, True), (16, 512, 160, True), (32, 6144, 2048, False)])
+def test_packed_skinny_every_row_tile_count(nt, M, K, N, glu):
+    """One to four 16-row weight tiles per workgroup, forced, on column counts whose tile number is not a multiple of
+    the forced count (the last workgroup has absent tiles), with one and two x row tiles per wavefront and with the
+    gate/up layout: against the oracle, and the same bits whatever the tile count (four K slices per workgroup in every case)."""
+    rng = np.random.default_rng(nt * 1000 + M + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.03 * rng.standard_normal((N, K)))
+    b = None if glu else h16(0.05 * rng.standard_normal(N))
+    l = gu.lib()
+    l.axhip_linear_f16_tune(0, nt, 4, 0)
+    try:
+        out = gu.linear_f16_packed(x, w, b, glu=glu)
+        out16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16, glu=glu)
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
+    l.axhip_linear_f16_tune(0, 1, 4, 0)
+    try:
+        base = gu.linear_f16_packed(x, w, b, glu=glu)
+    finally:
+        l.axhip_linear_f16_tune(0, 0, 0, 0)
+    np.testing.assert_array_equal(out, base)
+    x32, w32 = x.astype(np.float32), w.astype(np.float32)
+    if glu:
+        full = port.linear(x32, w32)
+        want = port.silu_mul(np.ascontiguousarray(full[:, : N // 2]), np.ascontiguousarray(full[:, N // 2:]))
+        np.testing.assert_allclose(out, want, rtol=0, atol=2e-5)
+    else:
+        want = port.linear(x32, w32, b.astype(np.float32))
+        assert np.all(np.abs(out - want) <= _order_bound(x32, w32, K, b.astype(np.float32)))
+    ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
+    assert np.all(np.abs(out16.astype(np.float32) - want) <= 0.5 * ulp + 2e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * 64)
+
+
+def test_fp32_activations_bias_odd_shapes():
+    """Row-major weights: fp32 activations (what the reference's Linear.forward passes,
+    src/ops/cuda/linear.cu:108-111), bias, shapes that are multiples of nothing but K % 8."""
+    rng = np.random.default_rng(5)
+    for (M, K, N) in [(8, 64, 32), (3, 72, 50), (17, 136, 33), (33, 520, 130), (130, 264, 190)]:
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        w = h16(0.05 * rng.standard_normal((N, K)))
+        b = h16(0.05 * rng.standard_normal(N))
+        check_linear(x, w, b)
+        check_linear(x, w)
+
+
+def test_fp16_output_variant():
+    rng = np.random.default_rng(6)
+    x = h16(rng.standard_normal((16, 2048)))
+    w = h16(0.02 * rng.standard_normal((2048, 2048)))
+    out16 = gu.linear_f16(x, w, out_dtype=np.float16)
+    x32, w32 = x.astype(np.float32), w.astype(np.float32)
+    want = port.linear(x32, w32)
+    ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
+    assert np.all(np.abs(out16.astype(np.float32) - want) <= 0.5 * ulp + _order_bound(x32, w32, 2048))
+
+
+def test_matches_fp32_linear_loosely_like_reference_test():
+    """tests/core/test_fp16.py:28-46 of the reference: fp16 Linear against fp32 Linear at 5e-2."""
+    rng = np.random.default_rng(1)
+    x = rng.normal(size=(8, 64)).astype(np.float32)
+    w = (rng.normal(size=(32, 64)) * 0.05).astype(np.float32)
+    b = (rng.normal(size=(32,)) * 0.05).astype(np.float32)
+    out = gu.linear_f16(x, h16(w), h16(b))
+    np.testing.assert_allclose(out, x @ w.T + b, rtol=5e-2, atol=5e-2)
+    np.testing.assert_allclose(gu.linear_f16_packed(x, h16(w), h16(b)), x @ w.T + b, rtol=5e-2, atol=5e-2)
+
+
+def test_error_codes():
+    l = gu.lib()
+    assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 60, 8, None, 0, None) == 1  # K % 8
+    assert l.axhip_linear_f16(None, 2, None, None, None, 5, 4, 64, 8, None, 0, None) == 3  # x dtype
+    assert l.axhip_linear_f16(None, 4, None, None, None, 5, 4, 64, 8, None, 0, None) == 7  # null pointers
+    assert l.axhip_linear_f16_packed(None, 2, None, None, None, 5, 4, 64, 8, 0, None) == 3
+    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 4, 64, 8, 0, None) == 7
+    assert l.axhip_linear_f16_packed(None, 4, None, None, None, 5, 4, 64, 40, 1, None) == 1  # gate/up needs N % 32 == 0
+    assert l.axhip_linear_f16_pack(None, None, 40, 64, 1, None) == 1
+
+
 def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
     rng = np.random.default_rng(8)
     for (M, K, N) in [(3, 72, 50), (17, 136, 33), (32, 520, 130), (5, 8, 7), (16, 40, 16)]:
@@ -103,7 +224,7 @@ def test_packed_weights_odd_shapes_bias_fp32_x_fp16_out():
     assert l.axhip_linear_f16_packed_bytes(17, 40) == 2 * 2 * 1024
 
 
-@pytest.mark.parametrize("M,K,I", [(16, 2048, 6144), (1, 2048, 6144), (32, 256, 96), (5, 72, 32)])
+@pytest.mark.parametrize("M,K,I", [(16, 2048, 6144), (1, 2048, 6144), (32, 2048, 6144), (32, 256, 96), (5, 72, 32)])
 def test_packed_gate_up_with_silu_mul_epilogue(M, K, I):
     """Fused [gate ; up] projection with the SiLU-mul epilogue against Linear then silu_mul of the oracle."""
     rng = np.random.default_rng(M + K + I)

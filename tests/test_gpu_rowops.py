@@ -1,8 +1,9 @@
 """Fused / row-wise / rotary / cache-append kernels on the GPU against the CPU oracle.
 
-Tolerances: fp32 max abs error <= 1e-5; fp16 <= 2e-3 against the fp32 oracle on fp16-rounded
-inputs (the kernel rounds once at the store; where |value| >= 4 half an fp16 ulp alone is 1.95e-3,
-so those few elements are compared at one ulp of their magnitude).  Byte movers are bit exact.
+Tolerances: fp32 max abs error <= 1e-5.  fp16 (fp32 oracle on fp16-rounded inputs): the kernel rounds once at
+the store, so the bound is half an fp16 ulp of the value plus the operator's own fp32 disagreement term
+(assert_fp16_close; always inside the stated 2e-3 for |value| < 4, and above it only where half an ulp alone is);
+attention keeps 2e-3 absolute.  Byte movers are bit exact.
 """
 import os
 
@@ -23,13 +24,36 @@ def h16(a):
     return np.asarray(a, np.float32).astype(np.float16)
 
 
-def assert_fp16_close(got, want):
-    """<= 2e-3 absolute, or for large magnitudes half an fp16 ulp of the value plus 2e-3 relative slack."""
+def assert_fp16_close(got, want, rel=0.0, abs_=0.0):
+    """The device rounds its fp32 result once to fp16, so against the oracle's fp32 value it may be off by half an
+    fp16 ulp plus however far the two fp32 values can be apart before that rounding: `rel` * |want| + `abs_`, stated
+    per operator by the caller (nothing for a sum of two fp16 values, which is exact in fp32)."""
     got = got.astype(np.float32)
     err = np.abs(got - want)
     ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
-    bound = np.maximum(TOL16, 0.5 * ulp + 1e-3 * np.abs(want))
-    assert np.all(err <= bound), (err.max(), np.abs(want).max())
+    bound = 0.5 * ulp + rel * np.abs(want) + abs_
+    assert np.all(err <= bound), (float(err.max()), float((err - bound).max()), float(np.abs(want).max()))
+
+
+def norm_terms(hidden):
+    """fp32 disagreement of an RMSNorm output: the sum of squares in another order (<= 4 sqrt(H) 2^-24 relative, the
+    bound the Linear tests use for a reordered sum) and three more roundings (rsqrt, two products)."""
+    return dict(rel=(4 * np.sqrt(hidden) + 4) * 2.0 ** -24, abs_=1e-7)
+
+
+# silu(g) * u in fp32: the exponential's argument is rounded once more on the device (exp2 of a product), the
+# exponential and the reciprocal are each good to an ulp: a few 2^-24 relative
+SILU = dict(rel=4e-6, abs_=1e-7)
+# rotation by an angle formed in fp32 exactly as the oracle forms it; accurate sine / cosine on both sides
+# (<= 2 ulp each) and two products + one sum: the fp32 bar of the same operator
+ROPE = dict(abs_=TOL32)
+
+
+def assert_fp16_attention(got, want):
+    """Attention in fp16 keeps the stated bar of 2e-3 absolute: on the matrix-core route the probabilities are
+    themselves rounded to fp16 before the second product, which is not a reduction-order effect."""
+    err = np.abs(got.astype(np.float32) - want)
+    assert np.all(err <= TOL16), float(err.max())
 
 
 # ---- config 1 (fp32 op check) and golden fixtures ---------------------------------------------
@@ -92,17 +116,17 @@ def test_add_rms_norm_fp16_config2():
     for w in (h16(w32),):
         y, out = gu.add_rms_norm(x, r, w, 1e-6)
         np.testing.assert_array_equal(y.view(np.uint16), wy.astype(np.float16).view(np.uint16))  # one rounding of an exact-in-fp32 sum
-        assert_fp16_close(out, wout)
+        assert_fp16_close(out, wout, **norm_terms(2048))
     # fp32 weights with fp16 activations
     wy, wout = port.add_rms_norm(x, r, w32, 1e-6)
     y, out = gu.add_rms_norm(x, r, w32, 1e-6)
-    assert_fp16_close(out, wout)
+    assert_fp16_close(out, wout, **norm_terms(2048))
 
 
 def test_silu_mul_fp16_config2():
     rng = np.random.default_rng(21)
     g, u = h16(rng.standard_normal((32, 6144))), h16(rng.standard_normal((32, 6144)))
-    assert_fp16_close(gu.silu_mul(g, u), port.silu_mul(g, u))
+    assert_fp16_close(gu.silu_mul(g, u), port.silu_mul(g, u), **SILU)
 
 
 @pytest.mark.parametrize("n", [8 * (1024 * 3 + 700) + 5, 8 * 1024 * 2, 8 * 1023 + 7, 3])
@@ -113,7 +137,7 @@ def test_elementwise_whole_and_partial_passes(n):
     g, u = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
     np.testing.assert_allclose(gu.silu_mul(g, u), port.silu_mul(g, u), rtol=2e-6, atol=1e-6)
     np.testing.assert_array_equal(gu.add(g, u), g + u)
-    assert_fp16_close(gu.silu_mul(h16(g), h16(u)), port.silu_mul(h16(g).astype(np.float32), h16(u).astype(np.float32)))
+    assert_fp16_close(gu.silu_mul(h16(g), h16(u)), port.silu_mul(h16(g).astype(np.float32), h16(u).astype(np.float32)), **SILU)
 
 
 def test_elementwise_streaming_form():
@@ -134,7 +158,7 @@ def test_rope_fp16_config2():
     pos = rng.integers(0, 8192, 32).astype(np.int64)
     for heads in (16, 8):
         x = h16(rng.standard_normal((32, heads, 128)))
-        assert_fp16_close(gu.rope(x, pos, 1e6), port.rope(x, pos, 1e6))
+        assert_fp16_close(gu.rope(x, pos, 1e6), port.rope(x, pos, 1e6), **ROPE)
     # fp32 at the same positions: the fp32 angle products are formed exactly as on the CPU
     x = rng.standard_normal((32, 16, 128)).astype(np.float32)
     np.testing.assert_allclose(gu.rope(x, pos, 1e6), port.rope(x, pos, 1e6), rtol=0, atol=TOL32)
@@ -156,8 +180,8 @@ def test_rope_q_and_k_in_one_launch(rows, hq, hk, dim):
         np.testing.assert_array_equal(gq.view(bits), gu.rope(q, pos, 1e6).view(bits))
         np.testing.assert_array_equal(gk.view(bits), gu.rope(k, pos, 1e6).view(bits))
         if dtype == np.float16:
-            assert_fp16_close(gq, port.rope(q, pos, 1e6))
-            assert_fp16_close(gk, port.rope(k, pos, 1e6))
+            assert_fp16_close(gq, port.rope(q, pos, 1e6), **ROPE)
+            assert_fp16_close(gk, port.rope(k, pos, 1e6), **ROPE)
         else:
             np.testing.assert_allclose(gq, port.rope(q, pos, 1e6), rtol=0, atol=TOL32)
             np.testing.assert_allclose(gk, port.rope(k, pos, 1e6), rtol=0, atol=TOL32)
@@ -175,7 +199,7 @@ def test_mrope_family():
     pos3 = rng.integers(0, 8192, (3, rows)).astype(np.int64)
     x = rng.standard_normal((rows, 4, 128)).astype(np.float32)
     np.testing.assert_allclose(gu.rope_thd(x, pos3, inv, [24, 20, 20]), port.rope_thd(x, pos3, inv, [24, 20, 20]), rtol=0, atol=TOL32)
-    assert_fp16_close(gu.rope_thd(h16(x), pos3, inv, [24, 20, 20]), port.rope_thd(h16(x), pos3, inv, [24, 20, 20]))
+    assert_fp16_close(gu.rope_thd(h16(x), pos3, inv, [24, 20, 20]), port.rope_thd(h16(x), pos3, inv, [24, 20, 20]), **ROPE)
     c, s = gu.mrope_cos_sin(pos3, inv, 20, 20)
     wc, ws = port.mrope_cos_sin(pos3, inv, 20, 20)
     np.testing.assert_allclose(c, wc, rtol=0, atol=TOL32)
@@ -199,7 +223,7 @@ def test_rope_many_rows_shares_angles_across_heads():
         pos = rng.integers(0, 32768, rows).astype(np.int64)
         x = h16(rng.standard_normal((rows, heads, 128)))
         got = gu.rope(x, pos, 1e6)
-        assert_fp16_close(got, port.rope(x, pos, 1e6))
+        assert_fp16_close(got, port.rope(x, pos, 1e6), **ROPE)
         # the same rows in slices small enough for one head per thread
         part = np.concatenate([gu.rope(x[i:i + 256], pos[i:i + 256], 1e6) for i in range(0, 1024, 256)])
         np.testing.assert_array_equal(got[:1024].view(np.uint16), part.view(np.uint16))
@@ -319,7 +343,7 @@ def test_sdpa_fp16_on_the_matrix_cores(Sq, Skv, Hq, Hkv, D):
     v = h16(rng.standard_normal((Skv, Hkv, D)))
     f = lambda a: a.astype(np.float32)
     for causal in (True, False):
-        assert_fp16_close(gu.sdpa(q, k, v, causal), port.sdpa(f(q), f(k), f(v), causal))
+        assert_fp16_attention(gu.sdpa(q, k, v, causal), port.sdpa(f(q), f(k), f(v), causal))
 
 
 def test_fp16_output_variants_round_once():
@@ -433,7 +457,7 @@ def test_embedding_rms_norm_equals_the_three_operators():
         np.testing.assert_array_equal(xn.view(np.uint16), dxn2.download(np.float16, (n, dim)).view(np.uint16))
         # and the oracle
         want = port.rms_norm(rows, w.astype(np.float32), 1e-6)
-        assert_fp16_close(xn, want)
+        assert_fp16_close(xn, want, **norm_terms(dim))
     # int32 ids; argument checks
     di32 = gu.dev(ids.astype(np.int32))
     gu._run("axhip_embedding_rms_norm", di32.ptr, gu.I32, dtb.ptr, dw.ptr, gu.dt(w), 1e-6, dh.ptr, dxn.ptr, n, vocab, dim, None)
@@ -493,10 +517,10 @@ def test_row_operators_random_shapes(seed):
         xh, rh = h16(x), h16(r)
         y, out = gu.add_rms_norm(xh, rh, w, 1e-6)
         wy, wout = port.add_rms_norm(xh.astype(np.float32), rh.astype(np.float32), w, 1e-6)
-        assert_fp16_close(y, wy)
+        assert_fp16_close(y, wy)       # a sum of two fp16 values is exact in fp32: the one rounding only
         # the norm is computed from the fp32 sum, not from the rounded y
-        assert_fp16_close(out, wout)
-        assert_fp16_close(gu.silu_mul(xh, rh), port.silu_mul(xh.astype(np.float32), rh.astype(np.float32)))
+        assert_fp16_close(out, wout, **norm_terms(hidden))
+        assert_fp16_close(gu.silu_mul(xh, rh), port.silu_mul(xh.astype(np.float32), rh.astype(np.float32)), **SILU)
     else:
         y, out = gu.add_rms_norm(x, r, w, 1e-6)
         wy, wout = port.add_rms_norm(x, r, w, 1e-6)
@@ -515,8 +539,8 @@ def test_row_operators_random_shapes(seed):
     if half:
         xrh = h16(xr)
         f = xrh.astype(np.float32)
-        assert_fp16_close(gu.rope(xrh, pos, 1e6), port.rope(f, pos, 1e6))
-        assert_fp16_close(gu.rope_thd(xrh, pos3, inv, sec), port.rope_thd(f, pos3, inv, sec))
+        assert_fp16_close(gu.rope(xrh, pos, 1e6), port.rope(f, pos, 1e6), **ROPE)
+        assert_fp16_close(gu.rope_thd(xrh, pos3, inv, sec), port.rope_thd(f, pos3, inv, sec), **ROPE)
     else:
         np.testing.assert_allclose(gu.rope(xr, pos, 1e6), port.rope(xr, pos, 1e6), rtol=0, atol=2e-5)
         np.testing.assert_allclose(gu.rope_thd(xr, pos3, inv, sec), port.rope_thd(xr, pos3, inv, sec), rtol=0, atol=2e-5)
@@ -546,7 +570,7 @@ def test_general_attention_random_shapes(seed):
         if half:
             qh, kh, vh = h16(q), h16(k), h16(v)
             want = port.sdpa(qh.astype(np.float32), kh.astype(np.float32), vh.astype(np.float32), causal)
-            assert_fp16_close(gu.sdpa(qh, kh, vh, causal), want)
+            assert_fp16_attention(gu.sdpa(qh, kh, vh, causal), want)
         else:
             np.testing.assert_allclose(gu.sdpa(q, k, v, causal), port.sdpa(q, k, v, causal), rtol=0, atol=TOL32)
 

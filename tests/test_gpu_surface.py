@@ -467,7 +467,7 @@ def test_allocator_cache_and_budget():
 
 
 def test_ticket_counters_can_be_reset_for_recovery():
-    """axhip_reset_tickets (also part of empty_cache) zeroes the static ticket counters; attention that
+    """axhip_reset_tickets zeroes the static ticket counters (empty_cache leaves them alone); attention that
     merges key ranges in the kernel and the wide argmax give the same results before and after."""
     from axono_amd import _lib
     lib = _lib.load()

@@ -35,21 +35,23 @@ def _setup(B=3, S=21, max_len=64, seed=0, CFG=CFG):
 
 
 
-def assert_cache_rows(got, want, layer):
-    """Cache rows (fp16) of the device against the restatement's.  Layer 0 sees identical inputs: v is one rounding
-    of a Linear output (reordered sum: the Linear tests' bound, here a flat 2e-5), k goes through the k-norm (which
-    divides by an rms of about 0.3) and the rotation on top (1e-4): half an fp16 ulp plus that.  Deeper layers of a
-    free-running comparison see inputs that already differ by fp16 flips of the activations upstream; for them the
-    bound is two such flips at |v| < 4 (4e-3), and the layer-wise tests below compare them on identical inputs."""
+def assert_cache_rows(got, want, layer, fp32_term=1e-4):
+    """Cache rows (fp16) of the device against the restatement's: both sides round an fp32 value once, so they are
+    equal or neighbours wherever those fp32 values agree to within `fp32_term`.  What that term has to cover at
+    layer 0 (identical residual stream): the activation entering the qkv Linear is stored as fp16 on both sides, an
+    fp32 last-bit difference flips a few of its 256 elements by one fp16 ulp (1e-3 * |w| = 2e-5 each in the Linear
+    output), and the k-norm divides by the head's rms (0.3 at this width), which carries up to 2.5e-4 into k - hence
+    5e-4 for k and 1e-4 for v.  Deeper layers of a free-running comparison see a residual stream that already
+    differs by such flips; for them the bound is two fp16 steps at |v| < 4 (4e-3), and the layer-wise tests compare
+    every layer on identical inputs."""
     got, want = got.astype(np.float32), want.astype(np.float32)
+    err = np.abs(got - want)
     if layer > 0:
-        assert np.abs(got - want).max() <= 4e-3, (layer, float(np.abs(got - want).max()))
+        assert err.max() <= 4e-3, (layer, float(err.max()))
         return
     ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
-    err = np.abs(got - want)
-    # both sides are fp16 values: a difference below one ulp means equal, the fp32 term only decides near ties
-    assert np.all(err <= 0.5 * ulp + 1e-4 + 0.5 * ulp * (err > 0)), (layer, float(err.max()))
-    assert np.mean(err > 0) <= 0.05, float(np.mean(err > 0))   # flips are rare: only values whose fp32 forms straddle a tie
+    assert np.all(err <= ulp + fp32_term), (layer, float(err.max()), float((err - ulp).max()))
+    assert np.mean(err > 0) <= 0.2, float(np.mean(err > 0))
 
 
 def test_prefill_logits_and_cache():
@@ -61,7 +63,7 @@ def test_prefill_logits_and_cache():
     S = ids.shape[1]
     for i in range(CFG.num_hidden_layers):
         kc, vc = gpu.cache.get(i)
-        assert_cache_rows(kc.numpy()[:, :, :S], cpu.k[i][:, :, :S], i)
+        assert_cache_rows(kc.numpy()[:, :, :S], cpu.k[i][:, :, :S], i, 5e-4)
         assert_cache_rows(vc.numpy()[:, :, :S], cpu.v[i][:, :, :S], i)
         assert np.all(kc.numpy()[:, :, S:] == 0)
     np.testing.assert_array_equal(gpu.cache.seq_lens.to_numpy(), [S] * ids.shape[0])
@@ -92,7 +94,7 @@ def test_decode_steps_match_oracle(use_graph):
     np.testing.assert_array_equal(gpu.cache.seq_lens.to_numpy(), [S + n_steps] * B)
     # cache rows written by the decode steps
     for i in range(CFG.num_hidden_layers):
-        assert_cache_rows(gpu.cache.get(i)[0].numpy()[:, :, S:S + n_steps], cpu.k[i][:, :, S:S + n_steps], i)
+        assert_cache_rows(gpu.cache.get(i)[0].numpy()[:, :, S:S + n_steps], cpu.k[i][:, :, S:S + n_steps], i, 5e-4)
 
 
 def test_compiled_decode_loop_matches_the_captured_step():
@@ -171,7 +173,7 @@ def test_decode_steps_match_oracle_with_four_heads_per_kv_head():
     for i in range(CFG4.num_hidden_layers):
         kc, vc = gpu.cache.get(i)
         n = S + n_steps
-        assert_cache_rows(kc.numpy()[:, :, :n], cpu.k[i][:, :, :n], i)
+        assert_cache_rows(kc.numpy()[:, :, :n], cpu.k[i][:, :, :n], i, 5e-4)
         assert_cache_rows(vc.numpy()[:, :, :n], cpu.v[i][:, :, :n], i)
 
 
@@ -344,12 +346,15 @@ def test_captured_step_at_the_real_widths_of_the_2b_shape():
     for i in range(cfg.num_hidden_layers):
         err = float(np.abs(outs[i] - h_gpu[i + 1]).max())
         assert err <= 2e-3, (i, err)
-        # the new token's cache row: the oracle's fp16 row, or its neighbour where the fp32 value sits on a boundary
+        # the new token's cache row
         kc, vc = gpu.cache.get(i)
         gk, gv = kc.numpy()[:, :, ctx].astype(np.float32), vc.numpy()[:, :, ctx].astype(np.float32)
         wk, wv = cpu.k[i][:, :, ctx].astype(np.float32), cpu.v[i][:, :, ctx].astype(np.float32)
-        assert np.all(np.abs(gk - wk) <= np.spacing(np.abs(wk).astype(np.float16)).astype(np.float32)), i
-        assert np.all(np.abs(gv - wv) <= np.spacing(np.abs(wv).astype(np.float16)).astype(np.float32)), i
+        # teacher-forced: every layer is a "layer 0" (identical input).  Of the 2048 activations entering the qkv
+        # Linear a few flip by one fp16 ulp (up to 1.95e-3 for |x| in [2, 4)) times |w| up to 0.08: 3e-4 covers two
+        # such flips in one output; a head's rms is about 0.9 at this width, so k carries the same term
+        assert_cache_rows(gk, wk, 0, 3e-4)
+        assert_cache_rows(gv, wv, 0, 3e-4)
         assert np.all(kc.numpy()[:, :, ctx + 1:] == 0)
     err = float(np.abs(tf_logits - logits).max())
     assert err <= 2e-3, err

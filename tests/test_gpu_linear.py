@@ -124,8 +124,16 @@ def test_packed_weights_33_to_64_rows(M, K, N):
     out = gu.linear_f16_packed(x, w)
     x32, w32 = x.astype(np.float32), w.astype(np.float32)
     want = port.linear(x32, w32)
-    assert np.all(np.abs(out - want) <= _order_bound(x32, w32, K))
-    np.testing.assert_array_equal(gu.linear_f16_packed(x32, w), out)
+    bound = _order_bound(x32, w32, K)
+    assert np.all(np.abs(out - want) <= bound)
+    # fp32 activations are rounded to fp16 on load: the same values enter the products.  The weight-streaming
+    # kernels then sum in the same order (same bits); the tiled GEMM may pick another tile for fp32 x (the form
+    # that sums K in two halves takes fp16 x only), i.e. another order within the same bound
+    out32 = gu.linear_f16_packed(x32, w)
+    if M <= 64 and N <= 2048:
+        np.testing.assert_array_equal(out32, out)
+    else:
+        assert np.all(np.abs(out32 - want) <= bound)
 
 
 @pytest.mark.parametrize("nt", [1, 2, 3, 4])
@@ -156,7 +164,8 @@ def test_packed_skinny_every_row_tile_count(nt, M, K, N, glu):
     if glu:
         full = port.linear(x32, w32)
         want = port.silu_mul(np.ascontiguousarray(full[:, : N // 2]), np.ascontiguousarray(full[:, N // 2:]))
-        np.testing.assert_allclose(out, want, rtol=0, atol=2e-5)
+        # the reordered sums of the two projections (a few 1e-6 at K = 2048) carried through silu(g) * u
+        np.testing.assert_allclose(out, want, rtol=2e-5, atol=2e-5)
     else:
         want = port.linear(x32, w32, b.astype(np.float32))
         assert np.all(np.abs(out - want) <= _order_bound(x32, w32, K, b.astype(np.float32)))

@@ -474,6 +474,46 @@ def test_prefill_attention_both_workgroup_shapes_peaked_scores(Hq, Hkv, S, B):
     test_prefill_attention_matches_causal_oracle(Hq, Hkv, 128, S, [0] * B, q_scale=3.0)
 
 
+@pytest.mark.parametrize("gap,peak_at", [(7.9, 3000), (8.1, 3000), (7.9, 5), (7.9, 4150)])
+def test_prefill_attention_peak_next_to_a_long_plateau(gap, peak_at):
+    """The running maximum of the prefill kernel follows a block only when it exceeds it by more than 8 (log2).
+    Rows built to sit on that rule: 4200 keys, all with the same score except one peak `gap` log2 units above
+    them - just inside the threshold (the maximum stays at the plateau, the peak's probability is 2^7.9 = 239 in
+    fp16) and just outside (the maximum moves, everything accumulated is rescaled) - arriving after the maximum has
+    settled, at the start, or in the last block; plus a second tier of 1000 keys 2^-10 below the plateau, whose
+    probabilities would be subnormal in fp16 had the maximum followed the peak.  Every query row that sees the peak
+    must match the oracle to the usual fp16 bar."""
+    rng = np.random.default_rng(int(gap * 10) + peak_at)
+    Hq, Hkv, D, S = 4, 2, 128, 4200
+    c = 4.0
+    x_peak = float(np.float16(gap * np.sqrt(D) / (c * np.log2(np.e))))
+    x_low = float(np.float16(-10.0 * np.sqrt(D) / (c * np.log2(np.e))))
+    q = np.zeros((1, S, Hq, D), np.float16)
+    q[..., 0] = c
+    q[..., 1:] = (0.01 * rng.standard_normal((1, S, Hq, D - 1))).astype(np.float16)
+    kc = np.zeros((1, Hkv, S, D), np.float16)
+    low = rng.choice(np.setdiff1d(np.arange(S), [peak_at]), 1000, replace=False)
+    kc[0, :, low, 0] = x_low
+    kc[0, :, peak_at, 0] = x_peak
+    vc = rng.standard_normal((1, Hkv, S, D)).astype(np.float16)
+    dq, dk, dv = (gu.dev(a) for a in (q, kc, vc))
+    out = gu.DeviceBuffer(q.nbytes)
+    gu._run("axhip_prefill_attention", dq.ptr, dk.ptr, dv.ptr, None, out.ptr, gu.F16, 1, S, Hq, Hkv, D, S, None)
+    gu.synchronize()
+    got = out.download(np.float16, q.shape).astype(np.float32)[0]
+    k = np.ascontiguousarray(np.transpose(kc[0], (1, 0, 2)), dtype=np.float32)
+    v = np.ascontiguousarray(np.transpose(vc[0], (1, 0, 2)), dtype=np.float32)
+    rows = sorted({peak_at, min(peak_at + 1, S - 1), min(peak_at + 40, S - 1), (peak_at + S) // 2, S - 1, max(peak_at - 1, 0)})
+    for i in rows:
+        want = port.sdpa(q[0, i:i + 1].astype(np.float32), k[:i + 1], v[:i + 1], False)[0]
+        err = float(np.abs(got[i] - want).max())
+        assert err <= TOL16, (gap, peak_at, i, err)
+    # the weight of the peak against the plateau is what the construction says (a check of the test itself)
+    i = S - 1
+    sc = (q[0, i, 0].astype(np.float32) @ k[:, 0].T) / np.sqrt(D) * np.log2(np.e)
+    assert abs((sc[peak_at] - np.median(sc)) - gap) < 0.05
+
+
 def test_workgroups_are_dealt_by_length():
     """Very uneven batches under the default plan: one long sequence among short ones, all equal,
     and lengths that leave some of the launch's workgroup slots unused."""

@@ -113,6 +113,7 @@ struct LinearArgs {
 };
 
 // Final store of 4 consecutive n for one m, bias added.
+template <bool NT = false>
 __device__ __forceinline__ void store_out4(const LinearArgs &a, int m, int n, const float (&v)[4]) {
   if (m >= a.M) return;
   const int64_t o = static_cast<int64_t>(m) * a.N + n;
@@ -126,7 +127,10 @@ __device__ __forceinline__ void store_out4(const LinearArgs &a, int m, int n, co
       for (int r = 0; r < 4; ++r) h[r] = static_cast<_Float16>(y[r]);
       *reinterpret_cast<half4_t *>(static_cast<__half *>(a.out) + o) = h;
     } else {
-      *reinterpret_cast<float4_t *>(static_cast<float *>(a.out) + o) = float4_t{y[0], y[1], y[2], y[3]};
+      if constexpr (NT)
+        __builtin_nontemporal_store(float4_t{y[0], y[1], y[2], y[3]}, reinterpret_cast<float4_t *>(static_cast<float *>(a.out) + o));
+      else
+        *reinterpret_cast<float4_t *>(static_cast<float *>(a.out) + o) = float4_t{y[0], y[1], y[2], y[3]};
     }
     return;
   }
@@ -594,6 +598,7 @@ void dispatch_packed(const PackedArgs &a, const SkinnyPlan &p, hipStream_t st) {
 constexpr int kGK = 128;  // workgroup tile: 64 TW weight rows (TW row tiles per wavefront) x GM rows of x, K in steps of kGK
 int g_gemm_rows = 0;                 // measurement hook: 64 or 128 rows of x per workgroup (0 = default)
 int g_gemm_tiles = 0;                // measurement hook: 1, 2 or 4 row tiles of W per wavefront (0 = by size)
+int g_tile_order = -1;               // measurement hook: A * 256 + B rectangles of 256 x 128 tiles per XCD (0 = plain order, -1 = by size)
 constexpr int kXcds = 8;
 
 // FULL: K is a multiple of the 128-column step, so no load needs a predicate (rows and tiles past
@@ -826,56 +831,97 @@ __global__ __launch_bounds__(256, GM == 64 ? 2 : 4) void linear_gemm_packed_deep
   }
 }
 
-// 256 weight rows x 128 rows of x with two workgroups per CU.  Against the 256 x 64 tile this halves
-// the W bytes that pass through the CU's vector memory path per product (that path, 64 bytes per
-// clock, is what bounds the smaller tile), but its 128 accumulators leave room for little else in the
-// 256 registers of a wavefront at this occupancy: the W fragments are held for two chunks of 32 K only
-// (chunk j+2 is requested when chunk j has been used), and the x fragments of a chunk are read from
-// LDS when they are needed.  K % 128 == 0, N in whole row tiles handled by clamping.
-template <typename XT>
-__global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedArgs a, int n_blocks, int m_blocks) {
-  constexpr int GM = 128, MT = 8, TW = 4;
-  constexpr int XV = GM * 16 / 256;
+// 256 weight rows x 128 rows of x with two workgroups per CU (fp16 x, K % 128 == 0).  Against the 256 x 64 tile
+// this halves the W bytes that pass through the CU's vector memory path per product.  Measured facts that shape it:
+// the matrix pipes of this part are clocked by power - the same launch runs 20-45 % faster on all-zero data - and the
+// time of a launch is, to within a few percent, the sum of what its matrix instructions take alone (the loop with
+// every load and store removed) and what each kind of data movement adds when it is put back: output stores, x
+// loads, W loads, LDS reads, in that order of cost.  Hiding latency better buys nothing (a second set of x
+// fragments read one half chunk ahead, W fragments three or four chunks ahead: same time); moving fewer bytes does.
+// Hence:
+//  * all global loads are buffer loads - one 32-bit lane offset for the eight x vectors of a step and one for the W
+//    fragments, everything else in scalar registers; rows of x past M read as zeros by the buffer's bounds check;
+//  * the x fragments of a half chunk (4 of the 8 row tiles) are read from LDS while the 16 products of the half
+//    chunk before them issue (two register sets: the registers the scalar addressing freed);
+//  * tiles are handed out in rectangles of A weight-row blocks x B blocks of x rows, one rectangle to one XCD at a
+//    time (workgroup ids are dealt round-robin to the XCDs): the 64 workgroups an XCD runs together then share A W
+//    tiles and B x tiles through its L2 instead of one W tile and 64 x tiles (2048 -> 151936 at M = 4096: 947 ->
+//    1074 TFLOP/s; nothing where x fits the L2 anyway, as at M = 512).
+// Every output element sums its products in K order: the same bits as the 64-row tile.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half8_t buffer_load_h8(__amdgpu_buffer_rsrc_t rsrc, int voffset, int soffset) {
+  return __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voffset, soffset, 0));
+}
+
+struct TileOrder {
+  int A, B;  // rectangle of A n-blocks x B m-blocks per XCD at a time; A == 0: n-blocks dealt to XCDs, m fastest
+};
+
+__global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedArgs a, int n_blocks, int m_blocks, TileOrder ord) {
+  constexpr int GM = 128, MT = 8, TW = 4, XV = 8;
   __shared__ __attribute__((aligned(16))) _Float16 xs[2][GM * kGK];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int id = blockIdx.x;
   const int xcd = id % kXcds, slot = id / kXcds;
-  const int nb = (slot / m_blocks) * kXcds + xcd, mb = slot % m_blocks;
+  int nb, mb;
+  if (ord.A > 0) {
+    const int per = ord.A * ord.B, within = slot % per;
+    const int rect = (slot / per) * kXcds + xcd;          // rectangles in the order they are handed out
+    const int rect_m = (m_blocks + ord.B - 1) / ord.B;
+    mb = (rect % rect_m) * ord.B + within % ord.B;
+    nb = (rect / rect_m) * ord.A + within / ord.B;
+    if (mb >= m_blocks) return;
+  } else {
+    nb = (slot / m_blocks) * kXcds + xcd;
+    mb = slot % m_blocks;
+  }
   if (nb >= n_blocks) return;
   const int n_tiles = (a.N + 15) / 16;
   const int tile0 = (nb * 4 + wave) * TW;
   const int m0 = mb * GM;
-  const XT *x = static_cast<const XT *>(a.x);
   const int chunks = a.K / 32, steps = chunks / 4;
 
-  const __half *wt[TW];
+  // W: a buffer per wavefront that starts at its first row tile (tiles past the last one: the last one again)
+  const int t0c = min(tile0, n_tiles - 1);
+  const int64_t wbytes = static_cast<int64_t>(n_tiles - t0c) * a.KC * 1024;
+  const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<__half *>(a.wp + static_cast<int64_t>(t0c) * a.KC * 512), 0,
+      static_cast<int>(wbytes < 0x7fffffff ? wbytes : 0x7fffffff), 0x00020000);
+  int wso[TW];
 #pragma unroll
-  for (int t = 0; t < TW; ++t)
-    wt[t] = a.wp + (static_cast<int64_t>(min(tile0 + t, n_tiles - 1)) * a.KC) * 512 + lane * 8;
+  for (int t = 0; t < TW; ++t) wso[t] = (min(tile0 + t, n_tiles - 1) - t0c) * a.KC * 1024;
+  const int wvo = lane * 16;
   auto load_w = [&](int chunk, half8_t (&f)[TW]) {
-    const int64_t off = static_cast<int64_t>(min(chunk, chunks - 1)) * 512;  // past the end: the last chunk again
+    const int co = min(chunk, chunks - 1) * 1024;  // past the end: the last chunk again
 #pragma unroll
-    for (int t = 0; t < TW; ++t) f[t] = load_h8(wt[t] + off);
+    for (int t = 0; t < TW; ++t) f[t] = buffer_load_h8(wrs, wvo, wso[t] + co);
   };
-  // x staging: 128 rows x 16 units of 16 bytes per step, 8 per thread; 32-bit element offsets
-  unsigned xo[XV];
-#pragma unroll
-  for (int p = 0; p < XV; ++p) {
-    const int v = p * 256 + tid;
-    xo[p] = static_cast<unsigned>(min(m0 + (v >> 4), a.M - 1)) * static_cast<unsigned>(a.K) + (v & 15) * 8;
-  }
+  // x: a buffer of this workgroup's rows; vector p of a thread is row (tid >> 4) + 16 p, 16-byte unit tid & 15
+  const int rows_here = min(GM, a.M - m0);
+  const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16 *>(static_cast<const _Float16 *>(a.x) + static_cast<int64_t>(m0) * a.K), 0,
+      rows_here * a.K * 2, 0x00020000);
+  const int xvo = ((tid >> 4) * a.K + (tid & 15) * 8) * 2;
+  const int xrow16 = 16 * a.K * 2;
   auto load_x = [&](int step, half8_t (&xv)[XV]) {
 #pragma unroll
-    for (int p = 0; p < XV; ++p) xv[p] = load_h8(x + (static_cast<size_t>(xo[p]) + step * kGK));
+    for (int p = 0; p < XV; ++p) xv[p] = buffer_load_h8(xrs, xvo, p * xrow16 + step * (kGK * 2));
   };
+  const int xrow = tid >> 4, xunit = tid & 15;
+  _Float16 *xst = &xs[0][xrow * kGK + ((xunit ^ (xrow & 15)) * 8)];  // rows 16 apart keep row & 15
   auto store_x = [&](int buf, const half8_t (&xv)[XV]) {
 #pragma unroll
-    for (int p = 0; p < XV; ++p) {
-      const int v = p * 256 + tid;
-      const int row = v >> 4, unit = v & 15;
-      *reinterpret_cast<half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]) = xv[p];
-    }
+    for (int p = 0; p < XV; ++p) *reinterpret_cast<half8_t *>(xst + buf * (GM * kGK) + p * 16 * kGK) = xv[p];
+  };
+  // fragment reads: row tile u, chunk j of the step -> rows u*16 + r, unit j*4 + g
+  const _Float16 *xrd = &xs[0][r * kGK];
+  auto load_bf = [&](int buf, int j, int uh, half8_t (&f)[4]) {
+    const int uo = ((j * 4 + g) ^ r) * 8;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      f[u] = *reinterpret_cast<const half8_t *>(xrd + buf * (GM * kGK) + (uh + u) * 16 * kGK + uo);
   };
 
   float4_t acc[TW][MT];
@@ -886,6 +932,7 @@ __global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedAr
 
   half8_t wf[2][TW];  // chunk c waits in wf[c & 1]
   half8_t xv[XV];
+  half8_t bfa[4], bfb[4];
   load_w(0, wf[0]);
   load_w(1, wf[1]);
   load_x(0, xv);
@@ -895,23 +942,28 @@ __global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedAr
   for (int i = 0; i < steps; ++i) {
     const int buf = i & 1;
     load_x(min(i + 1, steps - 1), xv);
+    load_bf(buf, 0, 0, bfa);
+    // the scheduling barriers keep the requests where they are written: left alone, the scheduler sinks them to
+    // their uses (shorter live ranges) and every group of products then waits out a full latency
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      load_bf(buf, j, 4, bfb);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int uh = 0; uh < MT; uh += 4) {  // x fragments four at a time: registers
-        half8_t bf[4];
+      for (int t = 0; t < TW; ++t)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int row = (uh + u) * 16 + r, unit = j * 4 + g;
-          bf[u] = *reinterpret_cast<const half8_t *>(&xs[buf][row * kGK + ((unit ^ (row & 15)) * 8)]);
-        }
+        for (int u = 0; u < 4; ++u)
+          acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j & 1][t], bfa[u], acc[t][u], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j + 1 < 4) load_bf(buf, j + 1, 0, bfa);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < TW; ++t)
+      for (int t = 0; t < TW; ++t)
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
-            acc[t][uh + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j & 1][t], bf[u], acc[t][uh + u], 0, 0, 0);
-      }
+        for (int u = 0; u < 4; ++u)
+          acc[t][4 + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[j & 1][t], bfb[u], acc[t][4 + u], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
       load_w(i * 4 + j + 2, wf[j & 1]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -941,6 +993,45 @@ __global__ __launch_bounds__(256, 2) void linear_gemm_packed_128_kernel(PackedAr
       }
     }
   }
+}
+
+// How the 256 x 128 tiles of a problem are handed to the XCDs.  An XCD runs 64 workgroups at a time (32 CUs, two
+// each).  In the plain order they are a strip of up to 64 x blocks under one or two W blocks; a rectangle of A W
+// blocks x B x blocks has the same workgroups share A W tiles and B x tiles through the XCD's L2.  The choice is
+// the rectangle (A, B powers of two, 16 to 64 tiles) with the smallest estimate of
+//   (workgroup slots launched / tiles) x (1 + 0.3 x operand bytes fetched per tile / bytes of a W tile):
+// slots count the rectangles rounded up to whole rounds over the eight XCDs (few rectangles leave XCDs idle: 2048 ->
+// 2048 at M = 4096 is 256 tiles = 8 rectangles of 8 x 4, not 4 of 8 x 8), and 0.3 fits the measured gains (M = 4096:
+// 2048 -> 4096 861 -> 969 TFLOP/s, 2048 -> 151936 926 -> 992; M = 65536: 2048 -> 2048 849 -> 905).  Not worth it
+// while x (M x K) fits one XCD's L2 next to the W stream, as at M = 512.
+TileOrder gemm_tile_order(const PackedArgs &a, int n_blocks, int m_blocks) {
+  TileOrder o{0, 0};
+  if (g_tile_order >= 0) {  // measurement hook: A * 256 + B, 0 = the plain order
+    o.A = g_tile_order >> 8;
+    o.B = g_tile_order & 255;
+    if (o.A <= 0 || o.B <= 0) o = TileOrder{0, 0};
+    return o;
+  }
+  if (static_cast<int64_t>(a.M) * a.K * 2 <= (3 << 20)) return o;
+  const double tiles = static_cast<double>(n_blocks) * m_blocks;
+  auto estimate = [&](double slots, double A, double B) { return slots / tiles * (1.0 + 0.3 * (A + 0.5 * B) / (A * B)); };
+  // plain order: n-blocks dealt to the XCDs, whole rounds; the 64 workgroups of an XCD are x blocks first
+  const double nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
+  const double Bp = m_blocks < 64 ? m_blocks : 64, Ap = m_blocks < 64 ? (64 + m_blocks - 1) / m_blocks : 1;
+  double best = estimate(nb_pad * m_blocks, Ap, Bp);
+  for (int A = 1; A <= 16; A *= 2)
+    for (int B = 1; B <= 64; B *= 2) {
+      const int per = A * B;
+      if (per < 16 || per > 64 || A > 2 * n_blocks || B > 2 * m_blocks) continue;
+      const int64_t rects = static_cast<int64_t>((n_blocks + A - 1) / A) * ((m_blocks + B - 1) / B);
+      const double slots = static_cast<double>((rects + kXcds - 1) / kXcds * kXcds) * per;
+      const double e = estimate(slots, A, B) * (per < 64 ? 1.02 : 1.0);  // ties go to full rectangles
+      if (e < best) {
+        best = e;
+        o = TileOrder{A, B};
+      }
+    }
+  return o;
 }
 
 // One workgroup per CU with eight wavefronts for the problems that give a CU only one tile of 64 TW weight
@@ -1116,8 +1207,13 @@ void launch_gemm_packed(const PackedArgs &a, hipStream_t st) {
     if (fits && (g_gemm_rows == 256 || (g_gemm_rows == 0 && g_gemm_tiles == 0 && tiles128 >= 3 * device_cu_count() / 4))) {
       const int n_blocks = (a.N + 255) / 256, m_blocks = (a.M + 127) / 128;
       const int nb_pad = (n_blocks + kXcds - 1) / kXcds * kXcds;
-      hipLaunchKernelGGL((linear_gemm_packed_128_kernel<XT>), dim3(static_cast<unsigned>(nb_pad) * m_blocks), dim3(256), 0,
-                         st, a, n_blocks, m_blocks);
+      const TileOrder ord = gemm_tile_order(a, n_blocks, m_blocks);
+      unsigned grid128 = static_cast<unsigned>(nb_pad) * m_blocks;
+      if (ord.A > 0) {
+        const int64_t rects = static_cast<int64_t>((n_blocks + ord.A - 1) / ord.A) * ((m_blocks + ord.B - 1) / ord.B);
+        grid128 = static_cast<unsigned>((rects + kXcds - 1) / kXcds * kXcds * ord.A * ord.B);
+      }
+      hipLaunchKernelGGL(linear_gemm_packed_128_kernel, dim3(grid128), dim3(256), 0, st, a, n_blocks, m_blocks, ord);
       return;
     }
   }
@@ -1186,6 +1282,9 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
   g_gemm_tiles = gemm_rows >= 1000 ? gemm_rows / 1000 : 0;
   gemm_rows %= 1000;
   g_gemm_rows = (gemm_rows == 32 || gemm_rows == 64 || gemm_rows == 128 || gemm_rows == 256 || gemm_rows == 512) ? gemm_rows : 0;
+  // target_waves >= 100000 carries a tile order for the 256 x 128 GEMM tile: 100000 + A * 256 + B (100000: plain order)
+  g_tile_order = target_waves >= 100000 ? target_waves - 100000 : -1;
+  if (target_waves >= 100000) target_waves = 0;
   g_lin.target_waves = target_waves > 0 ? target_waves : 0;
   g_lin.force_nt = (force_nt >= 1 && force_nt <= 4) ? force_nt : 0;
   g_lin.force_waves = (force_waves == 4 || force_waves == 8 || force_waves == 16) ? force_waves : 0;

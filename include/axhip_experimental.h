@@ -27,7 +27,10 @@ AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
  * (the default for large problems), 512 = the eight-wavefront workgroup that sums K in two halves (fp16 x,
  * K % 512 == 0, otherwise ignored; with 1000 t: t = 1 or 2 row tiles), plus 1000 t to force t = 1, 2 or 4 row
  * tiles of W per wavefront (64, 128 or 256 weight rows per workgroup; by default the largest that still
- * gives every CU a workgroup). */
+ * gives every CU a workgroup).  target_waves >= 100000 does not set the skinny plan but the order in which the
+ * 256 x 128 tiles are handed to the XCDs: 100000 + 256 A + B = rectangles of A weight-row blocks x B blocks of
+ * x rows per XCD at a time, 100000 = weight-row blocks dealt to the XCDs with the x blocks fastest (the default
+ * picks by problem size). */
 AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows);
 
 #ifdef __cplusplus

@@ -46,9 +46,14 @@ def _time(lib, fn, steps, warmup=5):
     return ms.value / steps * 1e3  # us
 
 
+ZERO_DATA = False   # --zero-data: operands of all zeros (the same instructions on data that toggles nothing)
+
+
 def _rand_fill(buf, nbytes, seed):
     rng = np.random.default_rng(seed)
     block = rng.standard_normal(8 * 1024 * 1024).astype(np.float32).astype(np.float16)
+    if ZERO_DATA:
+        block[:] = 0
     off = 0
     while off < nbytes:
         n = min(block.nbytes, nbytes - off)
@@ -311,6 +316,8 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
     shapes = shapes or [(2048, 2048), (2048, 12288), (6144, 2048), (2048, 151936)]
     for K, N in shapes:
         w_host = (0.02 * rng.standard_normal((min(N, 4096), K))).astype(np.float32).astype(np.float16)
+        if ZERO_DATA:
+            w_host[:] = 0
         # several weight copies are rotated when one is smaller than the Infinity Cache
         n_rot = rot or max(1, min(8, int(600e6 // (2 * K * N)) + 1))
         ws_ = []
@@ -328,7 +335,10 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
                 wb = pb
             ws_.append(wb)
         for M in Ms:
-            x = DeviceBuffer.from_numpy(rng.standard_normal((M, K)).astype(np.float32).astype(np.float16))
+            x_host = rng.standard_normal((M, K)).astype(np.float32).astype(np.float16)
+            if ZERO_DATA:
+                x_host[:] = 0
+            x = DeviceBuffer.from_numpy(x_host)
             out = DeviceBuffer(M * N * 4)
             wsb = lib.axhip_linear_f16_workspace_bytes(M, K, N)
             ws = DeviceBuffer(max(wsb, 256))
@@ -354,6 +364,8 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "gqa-paged", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
+    ap.add_argument("--zero-data", action="store_true",
+                    help="prefill-attn, linear-packed: all-zero operands (how much of the time is the power the data costs)")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -368,6 +380,8 @@ def main(argv=None):
     ap.add_argument("--gemm-rows", type=int, default=0, help="linear: rows of x per GEMM workgroup (64 or 128)")
     ap.add_argument("--rot", type=int, default=0, help="linear: number of weight copies rotated through (1 = cache-hot)")
     args = ap.parse_args(argv)
+    global ZERO_DATA
+    ZERO_DATA = bool(args.zero_data)
     lib = _lib.load()
     if _lib.device_count() < 1:
         sys.exit("no HIP device")

@@ -31,6 +31,7 @@ namespace axhip {
 namespace {
 
 constexpr int kStageKeys = 64;  // keys per LDS stage
+constexpr int kXcdCount = 8;
 constexpr float kMasked = -1.0e30f;
 
 struct PrefillArgs {
@@ -44,6 +45,7 @@ struct PrefillArgs {
   // general form only (GEN): K/V strides in elements, and whether the causal rule applies
   int64_t kv_batch_stride, kv_head_stride, kv_row_stride;
   int causal;
+  int pos_blocks, head_groups, n_pairs, pairs_by_xcd;  // launch geometry (filled by launch_prefill)
 };
 
 // Up to two query heads per workgroup the kernel is held to 256 registers, so that two workgroups share
@@ -59,6 +61,12 @@ struct PrefillArgs {
 // blocks: best when a launch runs many workgroups per CU one after the other).  WAVES = 8: 128 positions, one
 // workgroup per CU, every K/V stage fetched and written to LDS once for eight wavefronts instead of four (best
 // when every workgroup has a long row of stages, or the launch is a single round of workgroups).
+//
+// Measured and not kept: the blocks of a wavefront as a software pipeline - the scores of block n + 1 issued
+// before the softmax of block n, K one stage ahead of V in a ring of three LDS stages, matrix and vector
+// instructions interleaved by scheduling groups (one basic block per mask variant).  Same results, 2 % slower:
+// what bounded this kernel was not the dependency chain inside a wavefront but the fabric - see the workgroup
+// order below.
 template <int D, int G, bool GEN, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void prefill_attn_kernel(PrefillArgs a) {
   constexpr int kPThreads = WAVES * 64;
@@ -72,8 +80,22 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int c = lane & 15, g = lane >> 4;
-  const int pb = gridDim.x - 1 - blockIdx.x;  // long rows first
-  const int hg = blockIdx.y, b = blockIdx.z;
+  // Workgroup ids are dealt round-robin to the eight XCDs.  All position blocks of one (sequence, head group) go to
+  // the same XCD, one pair after the other, so that the pair's keys and values (re-read by every position block)
+  // stay in that XCD's L2 instead of coming over the fabric once per workgroup.
+  // (With fewer pairs than would keep eight XCDs busy the position blocks of a pair are spread over all of them.)
+  int pair, pb;
+  if (a.pairs_by_xcd) {
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    pair = (slot / a.pos_blocks) * kXcdCount + xcd;
+    pb = slot % a.pos_blocks;
+  } else {
+    pair = blockIdx.x / a.pos_blocks;
+    pb = blockIdx.x % a.pos_blocks;
+  }
+  if (pair >= a.n_pairs) return;
+  pb = a.pos_blocks - 1 - pb;  // long rows first
+  const int hg = pair % a.head_groups, b = pair / a.head_groups;
   const int h0 = hg * G, hk = h0 / a.group;
   const int start = a.start ? max(a.start[b], 0) : 0;
   const int p0 = pb * kPosPerWg;
@@ -179,20 +201,11 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
   }
 
   const int n_stages = (k_end + kStageKeys - 1) / kStageKeys;
-  load_stage(0);
-  store_stage(0, 0);
-  __syncthreads();
-
-  // One block of 32 keys for this wavefront.  DIAG: some key of the block may lie behind a query of the
-  // wavefront (the block touches the diagonal, or the end of the cache); every other block skips the
-  // masks, which are a third of the softmax instructions.  The scale is folded into the exponent's
-  // argument: p = exp2(s * scale - m) with m the running maximum of s * scale.
   const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
-  auto block = [&](int buf, int sub, int kb, auto diag_c) __attribute__((always_inline)) {
-    constexpr bool DIAG = decltype(diag_c)::value;
-    const _Float16 *kst_l = &ks[buf][sub * 32 * D];
-    // ---- S^T = K . Q^T for two tiles of 16 keys ----
-    float4_t sc[G][2];
+
+  // ---- the three parts of a block of 32 keys for this wavefront ---------------------------------------------
+  // scores S^T = K . Q^T of the 32 keys at rows `row0` of the K stage `kst_l`
+  auto scores = [&](const _Float16 *kst_l, float4_t (&sc)[G][2]) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < G; ++t) sc[t][0] = sc[t][1] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -205,8 +218,15 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
         for (int t = 0; t < G; ++t)
           sc[t][tk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][kk], sc[t][tk], 0, 0, 0);
       }
-    // ---- mask, online softmax ----
-    half8_t pf[G];
+  };
+  // mask + online softmax of a block's scores -> probabilities in the B layout of the second product.
+  // DIAG: some key of the block may lie behind a query of the wavefront (the block touches the diagonal, or the
+  // end of the cache); every other block skips the masks, which are a third of the softmax instructions.  The
+  // scale is folded into the exponent's argument: p = exp2(s * scale - m) with m the running maximum of s * scale.
+  auto softmax = [&](const float4_t (&sc)[G][2], int kb, half8_t (&pf)[G], auto diag_c) __attribute__((always_inline)) {
+    constexpr bool DIAG = decltype(diag_c)::value;
+    bool moved[G];
+    float mnew[G];
 #pragma unroll
     for (int t = 0; t < G; ++t) {
       float x[8];
@@ -229,10 +249,12 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
       // The running maximum moves only when a block exceeds it by more than 8 (a factor 256): until then
       // the exponents stay <= 8, p <= 256 keeps its 11 bits in fp16 whatever its magnitude, and the block
       // rescales nothing - with a maximum that follows every block, most blocks of a row's first few
-      // hundred keys pay 4 DT multiplications per query tile.
+      // hundred keys pay 4 DT multiplications per query tile.  (A maximum that lags makes every p larger, never
+      // smaller: nothing that the exact maximum would keep is flushed.)
       const float mxs = mx * a.scale_log2e;
-      const bool moved = __any(mxs > m[t] + 8.0f);
-      const float mn = moved ? fmaxf(m[t], mxs) : m[t];
+      moved[t] = __any(mxs > m[t] + 8.0f);
+      const float mn = moved[t] ? fmaxf(m[t], mxs) : m[t];
+      mnew[t] = mn;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         float p = __builtin_amdgcn_exp2f(__builtin_fmaf(x[j], a.scale_log2e, -mn));
@@ -242,17 +264,23 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
         }
         pf[t][j] = static_cast<_Float16>(p);
       }
-      if (moved) {
-        const float corr = __builtin_amdgcn_exp2f(m[t] - mn);
+    }
+    // the rescaling, where the maximum moved (rare after a row's first blocks), after all the straight-line work
+#pragma unroll
+    for (int t = 0; t < G; ++t) {
+      if (moved[t]) {
+        const float corr = __builtin_amdgcn_exp2f(m[t] - mnew[t]);
         lsum[t] *= corr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[t][dt] *= corr;
-        m[t] = mn;
+        m[t] = mnew[t];
       }
-      lsum[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pf[t], lsum[t], 0, 0, 0);
     }
-    // ---- O^T += V^T . P^T ----
-    const _Float16 *vst_l = &vs[buf][sub * 32 * D];
+  };
+  // row sums (a product with ones) and O^T += V^T . P^T over the 32 keys at `vst_l`
+  auto accumulate = [&](const _Float16 *vst_l, const half8_t (&pf)[G]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < G; ++t) lsum[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pf[t], lsum[t], 0, 0, 0);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       const half4_t lo = lds_v_tr<D>(vst_l, 4 * g, dt * 16, c);
@@ -262,6 +290,18 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
       for (int t = 0; t < G; ++t)
         o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][dt], 0, 0, 0);
     }
+  };
+
+  load_stage(0);
+  store_stage(0, 0);
+  __syncthreads();
+
+  auto block = [&](int buf, int sub, int kb, auto diag_c) __attribute__((always_inline)) {
+    float4_t sc[G][2];
+    half8_t pf[G];
+    scores(&ks[buf][sub * 32 * D], sc);
+    softmax(sc, kb, pf, diag_c);
+    accumulate(&vs[buf][sub * 32 * D], pf);
   };
 
   for (int s = 0; s < n_stages; ++s) {
@@ -301,13 +341,24 @@ __global__ __launch_bounds__(WAVES * 64, (WAVES == 4 && G <= 2) ? 2 : 1) void pr
 }
 
 template <int D, bool GEN>
-int launch_prefill(const PrefillArgs &a, int B, int G, hipStream_t st) {
+int launch_prefill(const PrefillArgs &a_in, int B, int G, hipStream_t st) {
+  const PrefillArgs &a0 = a_in;
   // eight wavefronts per workgroup where every workgroup has all keys to go through (no causal rule), or where
   // the launch is one round of workgroups anyway; G = 4 keeps four (its registers leave no room for eight)
-  const int64_t wgs8 = static_cast<int64_t>((a.S + 127) / 128) * (a.Hq / G) * B;
-  const bool eight = G <= 2 && ((GEN && !a.causal) || wgs8 <= device_cu_count());
+  const int64_t wgs8 = static_cast<int64_t>((a0.S + 127) / 128) * (a0.Hq / G) * B;
+  const bool eight = G <= 2 && ((GEN && !a0.causal) || wgs8 <= device_cu_count());
   const int pos = eight ? 128 : 64;
-  const dim3 grid((a.S + pos - 1) / pos, a.Hq / G, B);
+  PrefillArgs a = a_in;
+  a.pos_blocks = (a.S + pos - 1) / pos;
+  a.head_groups = a.Hq / G;
+  a.n_pairs = a.head_groups * B;
+  // a pair per XCD at a time needs enough pairs to go round: whole rounds of eight, or so many that a short last
+  // round does not matter
+  a.pairs_by_xcd = (a.n_pairs % kXcdCount == 0 || a.n_pairs >= 4 * kXcdCount) ? 1 : 0;
+  const int64_t wgs = a.pairs_by_xcd ? static_cast<int64_t>((a.n_pairs + kXcdCount - 1) / kXcdCount * kXcdCount) * a.pos_blocks
+                                     : static_cast<int64_t>(a.n_pairs) * a.pos_blocks;
+  if (wgs > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
+  const dim3 grid(static_cast<unsigned>(wgs));
   if (eight) {
     if (G == 2) hipLaunchKernelGGL((prefill_attn_kernel<D, 2, GEN, 8>), grid, dim3(512), 0, st, a);
     else hipLaunchKernelGGL((prefill_attn_kernel<D, 1, GEN, 8>), grid, dim3(512), 0, st, a);

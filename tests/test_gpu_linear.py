@@ -339,6 +339,43 @@ def test_packed_gemm_256x128_tile(M, K, N):
     np.testing.assert_allclose(glu, wantg, rtol=0, atol=2e-5)
 
 
+@pytest.mark.parametrize("order", [(0, 0), (1, 16), (4, 4), (8, 8), (2, 32), (16, 1), (3, 5)])
+@pytest.mark.parametrize("M,K,N", [(1000, 256, 2100), (2200, 128, 530), (128, 384, 256)])
+def test_packed_gemm_tile_order_over_the_xcds(order, M, K, N):
+    """The 256 x 128 tile handed to the XCDs in rectangles of A weight-row blocks x B blocks of x rows, every
+    rectangle shape forced on grids it does not divide (rectangles that hang over both edges, fewer rectangles than
+    XCDs, a single tile): every output element is written exactly once with the bits of the plain order."""
+    rng = np.random.default_rng(M + K + N)
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    b = h16(0.05 * rng.standard_normal(N))
+    with gu.linear_tuned(100000, 0, 0, 256):
+        plain = gu.linear_f16_packed(x, w, b)
+    with gu.linear_tuned(100000 + 256 * order[0] + order[1], 0, 0, 256):
+        out = gu.linear_f16_packed(x, w, b)
+    np.testing.assert_array_equal(out, plain)
+    x32, w32 = x.astype(np.float32), w.astype(np.float32)
+    want = port.linear(x32, w32, b.astype(np.float32))
+    assert np.all(np.abs(out - want) <= _order_bound(x32, w32, K, b.astype(np.float32)))
+
+
+def test_packed_gemm_default_order_at_a_prefill_shape():
+    """A shape whose default is the rectangle order (x does not fit an XCD's L2): 8192 rows through 2048 -> 4096,
+    against the plain order bit for bit and the oracle on a sample of rows."""
+    rng = np.random.default_rng(77)
+    M, K, N = 8192, 2048, 4096
+    x = h16(rng.standard_normal((M, K)))
+    w = h16(0.02 * rng.standard_normal((N, K)))
+    out = gu.linear_f16_packed(x, w)
+    with gu.linear_tuned(100000, 0, 0, 256):
+        plain = gu.linear_f16_packed(x, w)
+    np.testing.assert_array_equal(out, plain)
+    rows = np.unique(np.concatenate([np.arange(0, M, 257), [M - 1]]))
+    x32, w32 = x[rows].astype(np.float32), w.astype(np.float32)
+    want = port.linear(x32, w32)
+    assert np.all(np.abs(out[rows] - want) <= _order_bound(x32, w32, K))
+
+
 @pytest.mark.parametrize("tiles,M,K,N", [(1, 512, 2048, 2048), (1, 512, 6144, 2048), (2, 512, 2048, 4096), (1, 130, 512, 200),
                                          (2, 333, 1024, 1000), (1, 65, 1536, 64)])
 def test_packed_gemm_k_in_two_halves(tiles, M, K, N):

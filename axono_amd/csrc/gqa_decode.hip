@@ -432,6 +432,43 @@ __device__ __forceinline__ void write_zero_rows(const DecodeArgs &a, int b, int 
     stf(static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.Hq + hg * G) * D + o, 0.0f);
 }
 
+// The merge of the n_valid partial states a (sequence, head) was cut into, for output element d of the head:
+//   out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M),  M = max_s m_s,
+// summed in range order - the arithmetic of gqa_decode_merge_kernel, so both forms of the merge give the same bits.
+// The partials were written past the local caches by other workgroups and are read the same way: a load costs
+// a trip to the memory side, so all loads of up to NB ranges are in flight before the first is used (one trip
+// for the 32 ranges a single long sequence is cut into; ranges beyond NB are fetched one at a time).
+template <int NB>
+__device__ __forceinline__ float merge_ranges(const float *ml, const float *pa, int n_valid, int D) {
+  float pm[NB], pl[NB], pv[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int sidx = min(i, n_valid - 1);
+    pm[i] = ld_agent(ml + 2 * sidx);
+    pl[i] = ld_agent(ml + 2 * sidx + 1);
+    pv[i] = ld_agent(pa + static_cast<int64_t>(sidx) * D);
+  }
+  float mx = kNegBig;
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+    if (i < n_valid) mx = fmaxf(mx, pm[i]);
+  for (int s = NB; s < n_valid; ++s) mx = fmaxf(mx, ld_agent(ml + 2 * s));
+  float lsum = 0.0f, asum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    if (i >= n_valid) continue;
+    const float w = __builtin_amdgcn_exp2f(pm[i] - mx);
+    lsum = __builtin_fmaf(pl[i], w, lsum);
+    asum = __builtin_fmaf(pv[i], w, asum);
+  }
+  for (int s = NB; s < n_valid; ++s) {
+    const float w = __builtin_amdgcn_exp2f(ld_agent(ml + 2 * s) - mx);
+    lsum = __builtin_fmaf(ld_agent(ml + 2 * s + 1), w, lsum);
+    asum = __builtin_fmaf(ld_agent(pa + static_cast<int64_t>(s) * D), w, asum);
+  }
+  return lsum > 0.0f ? asum / lsum : 0.0f;
+}
+
 // Keys [s0, s1) of sequence b for the G query heads of head group hg: range number `split` of the
 // `n_valid` non-empty ranges this sequence is cut into in this launch.  The only range of a sequence
 // writes the result itself when `direct_ok`; otherwise the range leaves a partial state and (fused
@@ -642,35 +679,8 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
     const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
     const float *ml = a.part_ml + bh * a.split_stride * 2;
     const float *pa = a.part_acc + bh * a.split_stride * D + d;
-    // eight ranges at a time, every load of a batch in flight before the first is used (the loads
-    // go past the local caches: one at a time they would cost a memory round trip each)
-    float mx = kNegBig, lsum = 0.0f, asum = 0.0f;
-    for (int s0m = 0; s0m < n_valid; s0m += 8) {
-      float pm[8], pl[8], pv[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int sidx = min(s0m + i, n_valid - 1);
-        pm[i] = ld_agent(ml + 2 * sidx);
-        pl[i] = ld_agent(ml + 2 * sidx + 1);
-        pv[i] = ld_agent(pa + static_cast<int64_t>(sidx) * D);
-      }
-      float bm = mx;
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (s0m + i < n_valid) bm = fmaxf(bm, pm[i]);
-      const float keep = __builtin_amdgcn_exp2f(mx - bm);
-      lsum *= keep;
-      asum *= keep;
-      mx = bm;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (s0m + i >= n_valid) continue;
-        const float w = __builtin_amdgcn_exp2f(pm[i] - mx);
-        lsum = __builtin_fmaf(pl[i], w, lsum);
-        asum = __builtin_fmaf(pv[i], w, asum);
-      }
-    }
-    stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
+    const float res = n_valid <= 8 ? merge_ranges<8>(ml, pa, n_valid, D) : merge_ranges<32>(ml, pa, n_valid, D);
+    stf(static_cast<T *>(a.out) + bh * D + d, res);
   }
 }
 
@@ -732,35 +742,8 @@ __device__ __forceinline__ void finish_range(const DecodeArgs &a, int b, int hg,
     const int64_t bh = static_cast<int64_t>(b) * a.Hq + h0 + g;
     const float *ml = a.part_ml + bh * a.split_stride * 2;
     const float *pa = a.part_acc + bh * a.split_stride * D + d;
-    // eight ranges at a time, every load of a batch in flight before the first is used (the loads
-    // go past the local caches: one at a time they would cost a memory round trip each)
-    float mx = kNegBig, lsum = 0.0f, asum = 0.0f;
-    for (int s0m = 0; s0m < n_valid; s0m += 8) {
-      float pm[8], pl[8], pv[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int sidx = min(s0m + i, n_valid - 1);
-        pm[i] = ld_agent(ml + 2 * sidx);
-        pl[i] = ld_agent(ml + 2 * sidx + 1);
-        pv[i] = ld_agent(pa + static_cast<int64_t>(sidx) * D);
-      }
-      float bm = mx;
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (s0m + i < n_valid) bm = fmaxf(bm, pm[i]);
-      const float keep = __builtin_amdgcn_exp2f(mx - bm);
-      lsum *= keep;
-      asum *= keep;
-      mx = bm;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (s0m + i >= n_valid) continue;
-        const float w = __builtin_amdgcn_exp2f(pm[i] - mx);
-        lsum = __builtin_fmaf(pl[i], w, lsum);
-        asum = __builtin_fmaf(pv[i], w, asum);
-      }
-    }
-    stf(static_cast<T *>(a.out) + bh * D + d, lsum > 0.0f ? asum / lsum : 0.0f);
+    const float res = n_valid <= 8 ? merge_ranges<8>(ml, pa, n_valid, D) : merge_ranges<32>(ml, pa, n_valid, D);
+    stf(static_cast<T *>(a.out) + bh * D + d, res);
   }
 }
 

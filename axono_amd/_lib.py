@@ -87,6 +87,7 @@ PROTOTYPES = {
     "axhip_linear_f16_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64]),
     "axhip_linear_f16_tune": (None, [c_i, c_i, c_i, c_i]),
     "axhip_linear_f16": (c_i, [c_vp, c_i, c_vp, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_vp, c_sz, c_vp]),
+    "axhip_linear_f32": (c_i, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "axhip_linear_f16_packed_bytes": (c_sz, [c_i64, c_i64]),
     "axhip_linear_f16_pack": (c_i, [c_vp, c_vp, c_i64, c_i64, c_i, c_vp]),
     "axhip_linear_f16_packed": (c_i, [c_vp, c_i, c_vp, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_i, c_vp]),

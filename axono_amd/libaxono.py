@@ -452,9 +452,6 @@ def _linear_impl(x: Tensor, weight: Tensor, bias: Tensor | None, out_dtype: Data
     if x.is_hip != weight.is_hip or (has_b and bias.is_hip != x.is_hip):
         raise RuntimeError("linear: 输入张量不在同一设备上")
     _need_hip(op, x, weight, bias if has_b else None)
-    if weight.dtype != DataType.FLOAT16 or x.dtype not in _FLOATS or (has_b and bias.dtype != DataType.FLOAT16):
-        # only the fp16-weight path of the decode step is provided on hip
-        raise RuntimeError("linear: 数据类型不一致")
     if x.ndim < 1 or weight.ndim != 2:
         raise AxhipError(op, Status.INVALID_ARGUMENT)
     k = x.shape[-1]
@@ -462,6 +459,19 @@ def _linear_impl(x: Tensor, weight: Tensor, bias: Tensor | None, out_dtype: Data
     if weight.shape[1] != k or (has_b and (bias.ndim != 1 or bias.shape[0] != n)):
         raise AxhipError(op, Status.SHAPE_MISMATCH)
     rows = x.num_elements // k if k else 0
+    if weight.dtype == DataType.FLOAT32:
+        # a Linear that has not been cast to fp16: the reference's FLOAT32 branch (linear.cu:178-251), x and bias
+        # FLOAT32 like the weight (linear.cu:178-181)
+        if x.dtype != DataType.FLOAT32 or (has_b and bias.dtype != DataType.FLOAT32) or \
+                (out_dtype is not None and DataType(out_dtype) != DataType.FLOAT32):
+            raise RuntimeError("linear: 数据类型不一致")
+        out = _new(DataType.FLOAT32, x.shape[:-1] + [n], x)
+        check(_lib_().axhip_linear_f32(x.data_ptr, weight.data_ptr, bias.data_ptr if has_b else None, out.data_ptr,
+                                       rows, k, n, current_stream()), op)
+        return out
+    if weight.dtype != DataType.FLOAT16 or x.dtype not in _FLOATS or (has_b and bias.dtype != DataType.FLOAT16):
+        # FLOAT64 weights (the reference's third branch) are not provided on hip
+        raise RuntimeError("linear: 数据类型不一致")
     odt = DataType(out_dtype) if out_dtype is not None else DataType.FLOAT32
     out = _new(odt, x.shape[:-1] + [n], x)
     lib = _lib_()

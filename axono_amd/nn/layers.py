@@ -10,8 +10,9 @@ from .module import Module
 
 
 class Linear(Module):
-    """y = x @ W^T + b.  Weights are created FLOAT32 like the reference's; the hip operator is the
-    fp16-weight path, so call `cast_linear_fp16()` (on the layer or any parent) before forward."""
+    """y = x @ W^T + b.  Weights are created FLOAT32 like the reference's and forward then runs the plain fp32
+    operator; after `cast_linear_fp16()` (on the layer or any parent) it runs the fp16-weight kernels of the
+    decode path over a packed copy of the weight."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device: str | None = None):
         super().__init__()
@@ -32,9 +33,7 @@ class Linear(Module):
     def forward(self, x: Tensor) -> Tensor:
         w = self._parameters["weight"]
         b = self._parameters["bias"]
-        if w.dtype != DataType.FLOAT16:
-            raise RuntimeError("linear: the hip operator takes FLOAT16 weights; call cast_linear_fp16() first")
-        if w.is_hip and x.num_elements:
+        if w.is_hip and w.dtype == DataType.FLOAT16 and x.num_elements:
             # The kernels read a packed copy of the weight.  It is made on first use and again whenever
             # the weight's storage was replaced or written since (load_state_dict, copy_from,
             # copy_from_numpy and fill* write in place and bump the storage's version), so forward

@@ -403,6 +403,13 @@ AXHIP_API int axhip_linear_f16(const void *x, int x_dtype, const void *w, const 
                                void *out, int out_dtype, int64_t M, int64_t K, int64_t N,
                                void *workspace, size_t workspace_bytes, axhip_stream stream);
 
+/* out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]), every operand FLOAT32: the Linear of a module whose weights have
+ * not been cast to fp16, ops::cuda::Linear's FLOAT32 branch (src/ops/cuda/linear.cu:178-251, cublasSgemm).
+ * fp32 products and sums in K order on the fp32 matrix instruction; bias may be NULL.  The FLOAT64 branch of
+ * the reference has no counterpart here.  Not on the decode path and not tuned. */
+AXHIP_API int axhip_linear_f32(const float *x, const float *w, const float *bias, float *out, int64_t M,
+                               int64_t K, int64_t N, axhip_stream stream);
+
 /* Packed weights for skinny M.  axhip_linear_f16_pack re-orders a row-major FLOAT16 W [N,K] once
  * into MFMA fragment order (1 KiB blocks of 16 rows x 32 K, consecutive along K; rows and K
  * zero-padded to whole blocks) into a buffer of axhip_linear_f16_packed_bytes(N,K) bytes, so that

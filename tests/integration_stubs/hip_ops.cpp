@@ -225,21 +225,30 @@ Status RmsNorm(const core::Context &, const Tensor &x, const Tensor &weight, flo
 }
 
 // src/ops/cuda/linear.cu:76-176, the fp16-weight branch: x FLOAT32 (rounded to fp16 on load, linear.cu:110) or
-// FLOAT16, weight FLOAT16 [out_f, k], bias FLOAT16 (or empty), result FLOAT32.  The other weight types stay with
-// the reference's own device code.
+// FLOAT16, weight FLOAT16 [out_f, k], bias FLOAT16 (or empty), result FLOAT32; FLOAT32 weights go to the plain fp32
+// operator.  FLOAT64 weights have no hip counterpart.
 Status Linear(const core::Context &, const Tensor &x, const Tensor &weight, const Tensor &bias, Tensor &result) {
   if (x.ndim() < 1 || weight.ndim() != 2) return Status::INVALID_ARGUMENT;
   const size_t k = x.shape().back(), out_f = weight.shape()[0];
   if (weight.shape()[1] != k) return Status::SHAPE_MISMATCH;
   const bool has_bias = bias.num_elements() != 0;
   if (has_bias && (bias.ndim() != 1 || bias.shape()[0] != out_f)) return Status::SHAPE_MISMATCH;
-  if (weight.dtype() != DataType::FLOAT16 || !IsFloat(x)) return Status::UNSUPPORTED_TYPE;
-  if (has_bias && bias.dtype() != DataType::FLOAT16) return Status::UNSUPPORTED_TYPE;
   core::Shape out_shape = x.shape();
   out_shape.back() = out_f;
+  const int64_t rows = static_cast<int64_t>(x.num_elements() / k);
+  if (weight.dtype() == DataType::FLOAT32) {
+    // the FLOAT32 branch (linear.cu:178-251): x and bias of the weight's type
+    if (x.dtype() != DataType::FLOAT32 || (has_bias && bias.dtype() != DataType::FLOAT32)) return Status::UNSUPPORTED_TYPE;
+    Status st32 = result.Resize(out_shape);
+    if (st32 != Status::OK) return st32;
+    return S(axhip_linear_f32(x.data<float>(), weight.data<float>(), has_bias ? bias.data<float>() : nullptr,
+                              result.data<float>(), rows, static_cast<int64_t>(k), static_cast<int64_t>(out_f),
+                              axhip_current_stream()));
+  }
+  if (weight.dtype() != DataType::FLOAT16 || !IsFloat(x)) return Status::UNSUPPORTED_TYPE;
+  if (has_bias && bias.dtype() != DataType::FLOAT16) return Status::UNSUPPORTED_TYPE;
   Status st = result.Resize(out_shape);
   if (st != Status::OK) return st;
-  const int64_t rows = static_cast<int64_t>(x.num_elements() / k);
   return S(axhip_linear_f16(x.data(), DT(x), weight.data(), has_bias ? bias.data() : nullptr, result.data(), DT(result),
                             rows, static_cast<int64_t>(k), static_cast<int64_t>(out_f), /*workspace=*/nullptr, 0,
                             axhip_current_stream()));

@@ -432,3 +432,37 @@ def test_packed_linear_random_shapes(seed):
     got16 = gu.linear_f16_packed(x, w, b, out_dtype=np.float16).astype(np.float32)
     ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
     assert np.all(np.abs(got16 - want) <= 0.5 * ulp + 1e-5 + 4 * np.sqrt(K) * 2.0 ** -24 * mag), (M, K, N)
+
+
+# ---- fp32 weights: a Linear that has not been cast (src/ops/cuda/linear.cu:178-251) ------------------------------
+def linear_f32(x, w, b=None):
+    M, K = x.shape
+    N = w.shape[0]
+    dx, dw = gu.dev(x), gu.dev(w)
+    db = gu.dev(b) if b is not None else None
+    do = gu.DeviceBuffer(M * N * 4)
+    gu._run("axhip_linear_f32", dx.ptr, dw.ptr, db.ptr if db else None, do.ptr, M, K, N, None)
+    gu.synchronize()
+    return do.download(np.float32, (M, N))
+
+
+@pytest.mark.parametrize("M,K,N", [(8, 64, 32), (1, 2048, 2048), (16, 2048, 4096), (3, 72, 50), (130, 264, 190),
+                                   (65, 37, 129), (512, 1024, 300), (64, 32, 64)])
+def test_linear_f32_against_the_oracle(M, K, N):
+    """fp32 x, W and bias: fp32 products summed in K order, so against the oracle's sequential fp32 sum only
+    the rounding of partial sums differs: 1e-5 + 8 sqrt(K) 2^-24 sum|terms| (products are no longer exact as
+    in the fp16 case, hence the factor 8 where the fp16 tests have 4).  K = 37 takes the scalar loads."""
+    rng = np.random.default_rng(M * 3 + K + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (0.05 * rng.standard_normal((N, K))).astype(np.float32)
+    b = (0.05 * rng.standard_normal(N)).astype(np.float32)
+    want = port.linear(x, w, b)
+    bound = 1e-5 + 8 * np.sqrt(K) * 2.0 ** -24 * (np.abs(x) @ np.abs(w).T + np.abs(b))
+    got = linear_f32(x, w, b)
+    assert np.all(np.abs(got - want) <= bound), float(np.abs(got - want).max())
+    got0 = linear_f32(x, w)
+    assert np.all(np.abs(got0 - port.linear(x, w)) <= bound)
+    l = gu.lib()
+    assert l.axhip_linear_f32(None, None, None, None, 4, 0, 8, None) == 1
+    assert l.axhip_linear_f32(None, None, None, None, 4, 8, 8, None) == 7
+    assert l.axhip_linear_f32(None, None, None, None, 0, 8, 8, None) == 0

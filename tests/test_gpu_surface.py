@@ -178,6 +178,28 @@ def test_linear_fp16_module_path(hip_env):
     np.testing.assert_allclose(nb(Tensor.from_numpy(x_np)).to_numpy(), want - b_np.astype(np.float16).astype(np.float32), rtol=0, atol=2e-5)
 
 
+def test_linear_fp32_module_path_before_the_cast(hip_env):
+    """nn.Linear as created (FLOAT32 weight and bias): forward runs the fp32 operator, like the reference's Linear
+    before cast_linear_fp16() (tests/nn/test_layers.py of the reference compares it with x @ W^T + b)."""
+    rng = np.random.default_rng(2)
+    x_np = rng.normal(size=(5, 3, 64)).astype(np.float32)
+    w_np = (rng.normal(size=(32, 64)) * 0.05).astype(np.float32)
+    b_np = (rng.normal(size=(32,)) * 0.05).astype(np.float32)
+    lin = nn.Linear(64, 32, device="hip")
+    lin.load_state_dict({"weight": w_np, "bias": b_np})
+    assert lin.weight.dtype == DataType.FLOAT32
+    out = lin(Tensor.from_numpy(x_np))
+    assert out.dtype == DataType.FLOAT32 and out.shape == [5, 3, 32]
+    want = port.linear(x_np.reshape(15, 64), w_np, b_np).reshape(5, 3, 32)
+    np.testing.assert_allclose(out.to_numpy(), want, rtol=0, atol=1e-5)
+    nb = nn.Linear(64, 32, bias=False, device="hip")
+    nb.load_state_dict({"weight": w_np})
+    np.testing.assert_allclose(nb(Tensor.from_numpy(x_np)).to_numpy(), want - b_np, rtol=0, atol=1e-5)
+    # fp16 activations with fp32 weights are a dtype mismatch, as in the reference (linear.cu:178-181)
+    with pytest.raises(RuntimeError):
+        lin(Tensor.from_numpy(x_np.astype(np.float16)))
+
+
 def test_linear_follows_weights_written_after_a_forward(hip_env):
     """A Linear that has run once keeps a packed copy of its weight; load_state_dict / copy_from /
     copy_from_numpy write the weight in place, and the next forward must use the new values (the

@@ -93,6 +93,7 @@ PROTOTYPES = {
     "axhip_linear_f16_packed": (c_i, [c_vp, c_i, c_vp, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_i, c_vp]),
     "axhip_embedding": (c_i, [c_vp, c_i, c_vp, c_vp, c_i, c_i64, c_i64, c_i64, c_vp]),
     "axhip_argmax": (c_i, [c_vp, c_vp, c_i, c_i64, c_i64, c_vp]),
+    "axhip_prefill_attention_tune": (None, [c_i]),
     "axhip_prefill_attention": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),
     "axhip_gqa_decode_qkv": (c_i, [c_vp, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i, c_i, c_vp,
                                    c_vp, c_vp, c_vp, c_vp, c_sz, c_i, c_i, c_i, c_i, c_i, c_i, c_i, c_vp]),

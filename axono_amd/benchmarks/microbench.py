@@ -366,6 +366,8 @@ def main(argv=None):
     ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "gqa-paged", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
     ap.add_argument("--zero-data", action="store_true",
                     help="prefill-attn, linear-packed: all-zero operands (how much of the time is the power the data costs)")
+    ap.add_argument("--tile-order", default="", help="linear-packed: 'plain' or 'A:B' rectangles of 256 x 128 GEMM tiles per XCD")
+    ap.add_argument("--by-xcd", type=int, default=-1, help="prefill-attn: 1 / 0 force the workgroup order over the XCDs")
     ap.add_argument("--B", type=int, default=32)
     ap.add_argument("--L", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=100)
@@ -415,6 +417,7 @@ def main(argv=None):
             for L in (1024, 2048, 8192, 32768, 131072):
                 bench_gqa(lib, 1, L, min(args.steps, 100), fp32=fp32, token_major=True, tag="gqa_single_sequence")
     elif args.what == "prefill-attn":
+        lib.axhip_prefill_attention_tune(args.by_xcd)
         for S in (1024, 4096, 16384):
             bench_prefill_attn(lib, max(1, min(args.B, 65536 // S)), S, max(5, min(args.steps, 20)))
         for S in (4096, 16384):
@@ -428,9 +431,12 @@ def main(argv=None):
         lib.axhip_linear_f16_tune(0, args.nt, args.waves, args.gemm_rows)
         bench_linear(lib, Ms=(args.M,) if args.M else (1, 16, 32, 512), rot=args.rot)
     elif args.what == "linear-packed":
-        lib.axhip_linear_f16_tune(0, args.nt, args.waves, args.gemm_rows)
+        order = 0
+        if args.tile_order:
+            order = 100000 if args.tile_order == "plain" else 100000 + 256 * int(args.tile_order.split(":")[0]) + int(args.tile_order.split(":")[1])
+        lib.axhip_linear_f16_tune(order, args.nt, args.waves, args.gemm_rows)
         bench_linear(lib, shapes=[(2048, 2048), (2048, 4096), (2048, 12288), (6144, 2048), (2048, 151936)],
-                     Ms=(args.M,) if args.M else (1, 16, 32, 512, 4096), packed=True, rot=args.rot)
+                     Ms=(args.M,) if args.M else (1, 16, 32, 512, 4096), packed=True, rot=args.rot, steps=min(args.steps, 50))
 
 
 if __name__ == "__main__":

@@ -32,6 +32,7 @@ namespace {
 
 constexpr int kStageKeys = 64;  // keys per LDS stage
 constexpr int kXcdCount = 8;
+int g_pairs_by_xcd = -1;  // measurement hook: 0 / 1 force the workgroup order, -1 = by pair count
 constexpr float kMasked = -1.0e30f;
 
 struct PrefillArgs {
@@ -355,6 +356,7 @@ int launch_prefill(const PrefillArgs &a_in, int B, int G, hipStream_t st) {
   // a pair per XCD at a time needs enough pairs to go round: whole rounds of eight, or so many that a short last
   // round does not matter
   a.pairs_by_xcd = (a.n_pairs % kXcdCount == 0 || a.n_pairs >= 4 * kXcdCount) ? 1 : 0;
+  if (g_pairs_by_xcd >= 0) a.pairs_by_xcd = g_pairs_by_xcd;  // measurement hook
   const int64_t wgs = a.pairs_by_xcd ? static_cast<int64_t>((a.n_pairs + kXcdCount - 1) / kXcdCount * kXcdCount) * a.pos_blocks
                                      : static_cast<int64_t>(a.n_pairs) * a.pos_blocks;
   if (wgs > INT32_MAX) return AXHIP_INVALID_ARGUMENT;
@@ -378,6 +380,9 @@ int launch_prefill(const PrefillArgs &a_in, int B, int G, hipStream_t st) {
 using namespace axhip;
 
 extern "C" {
+
+// Measurement hook: the order in which workgroups are handed to the XCDs (see the kernel).
+AXHIP_API void axhip_prefill_attention_tune(int pairs_by_xcd) { g_pairs_by_xcd = pairs_by_xcd < 0 ? -1 : (pairs_by_xcd ? 1 : 0); }
 
 AXHIP_API int axhip_prefill_attention(const void *q, const void *k_cache, const void *v_cache,
                                       const int32_t *start, void *out, int dtype, int B, int S, int Hq,

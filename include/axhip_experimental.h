@@ -33,6 +33,11 @@ AXHIP_API void axhip_gqa_decode_tune(int target_workgroups, int force_splits);
  * picks by problem size). */
 AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_waves, int gemm_rows);
 
+/* Prefill / general fp16 attention on the matrix cores: 1 = all position blocks of a (sequence, head group) run on
+ * one XCD, pair after pair (their keys and values stay in that XCD's L2), 0 = position blocks dealt round-robin over
+ * the XCDs, -1 = the default (by XCD when the pairs go round the eight XCDs evenly or there are at least 32). */
+AXHIP_API void axhip_prefill_attention_tune(int pairs_by_xcd);
+
 #ifdef __cplusplus
 }
 #endif

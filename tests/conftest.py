@@ -37,3 +37,4 @@ def _default_tuning_after_gpu_tests(request):
     l = _lib.load()
     l.axhip_gqa_decode_tune(0, 0)
     l.axhip_linear_f16_tune(0, 0, 0, 0)
+    l.axhip_prefill_attention_tune(-1)

@@ -514,6 +514,38 @@ def test_prefill_attention_peak_next_to_a_long_plateau(gap, peak_at):
     assert abs((sc[peak_at] - np.median(sc)) - gap) < 0.05
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,S", [(3, 4, 2, 300), (8, 2, 2, 130), (5, 16, 8, 200)])
+def test_prefill_attention_workgroup_order_over_the_xcds(B, Hq, Hkv, S):
+    """The two orders in which the workgroups of a launch are handed to the XCDs (all position blocks of a pair on
+    one XCD, or dealt round-robin), each forced on pair counts that do and do not go round eight XCDs evenly: same
+    bits, every output row written, and the oracle on a few rows."""
+    rng = np.random.default_rng(B * 100 + S)
+    D = 128
+    q = rng.standard_normal((B, S, Hq, D)).astype(np.float16)
+    kc = rng.standard_normal((B, Hkv, S, D)).astype(np.float16)
+    vc = rng.standard_normal((B, Hkv, S, D)).astype(np.float16)
+    dq, dk, dv = (gu.dev(a) for a in (q, kc, vc))
+    outs = []
+    l = gu.lib()
+    try:
+        for order in (0, 1):
+            l.axhip_prefill_attention_tune(order)
+            out = gu.DeviceBuffer(q.nbytes)
+            gu.check(l.axhip_fill_zero(out.ptr, q.nbytes), "fill")
+            gu._run("axhip_prefill_attention", dq.ptr, dk.ptr, dv.ptr, None, out.ptr, gu.F16, B, S, Hq, Hkv, D, S, None)
+            gu.synchronize()
+            outs.append(out.download(np.uint16, q.shape))
+    finally:
+        l.axhip_prefill_attention_tune(-1)
+    np.testing.assert_array_equal(outs[0], outs[1])
+    got = outs[1].view(np.float16).astype(np.float32)
+    for b in (0, B - 1):
+        k = np.ascontiguousarray(np.transpose(kc[b], (1, 0, 2)), dtype=np.float32)
+        v = np.ascontiguousarray(np.transpose(vc[b], (1, 0, 2)), dtype=np.float32)
+        want = port.sdpa(q[b].astype(np.float32), k, v, True)
+        assert np.abs(got[b] - want).max() <= TOL16
+
+
 def test_workgroups_are_dealt_by_length():
     """Very uneven batches under the default plan: one long sequence among short ones, all equal,
     and lengths that leave some of the launch's workgroup slots unused."""

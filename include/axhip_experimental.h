@@ -2,7 +2,9 @@
  * axhip_experimental.h - measurement hooks of libaxhip.so.  NOT part of the drop-in boundary (axhip.h):
  * these entry points exist so that tests can force every kernel variant and benchmarks can sweep plans.
  * They set process-global, unsynchronised state: call them from one thread while no operator call is in
- * flight, and restore the defaults (all arguments 0) afterwards.  No reference counterparts (the
+ * flight, and restore the defaults (all arguments 0) afterwards.  The library as a whole is a single-stream
+ * drop-in in this respect: operator calls themselves are safe from several threads and streams (the merging
+ * launches under distinct ticket lanes, axhip_set_ticket_lane in axhip.h), the hooks here are not.  No reference counterparts (the
  * reference hard-codes its split count, src/ops/cuda/gqa.cu:158-160, and leaves GEMM algorithm choice to
  * cuBLAS, src/ops/cuda/linear.cu:131-138).
  */

@@ -463,7 +463,7 @@ def device_label(reported):
             return f"{gpus[0]} {reported.strip()}"
     except (OSError, subprocess.SubprocessError):
         pass
-    return f"unnamed device {reported.strip()}"
+    return f"(the driver reports no device name) {reported.strip()}"
 
 
 def smoke_parity(lib):

@@ -32,12 +32,15 @@ def step_bytes(cfg: TextConfig, batch: int, context: int) -> int:
     return weights + kv
 
 
-def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) -> list:
+def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, once_copies: int = 8) -> list:
     """Where a decode step goes, kernel by kernel: every kind of launch of the step is captured as a graph
     of that launch for all layers (each layer's own weights and caches, so nothing is served from the
     memory-side cache) and replayed `reps` times between host clock reads.  Rows: calls per step, us per call
     inside such a back-to-back graph, algorithmic bytes per call and the fraction of HBM peak that is.
-    Run it after the timed loop: the attention launches overwrite the cache row at the current length."""
+    The three launches that a step holds once are captured `once_copies` times over, so that the fixed cost of
+    replaying a graph (some 20 us, which a one-node graph would charge to its only node) is spread as it is
+    in the step; the weight of lm_head is 622 MB, more than the memory-side cache holds, so its copies still
+    read HBM.  Run it after the timed loop: the attention launches overwrite the cache row at the current length."""
     from ..core.hip_graph import HIPGraph
     from ..core.tensor import Tensor
     from ..core.types import DataType
@@ -82,11 +85,12 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
          layers(lambda p, i: L.linear_packed(xn, model._packed[p + "mlp.gate_up_proj.weight"], 2 * I,
                                              out_dtype=DataType.FLOAT16, glu=True))),
         ("down Linear 6144->2048", nl, lin_bytes(I, H, 4), layers(lambda p, i: model._linear(act, p + "mlp.down_proj.weight"))),
-        ("lm_head Linear 2048->151936", 1, lin_bytes(H, V, 4), lambda: [model._linear(xn, "embed_tokens.weight")]),
-        ("argmax over 151936", 1, B * V * 4, lambda: [L.argmax(logits)]),
+        ("lm_head Linear 2048->151936", 1, lin_bytes(H, V, 4),
+         lambda: [model._linear(xn, "embed_tokens.weight") for _ in range(once_copies)]),
+        ("argmax over 151936", 1, B * V * 4, lambda: [L.argmax(logits) for _ in range(once_copies)]),
         ("embedding + first RMSNorm", 1, B * H * (2 + 4 + 2),
          lambda: [L.embedding_rms_norm(model._ids, W("embed_tokens.weight"), W("layers.0.input_layernorm.weight"),
-                                       cfg.rms_norm_eps)]),
+                                       cfg.rms_norm_eps) for _ in range(once_copies)]),
     ]
     rows = []
     for name, calls, nbytes, fn in kinds:
@@ -99,7 +103,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10) ->
         for _ in range(reps):
             g.launch_async()
         g.sync()
-        us = (time.perf_counter() - t0) * 1e6 / (reps * calls)
+        us = (time.perf_counter() - t0) * 1e6 / (reps * (calls if calls > 1 else once_copies))
         g.reset()
         rows.append({"kernel": name, "calls_per_step": calls, "us_per_call": round(us, 2),
                      "us_per_step": round(us * calls, 1), "bytes_per_call": int(nbytes),

@@ -50,6 +50,13 @@ Tuning g_tuning;
 constexpr int kTicketSlots = 1 << 16;  // per ticket lane
 __device__ unsigned int g_tickets[AXHIP_TICKET_LANES * kTicketSlots];
 
+// Atomics on one 128-byte line are served one after the other (about 10 ns each on MI355X), and the workgroups
+// of a launch finish together: neighbouring (sequence, head group) pairs therefore take counters 128 bytes
+// apart; the words in between belong to pairs 2048, 4096, ... further on.
+__device__ __forceinline__ unsigned int *ticket_of(int lane_base, int pair) {
+  return &g_tickets[lane_base + (((pair & 2047) << 5) | (pair >> 11))];
+}
+
 // Scratch of the entry point that allocates nothing (axhip_gqa_decode_static): the split partials live here
 // instead of in a caller's workspace.  Every device the library runs on holds its own copy of this array
 // until the process ends.  In host code the array's name is only a stand-in for the symbol: the address
@@ -437,7 +444,7 @@ __device__ __forceinline__ void write_zero_rows(const DecodeArgs &a, int b, int 
 // summed in range order - the arithmetic of gqa_decode_merge_kernel, so both forms of the merge give the same bits.
 // The partials were written past the local caches by other workgroups and are read the same way: a load costs
 // a trip to the memory side, so all loads of up to NB ranges are in flight before the first is used (one trip
-// for the 32 ranges a single long sequence is cut into; ranges beyond NB are fetched one at a time).
+// for the 32 ranges a single long sequence is cut into; ranges beyond NB follow in further rounds of NB loads).
 template <int NB>
 __device__ __forceinline__ float merge_ranges(const float *ml, const float *pa, int n_valid, int D) {
   float pm[NB], pl[NB], pv[NB];
@@ -452,7 +459,14 @@ __device__ __forceinline__ float merge_ranges(const float *ml, const float *pa, 
 #pragma unroll
   for (int i = 0; i < NB; ++i)
     if (i < n_valid) mx = fmaxf(mx, pm[i]);
-  for (int s = NB; s < n_valid; ++s) mx = fmaxf(mx, ld_agent(ml + 2 * s));
+  // more ranges than NB: their maxima, again NB loads at a time
+  for (int s0 = NB; s0 < n_valid; s0 += NB) {
+    float qm[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) qm[i] = ld_agent(ml + 2 * min(s0 + i, n_valid - 1));
+#pragma unroll
+    for (int i = 0; i < NB; ++i) mx = fmaxf(mx, qm[i]);  // (a repeated last range changes no maximum)
+  }
   float lsum = 0.0f, asum = 0.0f;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
@@ -461,10 +475,21 @@ __device__ __forceinline__ float merge_ranges(const float *ml, const float *pa, 
     lsum = __builtin_fmaf(pl[i], w, lsum);
     asum = __builtin_fmaf(pv[i], w, asum);
   }
-  for (int s = NB; s < n_valid; ++s) {
-    const float w = __builtin_amdgcn_exp2f(ld_agent(ml + 2 * s) - mx);
-    lsum = __builtin_fmaf(ld_agent(ml + 2 * s + 1), w, lsum);
-    asum = __builtin_fmaf(ld_agent(pa + static_cast<int64_t>(s) * D), w, asum);
+  for (int s0 = NB; s0 < n_valid; s0 += NB) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int sidx = min(s0 + i, n_valid - 1);
+      pm[i] = ld_agent(ml + 2 * sidx);
+      pl[i] = ld_agent(ml + 2 * sidx + 1);
+      pv[i] = ld_agent(pa + static_cast<int64_t>(sidx) * D);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      if (s0 + i >= n_valid) continue;
+      const float w = __builtin_amdgcn_exp2f(pm[i] - mx);
+      lsum = __builtin_fmaf(pl[i], w, lsum);
+      asum = __builtin_fmaf(pv[i], w, asum);
+    }
   }
   return lsum > 0.0f ? asum / lsum : 0.0f;
 }
@@ -667,7 +692,7 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0) {
-    unsigned int *ticket = &g_tickets[a.ticket_base + b * a.n_hg + hg];
+    unsigned int *ticket = ticket_of(a.ticket_base, b * a.n_hg + hg);
     const unsigned int t = atomicAdd(ticket, 1u);
     s_last = (t == static_cast<unsigned int>(n_valid - 1));
     if (s_last) atomicExch(ticket, 0u);  // ready for the next launch
@@ -730,7 +755,7 @@ __device__ __forceinline__ void finish_range(const DecodeArgs &a, int b, int hg,
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0) {
-    unsigned int *ticket = &g_tickets[a.ticket_base + b * a.n_hg + hg];
+    unsigned int *ticket = ticket_of(a.ticket_base, b * a.n_hg + hg);
     const unsigned int t = atomicAdd(ticket, 1u);
     *s_last = (t == static_cast<unsigned int>(n_valid - 1));
     if (*s_last) atomicExch(ticket, 0u);  // ready for the next launch

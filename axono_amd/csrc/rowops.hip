@@ -698,6 +698,12 @@ constexpr int kArgmaxMaxRows = 1024;  // per ticket lane
 __device__ float g_argmax_val[AXHIP_TICKET_LANES * kArgmaxMaxRows * kArgmaxParts];
 __device__ long long g_argmax_idx[AXHIP_TICKET_LANES * kArgmaxMaxRows * kArgmaxParts];
 __device__ unsigned int g_argmax_ticket[AXHIP_TICKET_LANES * kArgmaxMaxRows];
+// Atomics on one 128-byte line are served one after the other (about 10 ns each on MI355X; 64 workgroups x 16
+// rows on one line cost 10 us): neighbouring rows take counters 128 bytes apart, the words in between belong to
+// rows 32, 64, ... further on.
+__device__ __forceinline__ unsigned int *argmax_ticket_of(int lane_row0, int row) {
+  return &g_argmax_ticket[lane_row0 + (((row & 31) << 5) | (row >> 5))];
+}
 }  // namespace
 int reset_argmax_tickets() {
   void *p = nullptr;
@@ -790,9 +796,10 @@ __global__ __launch_bounds__(kBlock) void argmax_parts_kernel(const T *__restric
     __hip_atomic_store(&g_argmax_idx[trow * kArgmaxParts + part], static_cast<long long>(bi), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_s_waitcnt(0);  // both stores have completed before the ticket is taken
-    const unsigned int t = atomicAdd(&g_argmax_ticket[trow], 1u);
+    unsigned int *ticket = argmax_ticket_of(lane_row0, row);
+    const unsigned int t = atomicAdd(ticket, 1u);
     s_last = (t == kArgmaxParts - 1);
-    if (s_last) atomicExch(&g_argmax_ticket[trow], 0u);
+    if (s_last) atomicExch(ticket, 0u);
   }
   __syncthreads();
   if (!s_last || threadIdx.x >= 64) return;

@@ -154,6 +154,23 @@ def test_result_independent_of_split_count():
         np.testing.assert_allclose(o, want, rtol=0, atol=TOL32)
 
 
+def test_forced_ranges_with_more_than_2048_head_groups():
+    """Ticket counters are laid out so that neighbouring (sequence, head group) pairs sit on different cache lines
+    and pair 2048 takes the word next to pair 0: a batch with 2080 pairs, every sequence cut into two and three
+    merged ranges, twice in a row (the counters must be back at zero after a launch)."""
+    rng = np.random.default_rng(2080)
+    B, hq, hkv, d, L = 260, 16, 8, 64, 96
+    q = rng.standard_normal((B, hq, d)).astype(np.float16)
+    k = rng.standard_normal((B, hkv, L, d)).astype(np.float16)
+    v = rng.standard_normal((B, hkv, L, d)).astype(np.float16)
+    lens = rng.integers(1, L + 1, B).astype(np.int32)
+    want = port.gqa_decode_cache(q, k, v, lens)
+    for splits in (2, 3, 2):
+        with gu.gqa_tuned(0, splits):
+            got = gqa_decode(q, k, v, seq_lens=lens)
+        np.testing.assert_allclose(got.astype(np.float32), want, rtol=0, atol=TOL16)
+
+
 def test_invariants_full_size_headline():
     """B=32, L=8192 fp16 (1 GiB of cache): properties that need no oracle pass over the data.
     Identical keys give the mean of V; the first sequence is also checked against the oracle."""

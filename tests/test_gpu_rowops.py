@@ -311,6 +311,11 @@ def test_cast_add_embedding_argmax():
         t[3, :] = -np.inf         # nothing compares greater: index 0
         np.testing.assert_array_equal(gu.argmax(t), port.argmax(t))
         np.testing.assert_array_equal(gu.argmax(h16(t)), port.argmax(t))
+    # more rows than the 32 whose ticket counters take a cache line each (row 32 takes the word next to row 0's),
+    # twice in a row: the counters are back at zero after a launch
+    t = rng.standard_normal((70, 16392)).astype(np.float32)
+    for _ in range(2):
+        np.testing.assert_array_equal(gu.argmax(t), np.argmax(t, -1))
 
 
 def test_sdpa_prefill_and_small_heads():

@@ -361,9 +361,82 @@ def bench_linear(lib, steps=50, shapes=None, Ms=(1, 16, 32, 512), packed=False, 
                    "weight_copies": n_rot})
 
 
+def bench_layer_tail(lib, steps, layers=28, M=16, H=2048, K1=2048, I=6144, N=4096):
+    """The part of a decoder layer behind its attention plus the next q/k/v projection, over `layers` different
+    weight sets (nothing comes from the memory-side cache): six launches against the one persistent launch, each
+    as a captured graph of all layers replayed back to back; then where the time goes inside one launch in the
+    middle of such a chain (axhip_decode_layer_tail_trace)."""
+    import time
+    from axono_amd import libaxono as L
+    from axono_amd.core.hip_graph import HIPGraph
+    from axono_amd.core.tensor import Tensor
+    from axono_amd.core.types import DataType
+    rng = np.random.default_rng(0)
+
+    def dev(a):
+        return Tensor.from_numpy_ref(np.ascontiguousarray(a)).to("hip")
+
+    def lin(n, k):
+        return (0.02 * rng.standard_normal((n, k), dtype=np.float32)).astype(np.float16)
+
+    base = {"o": lin(H, K1), "gu": lin(2 * I, H), "d": lin(H, I), "q": lin(N, H)}
+    W = [{k: L.pack_linear_weight(dev(v), glu=(k == "gu")) for k, v in base.items()} for _ in range(layers)]
+    wn = dev(np.ones(H, np.float32))
+    attn = dev(rng.standard_normal((M, K1)).astype(np.float16))
+    h0 = dev(rng.standard_normal((M, H)).astype(np.float32))
+    ws = Tensor(DataType.INT8, [lib.axhip_decode_layer_tail_workspace_bytes(H, I)], "hip")
+    L.synchronize()
+
+    def tails():
+        h = h0
+        for w in W:
+            h, _ = L.decode_layer_tail(attn, h, w["o"], wn, w["gu"], w["d"], wn, w["q"], N, 1e-6, ws)
+
+    def singles():
+        h = h0
+        for w in W:
+            o = L.linear_packed(attn, w["o"], H)
+            h, xn = L.add_rms_norm(o, h, wn, 1e-6, DataType.FLOAT16)
+            act = L.linear_packed(xn, w["gu"], 2 * I, out_dtype=DataType.FLOAT16, glu=True)
+            d = L.linear_packed(act, w["d"], H)
+            h, xn = L.add_rms_norm(d, h, wn, 1e-6, DataType.FLOAT16)
+            L.linear_packed(xn, w["q"], N)
+
+    nbytes = 2 * (H * K1 + 2 * I * H + H * I + N * H)
+    for name, fn in (("layer_tail_six_launches", singles), ("layer_tail_one_launch", tails)):
+        g = HIPGraph()
+        g.capture(fn)
+        g.replay()
+        L.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.launch_async()
+        g.sync()
+        us = (time.perf_counter() - t0) * 1e6 / (steps * layers)
+        g.reset()
+        _emit({"op": name, "M": M, "H": H, "I": I, "N_next": N, "us": round(us, 2), "bytes": nbytes,
+               "GBps": round(nbytes / us / 1e3, 1), "pct_hbm_peak": round(nbytes / us / 1e3 / 80.0, 1), "weight_sets": layers})
+    # the timeline of one launch in the middle of a chain
+    stamps = DeviceBuffer(256 * 32 * 8)
+    for rep in range(3):
+        for i, w in enumerate(W):
+            lib.axhip_decode_layer_tail_trace(stamps.ptr if (rep == 2 and i == layers // 2) else None)
+            L.decode_layer_tail(attn, h0, w["o"], wn, w["gu"], w["d"], wn, w["q"], N, 1e-6, ws)
+    L.synchronize()
+    lib.axhip_decode_layer_tail_trace(None)
+    t = stamps.download(np.uint64, (256, 2, 16)).astype(np.float64) / 100.0
+    t -= t[:, 0, 0].min()
+    points = ["start", "phase 1 matrix instructions done", "before barrier 1", "after barrier 1", "phase 2 row sums done",
+              "phase 2 matrix instructions done", "before barrier 2", "after barrier 2", "phase 3 matrix instructions done",
+              "before barrier 3", "after barrier 3", "phase 4 matrix instructions done", "end"]
+    _emit({"op": "layer_tail_timeline", "unit": "us after the first workgroup started; median over the 256 workgroups (max)",
+           "wavefront_0": {p: [round(float(np.median(t[:, 0, i])), 2), round(float(t[:, 0, i].max()), 2)] for i, p in enumerate(points)},
+           "failed_barrier_waits": L.decode_layer_tail_failed_waits()})
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "gqa-paged", "copy", "rowops", "linear", "linear-packed", "prefill-attn"])
+    ap.add_argument("what", choices=["gqa", "gqa-sweep", "gqa-shapes", "gqa-single", "gqa-step", "gqa-paged", "copy", "rowops", "linear", "linear-packed", "prefill-attn", "layer-tail"])
     ap.add_argument("--zero-data", action="store_true",
                     help="prefill-attn, linear-packed: all-zero operands (how much of the time is the power the data costs)")
     ap.add_argument("--tile-order", default="", help="linear-packed: 'plain' or 'A:B' rectangles of 256 x 128 GEMM tiles per XCD")
@@ -423,6 +496,8 @@ def main(argv=None):
         for S in (4096, 16384):
             for causal in (True, False):
                 bench_sdpa(lib, S, max(5, min(args.steps, 20)), causal)
+    elif args.what == "layer-tail":
+        bench_layer_tail(lib, min(args.steps, 20))
     elif args.what == "copy":
         bench_copy(lib, args.mib, args.steps)
     elif args.what == "rowops":

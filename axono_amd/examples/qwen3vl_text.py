@@ -146,7 +146,7 @@ class Qwen3VLTextDecoder(nn.Module):
     prefill of a sequence then runs over one dense scratch block and is copied into the sequence's pages."""
 
     def __init__(self, cfg: TextConfig, weights: dict, batch: int, max_len: int, device: str = "hip", paged: bool = False,
-                 n_pages: int | None = None):
+                 n_pages: int | None = None, fused_tail: bool | None = None):
         super().__init__()
         self._cfg = cfg
         self._device = device
@@ -180,6 +180,17 @@ class Qwen3VLTextDecoder(nn.Module):
         self._attn_ws = Tensor(DataType.INT8, [max(wsb, 256)], device)
         self._graph = None
         self._graph_out = None
+        # decode step: everything of a layer behind its attention + the next layer's q/k/v projection as one
+        # persistent launch, where the library is built for the widths (None: wherever it is)
+        n_qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
+        can = L.decode_layer_tail_supported(batch, cfg.hidden_size, cfg.num_attention_heads * cfg.head_dim,
+                                            cfg.intermediate_size, n_qkv)
+        if fused_tail and not can:
+            raise ValueError("decode_layer_tail is not built for these widths")
+        self._fused_tail = can if fused_tail is None else bool(fused_tail)
+        if self._fused_tail:
+            nbytes = self._lib.axhip_decode_layer_tail_workspace_bytes(cfg.hidden_size, cfg.intermediate_size)
+            self._tail_ws = Tensor(DataType.INT8, [nbytes], device)
 
     # ---- pieces ----------------------------------------------------------------------------
     def _w(self, name):
@@ -232,12 +243,28 @@ class Qwen3VLTextDecoder(nn.Module):
                                      cfg.rms_norm_eps)  # [B,H] each
         nl = cfg.num_hidden_layers
         nqd = cfg.num_attention_heads * cfg.head_dim
+        n_qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
+        qkv = None
         for i in range(nl):
             p = f"layers.{i}."
             if trace is not None:
                 trace.append(h)
-            qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")
+            if qkv is None:
+                qkv = self._linear(xn, p + "self_attn.qkv_proj.weight")
             attn = self._attention_step(qkv, p, i, pos, max_len)
+            qkv = None
+            if self._fused_tail and i + 1 < nl:
+                # o_proj + residual, norm, gate/up + SiLU-mul, down + residual, the next layer's norm and q/k/v
+                # projection: one launch
+                n = f"layers.{i + 1}."
+                h, qkv = L.decode_layer_tail(attn.reshape([B, nqd]), h, self._packed[p + "self_attn.o_proj.weight"],
+                                             self._w(p + "post_attention_layernorm.weight"),
+                                             self._packed[p + "mlp.gate_up_proj.weight"],
+                                             self._packed[p + "mlp.down_proj.weight"],
+                                             self._w(n + "input_layernorm.weight"),
+                                             self._packed[n + "self_attn.qkv_proj.weight"], n_qkv, cfg.rms_norm_eps,
+                                             self._tail_ws)
+                continue
             attn_out = self._linear(attn.reshape([B, nqd]), p + "self_attn.o_proj.weight")
             h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                     DataType.FLOAT16)
@@ -407,5 +434,12 @@ class Qwen3VLTextDecoder(nn.Module):
         if use_graph:
             self._graph.sync()
         L.synchronize()
+        if self._fused_tail:
+            # the persistent launch needs all its workgroups resident at once; a barrier wait that ran out means
+            # something else held compute units, and the tokens of those steps are not to be trusted
+            failed = L.decode_layer_tail_failed_waits(reset=True)
+            if failed:
+                raise RuntimeError(f"generate(): {failed} barrier waits of the fused layer launch ran out; "
+                                   "run the model with fused_tail=False when other work shares the device")
         self._cache.note_advanced(max_new_tokens)   # the steps advanced the lengths on the device
         return self._log.numpy()[:max_new_tokens].copy()

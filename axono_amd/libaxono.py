@@ -591,6 +591,48 @@ def embedding_rms_norm(ids: Tensor, table: Tensor, weight: Tensor, eps: float):
     return h, xn
 
 
+def decode_layer_tail_supported(m: int, hidden: int, k1: int, inter: int, n_next: int) -> bool:
+    """Whether decode_layer_tail is built for these widths (the 2B text tower's, and a small set for tests)."""
+    return m <= 16 and n_next % 16 == 0 and n_next <= 4096 and (hidden, k1, inter) in ((2048, 2048, 6144), (512, 512, 1024))
+
+
+def decode_layer_tail(attn: Tensor, h_in: Tensor, w_o: Tensor, w_post: Tensor, w_gate_up: Tensor, w_down: Tensor,
+                      w_next: Tensor, w_next_linear: Tensor, n_next: int, eps: float, workspace: Tensor,
+                      h_out: Tensor | None = None):
+    """Everything of a decoder layer behind the attention plus the next layer's fused q/k/v projection, for at
+    most 16 rows, as one persistent launch: returns (h_out FLOAT32 [M,H], y FLOAT32 [M,n_next]).  The weights are
+    the packed copies (pack_linear_weight; gate+up with glu=True).  h_out, if given, must not be h_in."""
+    op = "decode_layer_tail"
+    _need_hip(op, attn, h_in, w_o, w_post, w_gate_up, w_down, w_next, w_next_linear, workspace)
+    if attn.dtype != DataType.FLOAT16 or h_in.dtype != DataType.FLOAT32 or w_post.dtype != DataType.FLOAT32 or \
+            w_next.dtype != DataType.FLOAT32:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    m, hidden = h_in.shape
+    k1 = attn.num_elements // m
+    inter = w_down.num_elements // hidden
+    lib = _lib_()
+    need = lib.axhip_decode_layer_tail_workspace_bytes(hidden, inter)
+    if workspace.num_bytes < need or w_post.num_elements != hidden or w_next.num_elements != hidden:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if h_out is None:
+        h_out = _new(DataType.FLOAT32, [m, hidden], h_in)
+    y = _new(DataType.FLOAT32, [m, n_next], h_in)
+    check(lib.axhip_decode_layer_tail(attn.data_ptr, h_in.data_ptr, w_o.data_ptr, w_post.data_ptr, w_gate_up.data_ptr,
+                                      w_down.data_ptr, w_next.data_ptr, w_next_linear.data_ptr, h_out.data_ptr, y.data_ptr,
+                                      workspace.data_ptr, workspace.num_bytes, m, hidden, k1, inter, n_next, float(eps),
+                                      current_stream()), op)
+    return h_out, y
+
+
+def decode_layer_tail_failed_waits(reset: bool = False) -> int:
+    """Barrier waits of decode_layer_tail that ran out since the last reset (0 in a healthy process)."""
+    n = C.c_uint(0)
+    check(_lib_().axhip_decode_layer_tail_status(0, C.byref(n)), "decode_layer_tail_status")
+    if reset and n.value:   # (resetting moves the counters: only when something went wrong, with the device idle)
+        check(_lib_().axhip_decode_layer_tail_status(1, None), "decode_layer_tail_status")
+    return int(n.value)
+
+
 def decode_advance(next_ids: Tensor, ids: Tensor | None = None, pos: Tensor | None = None, seq_lens: Tensor | None = None,
                    log: Tensor | None = None, counter: Tensor | None = None) -> None:
     """The closing of a greedy decode step in one launch: ids = next_ids, pos += 1 (INT64 [rows, B]),

@@ -524,6 +524,29 @@ AXHIP_API int axhip_embedding_rms_norm(const void *ids, int ids_dtype, const voi
                                        int w_dtype, float eps, void *h, void *xn, int64_t n_ids, int64_t vocab,
                                        int64_t dim, axhip_stream stream);
 
+/* Everything of a decoder layer behind the attention, plus the next layer's fused q/k/v projection, for at most
+ * 16 rows, in one persistent launch whose four phases are separated by barriers across the resident workgroups
+ * (one per CU; the weights of a phase are requested before the barrier in front of it):
+ *   h1 = attn . Wo^T + h_in;  act = silu(g) * u with [g | u] = rmsnorm(h1, w_post) . Wgu^T;
+ *   h_out = act . Wd^T + h1;  y = rmsnorm(h_out, w_next) . Wn^T.
+ * attn FLOAT16 [M, K1]; h_in, h_out FLOAT32 [M, H] (different buffers); w_post, w_next FLOAT32 [H]; w_o [H, K1],
+ * w_gate_up [2 I, H] (packed with glu = 1), w_down [H, I], w_next_linear [N_next, H]: packed by
+ * axhip_linear_f16_pack; y FLOAT32 [M, N_next]; workspace: axhip_decode_layer_tail_workspace_bytes(H, I) bytes,
+ * 128-byte aligned.  Built for K1 = H = 2048, I = 6144 (and K1 = H = 512, I = 1024 for tests), N_next <= 16 per
+ * workgroup: other widths return AXHIP_INVALID_ARGUMENT and the caller uses the single operators.  Must be the
+ * only work on the device while it runs (all its workgroups have to be resident); a barrier wait that runs out
+ * is counted, see axhip_decode_layer_tail_status, and the results of that launch are undefined.  Replaces
+ * the operator sequence of Qwen3VLTextDecoderLayer.forward behind the attention and the q/k/v projections that open
+ * the next layer (the reference runs them one launch each, examples/vlm/qwen3vl/model.py:408-436). */
+AXHIP_API size_t axhip_decode_layer_tail_workspace_bytes(int H, int I);
+AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const void *w_o, const float *w_post,
+                                      const void *w_gate_up, const void *w_down, const float *w_next,
+                                      const void *w_next_linear, float *h_out, float *y, void *workspace,
+                                      size_t workspace_bytes, int M, int H, int K1, int I, int N_next, float eps,
+                                      axhip_stream stream);
+/* Barrier waits of axhip_decode_layer_tail that ran out since the last reset (0 in a healthy process); reset != 0
+ * also puts the barrier counters back to zero (only while no such launch is in flight). */
+AXHIP_API int axhip_decode_layer_tail_status(int reset, unsigned *failed_waits);
 /* Last launch of a greedy decode step: ids[b] = next_ids[b]; pos[r, b] += 1 for r < pos_rows;
  * seq_lens[b] += 1; log[*counter, b] = next_ids[b] while *counter < log_rows; *counter += 1.  Any of
  * ids, pos (with pos_rows 0), seq_lens, log and counter may be NULL.  The reference does all of this

@@ -40,6 +40,16 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
  * the XCDs, -1 = the default (by XCD when the pairs go round the eight XCDs evenly or there are at least 32). */
 AXHIP_API void axhip_prefill_attention_tune(int pairs_by_xcd);
 
+/* Measurement: bit p of skip_phases set = phase p + 1 computes nothing, 32 = no barriers (results are then
+ * meaningless). */
+AXHIP_API void axhip_decode_layer_tail_tune(int skip_phases);
+/* Measurement: launches made while `stamps` is not null leave 32 readings of the 100 MHz device clock per
+ * workgroup there (device memory, workgroups x 32 x 8 bytes): slots 0-12 of wavefront 0 and 16-28 of wavefront 5 at
+ * the start, after the matrix instructions of phase 1, before and after barrier 1, after the row sums of phase 2,
+ * after its matrix instructions, before and after barrier 2, after the matrix instructions of phase 3, before and
+ * after barrier 3, after the matrix instructions of phase 4, at the end. */
+AXHIP_API void axhip_decode_layer_tail_trace(void *stamps);
+
 #ifdef __cplusplus
 }
 #endif

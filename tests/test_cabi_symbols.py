@@ -16,7 +16,9 @@ def declared_symbols(headers=("axhip.h", "axhip_experimental.h")):
 def test_measurement_hooks_are_not_part_of_the_boundary_header():
     boundary = declared_symbols(("axhip.h",))
     assert not [n for n in boundary if n.endswith("_tune")]
-    assert sorted(declared_symbols(("axhip_experimental.h",))) == ["axhip_gqa_decode_tune", "axhip_linear_f16_tune",
+    assert not [n for n in boundary if n.endswith("_trace")]
+    assert sorted(declared_symbols(("axhip_experimental.h",))) == ["axhip_decode_layer_tail_trace", "axhip_decode_layer_tail_tune",
+                                                                   "axhip_gqa_decode_tune", "axhip_linear_f16_tune",
                                                                    "axhip_prefill_attention_tune"]
 
 

@@ -1,0 +1,98 @@
+"""axhip_decode_layer_tail (o_proj + residual, norm, gate/up + SiLU-mul, down_proj + residual, norm and the next
+layer's q/k/v Linear in one persistent launch) against the CPU oracle's single operators with the same fp16
+storage points: the activation entering each Linear and `act` are fp16, everything else fp32.  Tolerances: the
+residual stream differs by fp32 summation order and, behind a norm, by activations that round to the neighbouring
+fp16 value (2e-3 + 1e-3 |value|, the fp16 bound of the other decode-path tests)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import gpu_util as gu
+from oracle import port
+
+pytestmark = pytest.mark.gpu
+
+
+def h16(a):
+    return np.asarray(a, np.float32).astype(np.float16)
+
+
+def _pack(w, glu=False):
+    l = gu.lib()
+    n, k = w.shape
+    dw = gu.dev(w)
+    p = gu.DeviceBuffer(l.axhip_linear_f16_packed_bytes(n, k))
+    gu._run("axhip_linear_f16_pack", dw.ptr, p.ptr, n, k, int(glu), None)
+    gu.synchronize()
+    return p
+
+
+def _oracle(attn, h_in, wo, w_post, wgu, wd, w_next, wn, eps):
+    f = lambda a: np.asarray(a, np.float32)
+    inter = wd.shape[1]
+    h_mid = port.linear(f(attn), f(wo)) + h_in
+    xn2 = f(h16(port.rms_norm(h_mid, w_post, eps)))
+    gu_ = port.linear(xn2, f(wgu))
+    act = h16(port.silu_mul(np.ascontiguousarray(gu_[:, :inter]), np.ascontiguousarray(gu_[:, inter:])))
+    h_out = port.linear(f(act), f(wd)) + h_mid
+    xn = f(h16(port.rms_norm(h_out, w_next, eps)))
+    return h_out, port.linear(xn, f(wn))
+
+
+@pytest.mark.parametrize("M,H,K1,I,N_next", [(16, 512, 512, 1024, 512), (5, 512, 512, 1024, 1024), (1, 512, 512, 1024, 16),
+                                             (16, 2048, 2048, 6144, 4096), (7, 2048, 2048, 6144, 4096)])
+def test_layer_tail_matches_operator_composition(M, H, K1, I, N_next):
+    rng = np.random.default_rng(100 + M + H)
+    eps = 1e-6
+    attn = h16(rng.standard_normal((M, K1)))
+    h_in = rng.standard_normal((M, H)).astype(np.float32) * 3
+    wo, wd, wn = (h16(0.02 * rng.standard_normal(s)) for s in ((H, K1), (H, I), (N_next, H)))
+    wgu = h16(0.02 * rng.standard_normal((2 * I, H)))
+    w_post = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    w_next = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    l = gu.lib()
+    d_wp, d_wn = gu.dev(w_post), gu.dev(w_next)
+    p_o, p_gu, p_d, p_n = _pack(wo), _pack(wgu, glu=True), _pack(wd), _pack(wn)
+    wsb = l.axhip_decode_layer_tail_workspace_bytes(H, I)
+    ws = gu.DeviceBuffer(wsb)
+    h_out, y = (gu.DeviceBuffer(n) for n in (M * H * 4, M * N_next * 4))
+    failed = C.c_uint(0)
+    assert l.axhip_decode_layer_tail_status(1, C.byref(failed)) == 0
+    for it in range(3):   # the barrier state must be clean again after every launch; new inputs every time, so that
+        # a block served from a cache line of the launch before would be a wrong value
+        attn_i = h16(attn * (1.0 + 0.5 * it))
+        h_i = (h_in * (1.0 - 0.3 * it)).astype(np.float32)
+        want = _oracle(attn_i, h_i, wo, w_post, wgu, wd, w_next, wn, eps)
+        d_attn, d_h = gu.dev(attn_i), gu.dev(h_i)
+        print(f"tail M={M} H={H} I={I} N_next={N_next} launch {it}", flush=True)
+        gu._run("axhip_decode_layer_tail", d_attn.ptr, d_h.ptr, p_o.ptr, d_wp.ptr, p_gu.ptr, p_d.ptr, d_wn.ptr,
+                p_n.ptr, h_out.ptr, y.ptr, ws.ptr, wsb, M, H, K1, I, N_next, eps, None)
+        gu.synchronize()
+        assert l.axhip_decode_layer_tail_status(0, C.byref(failed)) == 0 and failed.value == 0
+        got = (h_out.download(np.float32, (M, H)), y.download(np.float32, (M, N_next)))
+        for name, g_, w_ in (("h_out", got[0], want[0]), ("y", got[1], want[1])):
+            err = np.abs(g_ - w_)
+            print(f"  {name}: max abs err {float(err.max()):.3e} (max |value| {float(np.abs(w_).max()):.3f})", flush=True)
+            # 2e-3, plus one part in a thousand where a value is large enough for its fp16 spacing to matter
+            excess = float((err - (2e-3 + 1e-3 * np.abs(w_))).max())
+            assert excess <= 0.0, (name, excess)
+        # poison the outputs so that a launch that did nothing cannot pass
+        for b in (h_out, y):
+            b.upload(np.full(b.nbytes // 4, np.nan, np.float32))
+
+
+def test_layer_tail_argument_checks():
+    l = gu.lib()
+    b = gu.DeviceBuffer(1 << 22)
+    big = 1 << 22
+    args = [b.ptr] * 9 + [b.ptr + 4096, b.ptr, big]      # h_out differs from h_in
+    assert l.axhip_decode_layer_tail(*args, 17, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # more than 16 rows
+    assert l.axhip_decode_layer_tail(*args, 16, 1024, 2048, 6144, 4096, 1e-6, None) == 1   # widths it is not built for
+    assert l.axhip_decode_layer_tail(*args, 16, 2048, 2048, 6144, 4100, 1e-6, None) == 1   # N_next not whole tiles
+    assert l.axhip_decode_layer_tail(*args, 16, 2048, 2048, 6144, 8192, 1e-6, None) == 1   # more tiles than workgroups
+    assert l.axhip_decode_layer_tail(*([None] + args[1:]), 16, 2048, 2048, 6144, 4096, 1e-6, None) == 7
+    same = [b.ptr] * 11 + [big]
+    assert l.axhip_decode_layer_tail(*same, 16, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # h_out is h_in
+    assert l.axhip_decode_layer_tail(*args[:11], 1024, 16, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # workspace too small
+    assert l.axhip_decode_layer_tail(*args, 0, 2048, 2048, 6144, 4096, 1e-6, None) == 0

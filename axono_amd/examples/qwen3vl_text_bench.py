@@ -37,6 +37,8 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
     of that launch for all layers (each layer's own weights and caches, so nothing is served from the
     memory-side cache) and replayed `reps` times between host clock reads.  Rows: calls per step, us per call
     inside such a back-to-back graph, algorithmic bytes per call and the fraction of HBM peak that is.
+    With the fused layer launch the single launches it replaces still run once per step (the last layer; the first
+    layer's q/k/v projection): they are timed over all layers as before and counted once.
     The three launches that a step holds once are captured `once_copies` times over, so that the fixed cost of
     replaying a graph (some 20 us, which a one-node graph would charge to its only node) is spread as it is
     in the step; the weight of lm_head is 622 MB, more than the memory-side cache holds, so its copies still
@@ -70,30 +72,45 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
     def lin_bytes(K, N, out_b):
         return 2 * K * N + 2 * B * K + out_b * B * N
 
+    fused = model._fused_tail
+    per = (lambda n: 1 if fused else n)   # with the fused launch only one layer runs these as single launches
+    n_qkv = (nq + 2 * nkv) * D
     kinds = [
-        ("qkv Linear 2048->4096", nl, lin_bytes(H, (nq + 2 * nkv) * D, 4),
+        ("qkv Linear 2048->4096", nl, per(nl), lin_bytes(H, n_qkv, 4),
          layers(lambda p, i: model._linear(xn, p + "self_attn.qkv_proj.weight"))),
-        ("attention (qk-norm + M-RoPE + KV append + split-K decode + merge)", nl,
-         2 * nkv * D * 2 * B * (context + 1) + B * (nq + 2 * nkv) * D * 4 + B * nq * D * 2,
+        ("attention (qk-norm + M-RoPE + KV append + split-K decode + merge)", nl, nl,
+         2 * nkv * D * 2 * B * (context + 1) + B * n_qkv * 4 + B * nq * D * 2,
          layers(lambda p, i: model._attention_step(qkv, p, i, model._pos, model._decode_bound))),
-        ("o_proj Linear 2048->2048", nl, lin_bytes(nq * D, H, 4),
+        ("o_proj Linear 2048->2048", nl, per(nl), lin_bytes(nq * D, H, 4),
          layers(lambda p, i: model._linear(attn, p + "self_attn.o_proj.weight"))),
-        ("add + RMSNorm (fp32 residual, fp16 out)", 2 * nl, B * H * (4 + 4 + 4 + 2) + 4 * H,
+        ("add + RMSNorm (fp32 residual, fp16 out)", 2 * nl, 2 if fused else 2 * nl, B * H * (4 + 4 + 4 + 2) + 4 * H,
          lambda: [L.add_rms_norm(o32, h, W(f"layers.{i // 2}.post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                  DataType.FLOAT16) for i in range(2 * nl)]),
-        ("gate+up Linear 2048->12288 + SiLU-mul", nl, lin_bytes(H, 2 * I, 1),
+        ("gate+up Linear 2048->12288 + SiLU-mul", nl, per(nl), lin_bytes(H, 2 * I, 1),
          layers(lambda p, i: L.linear_packed(xn, model._packed[p + "mlp.gate_up_proj.weight"], 2 * I,
                                              out_dtype=DataType.FLOAT16, glu=True))),
-        ("down Linear 6144->2048", nl, lin_bytes(I, H, 4), layers(lambda p, i: model._linear(act, p + "mlp.down_proj.weight"))),
-        ("lm_head Linear 2048->151936", 1, lin_bytes(H, V, 4),
+        ("down Linear 6144->2048", nl, per(nl), lin_bytes(I, H, 4), layers(lambda p, i: model._linear(act, p + "mlp.down_proj.weight"))),
+        ("lm_head Linear 2048->151936", once_copies, 1, lin_bytes(H, V, 4),
          lambda: [model._linear(xn, "embed_tokens.weight") for _ in range(once_copies)]),
-        ("argmax over 151936", 1, B * V * 4, lambda: [L.argmax(logits) for _ in range(once_copies)]),
-        ("embedding + first RMSNorm", 1, B * H * (2 + 4 + 2),
+        ("argmax over 151936", once_copies, 1, B * V * 4, lambda: [L.argmax(logits) for _ in range(once_copies)]),
+        ("embedding + first RMSNorm", once_copies, 1, B * H * (2 + 4 + 2),
          lambda: [L.embedding_rms_norm(model._ids, W("embed_tokens.weight"), W("layers.0.input_layernorm.weight"),
                                        cfg.rms_norm_eps) for _ in range(once_copies)]),
     ]
+    if fused:
+        def tails():
+            hh = h
+            for i in range(nl - 1):
+                p, n = f"layers.{i}.", f"layers.{i + 1}."
+                hh, _ = L.decode_layer_tail(attn, hh, model._packed[p + "self_attn.o_proj.weight"],
+                                            W(p + "post_attention_layernorm.weight"), model._packed[p + "mlp.gate_up_proj.weight"],
+                                            model._packed[p + "mlp.down_proj.weight"], W(n + "input_layernorm.weight"),
+                                            model._packed[n + "self_attn.qkv_proj.weight"], n_qkv, cfg.rms_norm_eps, model._tail_ws)
+        kinds.insert(2, ("layer tail: o_proj + norm + gate/up + SiLU-mul + down + norm + next qkv, one persistent launch",
+                         nl - 1, nl - 1, 2 * (nq * D * H + 2 * I * H + H * I + n_qkv * H) + B * (nq * D * 2 + 2 * H * 4 + n_qkv * 4),
+                         tails))
     rows = []
-    for name, calls, nbytes, fn in kinds:
+    for name, graph_calls, calls, nbytes, fn in kinds:
         g = HIPGraph()
         g.capture(fn)
         g.replay()
@@ -103,7 +120,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
         for _ in range(reps):
             g.launch_async()
         g.sync()
-        us = (time.perf_counter() - t0) * 1e6 / (reps * (calls if calls > 1 else once_copies))
+        us = (time.perf_counter() - t0) * 1e6 / (reps * graph_calls)
         g.reset()
         rows.append({"kernel": name, "calls_per_step": calls, "us_per_call": round(us, 2),
                      "us_per_step": round(us * calls, 1), "bytes_per_call": int(nbytes),

@@ -105,6 +105,7 @@ PROTOTYPES = {
     "axhip_index_add": (c_i, [c_vp, c_i, c_i64, c_i64, c_vp]),
     "axhip_embedding_rms_norm": (c_i, [c_vp, c_i, c_vp, c_vp, c_i, c_f, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "axhip_decode_advance": (c_i, [c_vp, c_vp, c_vp, c_i, c_vp, c_vp, c_i64, c_vp, c_i, c_vp]),
+    "axhip_decode_layer_tail_supported": (c_i, [c_i, c_i, c_i, c_i, c_i]),
     "axhip_decode_layer_tail_workspace_bytes": (c_sz, [c_i, c_i]),
     "axhip_decode_layer_tail": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz,
                                       c_i, c_i, c_i, c_i, c_i, c_f, c_vp]),

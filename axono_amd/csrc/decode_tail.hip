@@ -513,6 +513,28 @@ int launch_tail(const TailArgs &a, int wgs, hipStream_t st) {
   return launch_status();
 }
 
+// The kernel instance for these widths on the current device: 0 = none (the caller uses the single operators),
+// 1 = <4,4,12,3> (K1 = H = 2048, I = 6144), 2 = <1,1,2,1> (K1 = H = 512, I = 1024).  Every phase must have at most
+// one unit per resident workgroup (one workgroup per compute unit, 256 at most).
+int tail_instance(int M, int H, int K1, int I, int N_next, int *wgs_out) {
+  if (M < 0 || M > kTailRows || H <= 0 || K1 <= 0 || I <= 0 || N_next <= 0) return 0;
+  if (H % 512 != 0 || K1 % 512 != 0 || I % 512 != 0 || N_next % 16 != 0 || H > kTailMaxH) return 0;
+  const int cus = device_cu_count();
+  const int wgs = cus < kTailMaxWgs ? cus : kTailMaxWgs;
+  if (wgs_out) *wgs_out = wgs;
+  const int ck1 = K1 / 512, ch = H / 512, ci = I / 512;
+  int nt2 = 0;
+  for (int t = 1; t <= 3; ++t)
+    if ((I / 8) % t == 0 && (I / 8) / t <= wgs) {
+      nt2 = t;
+      break;
+    }
+  if (nt2 == 0 || H / 8 > wgs || N_next / 16 > wgs) return 0;
+  if (ck1 == 4 && ch == 4 && ci == 12 && nt2 == 3) return 1;
+  if (ck1 == 1 && ch == 1 && ci == 2 && nt2 == 1) return 2;
+  return 0;
+}
+
 size_t tail_workspace_bytes(int H, int I) {
   return 2 * static_cast<size_t>(H / 8) * kHBlockBytes + static_cast<size_t>(I) * 32;
 }
@@ -534,8 +556,9 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
                                       const void *w_next_linear, float *h_out, float *y, void *workspace,
                                       size_t workspace_bytes, int M, int H, int K1, int I, int N_next, float eps,
                                       axhip_stream stream) {
-  if (M < 0 || M > kTailRows || H <= 0 || K1 <= 0 || I <= 0 || N_next <= 0) return AXHIP_INVALID_ARGUMENT;
-  if (H % 512 != 0 || K1 % 512 != 0 || I % 512 != 0 || N_next % 16 != 0 || H > kTailMaxH) return AXHIP_INVALID_ARGUMENT;
+  int wgs = 0;
+  const int instance = tail_instance(M, H, K1, I, N_next, &wgs);
+  if (instance == 0) return AXHIP_INVALID_ARGUMENT;  // widths this launch is not built for: use the single operators
   if (M == 0) return AXHIP_OK;
   if (!attn || !h_in || !w_o || !w_post || !w_gate_up || !w_down || !w_next || !w_next_linear || !h_out || !y ||
       !workspace)
@@ -549,17 +572,6 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
   if (all & 15) return AXHIP_INVALID_PTR;
   if (reinterpret_cast<uintptr_t>(workspace) & 127) return AXHIP_INVALID_PTR;
   if (workspace_bytes < tail_workspace_bytes(H, I)) return AXHIP_INVALID_ARGUMENT;
-  const int cus = device_cu_count();
-  const int wgs = cus < kTailMaxWgs ? cus : kTailMaxWgs;
-  const int ck1 = K1 / 512, ch = H / 512, ci = I / 512;
-  // every phase has at most one unit per resident workgroup
-  int nt2 = 0;
-  for (int t = 1; t <= 3; ++t)
-    if ((I / 8) % t == 0 && (I / 8) / t <= wgs) {
-      nt2 = t;
-      break;
-    }
-  if (nt2 == 0 || H / 8 > wgs || N_next / 16 > wgs) return AXHIP_INVALID_ARGUMENT;
   TailArgs a;
   a.attn = static_cast<const __half *>(attn);
   a.h_in = h_in;
@@ -583,9 +595,11 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
   a.skip = g_tail_skip;
   a.dbg = g_tail_dbg;
   hipStream_t st = as_stream(stream);
-  if (ck1 == 4 && ch == 4 && ci == 12 && nt2 == 3) return launch_tail<4, 4, 12, 3>(a, wgs, st);
-  if (ck1 == 1 && ch == 1 && ci == 2 && nt2 == 1) return launch_tail<1, 1, 2, 1>(a, wgs, st);  // 512 / 512 / 1024
-  return AXHIP_INVALID_ARGUMENT;  // widths this launch is not built for: use the single operators
+  return instance == 1 ? launch_tail<4, 4, 12, 3>(a, wgs, st) : launch_tail<1, 1, 2, 1>(a, wgs, st);
+}
+
+AXHIP_API int axhip_decode_layer_tail_supported(int M, int H, int K1, int I, int N_next) {
+  return tail_instance(M, H, K1, I, N_next, nullptr) != 0 ? 1 : 0;
 }
 
 // Barrier bookkeeping of axhip_decode_layer_tail: number of barrier waits that ran out since the last reset (0 in

@@ -592,8 +592,9 @@ def embedding_rms_norm(ids: Tensor, table: Tensor, weight: Tensor, eps: float):
 
 
 def decode_layer_tail_supported(m: int, hidden: int, k1: int, inter: int, n_next: int) -> bool:
-    """Whether decode_layer_tail is built for these widths (the 2B text tower's, and a small set for tests)."""
-    return m <= 16 and n_next % 16 == 0 and n_next <= 4096 and (hidden, k1, inter) in ((2048, 2048, 6144), (512, 512, 1024))
+    """Whether decode_layer_tail is built for these widths on the current device (the 2B text tower's on a device
+    with 256 compute units, and a small set for tests)."""
+    return hip_available() and bool(_lib_().axhip_decode_layer_tail_supported(m, hidden, k1, inter, n_next))
 
 
 def decode_layer_tail(attn: Tensor, h_in: Tensor, w_o: Tensor, w_post: Tensor, w_gate_up: Tensor, w_down: Tensor,

@@ -538,6 +538,9 @@ AXHIP_API int axhip_embedding_rms_norm(const void *ids, int ids_dtype, const voi
  * is counted, see axhip_decode_layer_tail_status, and the results of that launch are undefined.  Replaces
  * the operator sequence of Qwen3VLTextDecoderLayer.forward behind the attention and the q/k/v projections that open
  * the next layer (the reference runs them one launch each, examples/vlm/qwen3vl/model.py:408-436). */
+/* 1 when axhip_decode_layer_tail is built for these widths on the current device (it needs a workgroup per unit of
+ * every phase: 256 compute units for the 2B widths), else 0. */
+AXHIP_API int axhip_decode_layer_tail_supported(int M, int H, int K1, int I, int N_next);
 AXHIP_API size_t axhip_decode_layer_tail_workspace_bytes(int H, int I);
 AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const void *w_o, const float *w_post,
                                       const void *w_gate_up, const void *w_down, const float *w_next,

@@ -96,3 +96,9 @@ def test_layer_tail_argument_checks():
     assert l.axhip_decode_layer_tail(*same, 16, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # h_out is h_in
     assert l.axhip_decode_layer_tail(*args[:11], 1024, 16, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # workspace too small
     assert l.axhip_decode_layer_tail(*args, 0, 2048, 2048, 6144, 4096, 1e-6, None) == 0
+    # the question a caller asks before it chooses between this launch and the single operators
+    assert l.axhip_decode_layer_tail_supported(16, 2048, 2048, 6144, 4096) == 1
+    assert l.axhip_decode_layer_tail_supported(16, 512, 512, 1024, 48) == 1
+    assert l.axhip_decode_layer_tail_supported(17, 2048, 2048, 6144, 4096) == 0
+    assert l.axhip_decode_layer_tail_supported(16, 1024, 1024, 3072, 2048) == 0
+    assert l.axhip_decode_layer_tail_supported(16, 2048, 2048, 6144, 8192) == 0

@@ -16,15 +16,17 @@
 // every phase has at most one unit of work per workgroup, and a unit's weight fragments fit the registers of
 // its 16 wavefronts (<= 48 VGPRs each).
 //
-// One workgroup per CU (1024 threads = 16 wavefronts, 128 registers each).  The wavefronts of a workgroup split K and add their
-// fragments through LDS, as in the skinny Linear kernels; wavefront 0 finishes a unit (sum, epilogue, store),
-// arrives at the barrier and waits there, the other 15 request their next weights meanwhile (wavefront 0 right
-// after its first look at the flag: a look that follows those loads also waits for them, the memory counter
-// being in order).
+// One workgroup per CU (1024 threads = 16 wavefronts, 128 registers each).  The wavefronts of a workgroup split K
+// and add their fragments through LDS, as in the skinny Linear kernels; wavefront 0 finishes a unit (epilogue,
+// store), arrives at the barrier and waits there, the other 15 request their next weights meanwhile (wavefront 0
+// right after its first look at the flag: a look that follows those loads also waits for them, the memory
+// counter being in order).  Barriers inside the workgroup wait for LDS traffic only (lds_barrier): __syncthreads()
+// would wait for the weights in flight.
 //
 // Data that crosses a barrier is written with agent-scope (write-through) stores into blocks that a single
 // workgroup owns as whole 128-byte lines (the residual stream as [unit][16 rows][8 columns] + the rows' partial
-// sums of squares, the activations as [unit][16 rows][8 NT columns]), and read with ordinary loads: a line that
+// sums of squares; the activations in matrix-instruction fragment order, 256 bytes per 8 columns: both are what a
+// lane of the consuming phase loads as contiguous bytes), and read with ordinary loads: a line that
 // no workgroup of an XCD has touched in this launch is not in that XCD's L2, so the load fetches what the
 // barrier made visible; no cache invalidate is needed.  Each such buffer is written in exactly one phase and
 // first read after the barrier behind it.  Results for the next launch (h_out, y) are also stored row-major.
@@ -132,7 +134,9 @@ struct TailArgs {
 
 extern __shared__ __attribute__((aligned(16))) unsigned char tail_smem[];
 constexpr int kStripBytes = kTailRows * 4 * 32 * 2;                     // per wavefront: 16 rows x 128 halves
-constexpr int kRedOffset = kTailWaves * kStripBytes;                    // 64 KiB (phase 1 strips; later the sums of squares)
+// LDS: [0, 64 KiB) the x strips of phase 1, later the transposed partial sums of squares; then the parked fragments
+// of the K slices, their partial sums, the rows' rstd, both norm weights.
+constexpr int kRedOffset = kTailWaves * kStripBytes;
 constexpr int kRedBytes = kTailWaves * 3 * 64 * 16;                     // up to three tiles per unit
 constexpr int kRed2Offset = kRedOffset + kRedBytes;                     // partial sums of four wavefronts each
 constexpr int kRstdOffset = kRed2Offset + 3 * 4 * 64 * 16;
@@ -144,7 +148,6 @@ constexpr int kSsqStride = 260;                                         // float
 __device__ __forceinline__ half8_t ld_w(const __half *p) {
   return __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(p));
 }
-#define LDW(p) ld_w(p)
 
 // x fragments of SC chunks from this wavefront's strip (rows of SC*32 halves, 16-byte units XOR-ed with the row)
 template <int SC>
@@ -153,24 +156,6 @@ __device__ __forceinline__ void read_frags(const _Float16 *strip, int r, int g, 
   for (int j = 0; j < SC; ++j) {
     const int un = j * 4 + g;
     bf[j] = *reinterpret_cast<const half8_t *>(strip + r * (SC * 32) + ((un ^ (r & (SC * 4 - 1))) << 3));
-  }
-}
-
-// fp16 rows in global memory -> strip.  `addr(row, col)` gives the address of 8 halves of row `row` from column `col`.
-template <int SC, typename F>
-__device__ __forceinline__ void stage_f16(F addr, int col0, _Float16 *strip, int lane) {
-  half8_t xv[SC];
-#pragma unroll
-  for (int p = 0; p < SC; ++p) {
-    const int v = p * 64 + lane;
-    const int row = v / (SC * 4), un = v % (SC * 4);
-    xv[p] = *reinterpret_cast<const half8_t *>(addr(row, col0 + un * 8));
-  }
-#pragma unroll
-  for (int p = 0; p < SC; ++p) {
-    const int v = p * 64 + lane;
-    const int row = v / (SC * 4), un = v % (SC * 4);
-    *reinterpret_cast<half8_t *>(strip + row * (SC * 32) + ((un ^ (row & (SC * 4 - 1))) << 3)) = xv[p];
   }
 }
 
@@ -202,7 +187,7 @@ __device__ __forceinline__ void row_rstd(const unsigned char *blocks, int n_unit
   }
   lds_barrier();
 }
-static_assert(kTailWaves == kTailRows && kTailWaves == 16, "one wavefront per row in row_rstd; four times four fragments in total()");
+static_assert(kTailWaves == kTailRows && kTailWaves == 16, "one wavefront per row in row_rstd, four times four fragments in total()");
 
 // x fragments of a norm phase, straight from the residual blocks (a block holds a unit's 8 columns of all 16 rows:
 // lane (r, g) of chunk c reads 32 contiguous bytes of block 4c + g): request, then normalise.
@@ -253,18 +238,14 @@ __device__ __forceinline__ void total(float4_t (&acc)[NT], int wave, int lane) {
   }
 }
 
-// Residual epilogue of phases 1 and 3 (wavefront 0): the unit's 8 columns of 16 rows + residual -> block (+ the
-// rows' partial sums of squares), optionally row-major as well.
-template <typename R>
-__device__ __forceinline__ void store_residual_unit(const float4_t &tot, R residual4, unsigned char *blocks, int unit,
+// Residual epilogue of phases 1 and 3 (wavefront 0): the unit's 8 columns of 16 rows + residual (`rv`: this
+// lane's four values, requested earlier) -> block (+ the rows' partial sums of squares), optionally row-major too.
+__device__ __forceinline__ void store_residual_unit(const float4_t &tot, const float4_t &rv, unsigned char *blocks, int unit,
                                                     int half, float *row_major, int H, int M, int lane) {
   const int r = lane & 15, g = lane >> 4;
   const bool mine = (g >> 1) == half;  // output rows 4g .. 4g+3 of the tile belong to this half
   float4_t hn = {0.f, 0.f, 0.f, 0.f};
-  if (mine && r < M) {
-    const float4_t rv = residual4(r, (g & 1) * 4);
-    hn = tot + rv;
-  }
+  if (mine && r < M) hn = tot + rv;
   float s = 0.f;
 #pragma unroll
   for (int q = 0; q < 4; ++q) s = __builtin_fmaf(hn[q], hn[q], s);
@@ -318,7 +299,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
   {
     const __half *p = a.w_o + (static_cast<int64_t>(on1 ? wg >> 1 : 0) * (a.K1 / 32) + wave * CK1) * 512 + src_lane * 8;
 #pragma unroll
-    for (int j = 0; j < CK1; ++j) wA[j] = LDW(p + j * 512);
+    for (int j = 0; j < CK1; ++j) wA[j] = ld_w(p + j * 512);
     if (!(a.skip & 1)) {
 #pragma unroll
       for (int q = 0; q < CK1; ++q) {
@@ -332,7 +313,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     for (int t = 0; t < NT2; ++t) {
       const __half *q = a.w_gu + (static_cast<int64_t>(on2 ? wg * NT2 + t : 0) * (a.H / 32) + wave * CH) * 512 + lane * 8;
 #pragma unroll
-      for (int j = 0; j < CH; ++j) wB[t][j] = LDW(q + j * 512);
+      for (int j = 0; j < CH; ++j) wB[t][j] = ld_w(q + j * 512);
     }
   }
 
@@ -356,10 +337,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     STAMP(1);
     total<1>(acc, wave, lane);
     if (wave == 0) {
-      if (on1) {
-        auto res = [&](int, int) { return res1; };
-        store_residual_unit(acc[0], res, a.hmid, wg, half1, nullptr, a.H, M, lane);
-      }
+      if (on1) store_residual_unit(acc[0], res1, a.hmid, wg, half1, nullptr, a.H, M, lane);
     }
   }
   STAMP(2);
@@ -392,7 +370,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     if (wave != 0) {
       // the weights of phase 3 travel while the unit is finished and the barrier is crossed
 #pragma unroll
-      for (int j = 0; j < CI; ++j) wC[j] = LDW(pc + j * 512);
+      for (int j = 0; j < CI; ++j) wC[j] = ld_w(pc + j * 512);
     }
     total<NT2>(acc, wave, lane);
     if (wave == 0) {
@@ -422,7 +400,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
   {
     auto pf = [&] {
 #pragma unroll
-      for (int j = 0; j < CI; ++j) wC[j] = LDW(pc + j * 512);
+      for (int j = 0; j < CI; ++j) wC[j] = ld_w(pc + j * 512);
     };
     STAMP(6);
     if (bars) {
@@ -450,20 +428,17 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     STAMP(8);
     if (wave != 0) {
 #pragma unroll
-      for (int j = 0; j < CH; ++j) wD[j] = LDW(pd + j * 512);
+      for (int j = 0; j < CH; ++j) wD[j] = ld_w(pd + j * 512);
     }
     total<1>(acc, wave, lane);
     if (wave == 0) {
-      if (on1) {
-        auto res = [&](int, int) { return res3; };
-        store_residual_unit(acc[0], res, a.hout, wg, half1, a.h_out, a.H, a.M, lane);
-      }
+      if (on1) store_residual_unit(acc[0], res3, a.hout, wg, half1, a.h_out, a.H, a.M, lane);
     }
   }
   {
     auto pf = [&] {
 #pragma unroll
-      for (int j = 0; j < CH; ++j) wD[j] = LDW(pd + j * 512);
+      for (int j = 0; j < CH; ++j) wD[j] = ld_w(pd + j * 512);
     };
     STAMP(9);
     if (bars) {

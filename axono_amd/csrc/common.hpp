@@ -67,6 +67,11 @@ int reset_argmax_tickets();
 
 inline bool is_float_dtype(int dt) { return dt == AXHIP_FLOAT16 || dt == AXHIP_FLOAT32; }
 
+// Workgroup barrier that waits for this wavefront's LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load (s_waitcnt vmcnt(0)), i.e. it drains whatever a kernel has requested ahead across the
+// barrier.  Use where the barrier orders LDS writes and reads and nothing else.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---- 16-byte vector access ---------------------------------------------------------------------
 struct alignas(16) Vec16 {
   uint32_t w[4];

@@ -66,10 +66,6 @@ __device__ TailBarrier g_tail_bar;
 #define TAIL_ST(p, v) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define TAIL_ADD(p, v) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
-// Workgroup barrier that waits for this wavefront's LDS traffic only.  __syncthreads() also waits for every
-// outstanding global load, i.e. for the weights that are meant to stay in flight across it.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 // k-th barrier of this launch (k = 1, 2, 3), called by every thread; `base` = the group's flag when the launch
 // began.  Only wavefront 0 has stores in flight.  Wavefront 0 arrives, looks at the flag once and only then
 // requests its share of the next phase's weights (`prefetch`): the memory counter is in order, so a look at the

@@ -48,7 +48,7 @@ constexpr int kTailRows = 16;
 constexpr int kBarGroup = 16;
 constexpr int kBarMaxGroups = 16;
 constexpr int kTailMaxWgs = kBarGroup * kBarMaxGroups;  // 256
-constexpr int kSpinLimit = 1 << 20;
+constexpr int kSpinLimit = 1 << 17;  // looks at the flag before a wait gives up: about a tenth of a second (a barrier takes microseconds)
 constexpr int kHBlockBytes = 640;  // [16][8] fp32 + 16 partial sums of squares + padding: five whole lines
 
 // Counters and flags only ever grow (a launch adds 3 to every flag), so nothing has to be put back between
@@ -72,8 +72,11 @@ __device__ TailBarrier g_tail_bar;
 // flag that follows those loads also waits for them - which costs nothing, the wavefront needs them anyway.
 // Returns false when the wait ran out.
 template <typename F>
-__device__ __forceinline__ bool grid_sync(unsigned k, unsigned base, int *s_ok, F prefetch) {
-  if (threadIdx.x < 64) {
+__device__ __forceinline__ bool grid_sync(unsigned k, unsigned base, int *s_ok, F prefetch, int spin_limit,
+                                          unsigned failed_before = 0) {
+  if (threadIdx.x < 64 && failed_before != 0) {
+    if (threadIdx.x == 0) *s_ok = 0;
+  } else if (threadIdx.x < 64) {
     __builtin_amdgcn_s_waitcnt(0);  // the write-through stores of this wavefront have reached memory
     const unsigned n_wg = gridDim.x, wg = blockIdx.x;
     const unsigned grp = wg / kBarGroup, n_grp = (n_wg + kBarGroup - 1) / kBarGroup;
@@ -90,7 +93,7 @@ __device__ __forceinline__ bool grid_sync(unsigned k, unsigned base, int *s_ok, 
     __builtin_amdgcn_sched_barrier(0);
     prefetch();
     __builtin_amdgcn_sched_barrier(0);
-    int ok = 1, limit = kSpinLimit;
+    int ok = 1, limit = spin_limit;
     while (static_cast<int>(f - want) < 0) {
       if (--limit <= 0) {
         ok = 0;
@@ -125,7 +128,7 @@ struct TailArgs {
   int M, H, K1, I, N_next;
   float eps;
   unsigned long long *dbg;  // measurement: 32 timestamps per workgroup (axhip_decode_layer_tail_trace), or null
-  int skip;  // measurement: bits 0-3 = phase 1-4 computes nothing, 32 = no barriers
+  int skip;  // measurement: bits 0-3 = phase 1-4 computes nothing, 32 = no barriers, 256 = a barrier gives up after one look
 };
 
 extern __shared__ __attribute__((aligned(16))) unsigned char tail_smem[];
@@ -274,12 +277,18 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
   const int half1 = wg & 1;
   const int src_lane = (lane & ~8) | (half1 << 3);  // both halves of the fragment hold this half's 8 rows
   const bool bars = !(a.skip & 32);
+  const int spin_limit = (a.skip & 256) ? 1 : kSpinLimit;  // (256: a test of the path a wait that runs out takes)
   static_assert(CK1 <= 4 && CH <= 4, "one staging step per phase");
 
   STAMP(0);
   // where this group's barrier flag stands (wavefront 0 needs it at the first barrier)
-  unsigned base = 0;
-  if (wave == 0) base = TAIL_LD(&g_tail_bar.flag[(wg / kBarGroup) * 32]);
+  unsigned base = 0, failed_before = 0;
+  if (wave == 0) {
+    base = TAIL_LD(&g_tail_bar.flag[(wg / kBarGroup) * 32]);
+    // a wait that ran out in an earlier launch has left the counters in disorder: until the caller has reset them
+    // (axhip_decode_layer_tail_status) a launch gives up at its first barrier at once instead of spinning again
+    failed_before = TAIL_LD(&g_tail_bar.fail[0]);
+  }
   // both norm weights go to LDS (read there by every wavefront in phases 2 and 4), the residual of phase 1 to
   // wavefront 0: requested first, so that they are back before anything that follows
   float *s_wn = reinterpret_cast<float *>(tail_smem + kNormWOffset);
@@ -337,7 +346,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     }
   }
   STAMP(2);
-  if (bars && !grid_sync(1, base, &s_ok, [] {})) return;
+  if (bars && !grid_sync(1, base, &s_ok, [] {}, spin_limit, failed_before)) return;
   STAMP(3);
 
   // ---- phase 2: post-attention norm, gate + up, SiLU-mul -------------------------------------------------------------
@@ -400,7 +409,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     };
     STAMP(6);
     if (bars) {
-      if (!grid_sync(2, base, &s_ok, pf)) return;
+      if (!grid_sync(2, base, &s_ok, pf, spin_limit)) return;
     } else if (wave == 0) {
       pf();
     }
@@ -438,7 +447,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
     };
     STAMP(9);
     if (bars) {
-      if (!grid_sync(3, base, &s_ok, pf)) return;
+      if (!grid_sync(3, base, &s_ok, pf, spin_limit)) return;
     } else if (wave == 0) {
       pf();
     }

@@ -41,7 +41,8 @@ AXHIP_API void axhip_linear_f16_tune(int target_waves, int force_nt, int force_w
 AXHIP_API void axhip_prefill_attention_tune(int pairs_by_xcd);
 
 /* Measurement: bit p of skip_phases set = phase p + 1 computes nothing, 32 = no barriers (results are then
- * meaningless). */
+ * meaningless); 256 = every barrier gives up after one look at its flag, which is how the tests reach the path of
+ * a wait that runs out (the launch still ends by itself). */
 AXHIP_API void axhip_decode_layer_tail_tune(int skip_phases);
 /* Measurement: launches made while `stamps` is not null leave 32 readings of the 100 MHz device clock per
  * workgroup there (device memory, workgroups x 32 x 8 bytes): slots 0-12 of wavefront 0 and 16-28 of wavefront 5 at

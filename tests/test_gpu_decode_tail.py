@@ -102,3 +102,47 @@ def test_layer_tail_argument_checks():
     assert l.axhip_decode_layer_tail_supported(17, 2048, 2048, 6144, 4096) == 0
     assert l.axhip_decode_layer_tail_supported(16, 1024, 1024, 3072, 2048) == 0
     assert l.axhip_decode_layer_tail_supported(16, 2048, 2048, 6144, 8192) == 0
+
+
+def test_a_wait_that_runs_out_is_counted_and_later_launches_give_up_at_once_until_the_reset():
+    """The barrier's wait is bounded.  Forced from the host (a spin limit of one look): the launch ends by itself,
+    the failure is counted, the next launch - with the normal limit - gives up at its first barrier instead of
+    spinning on counters in disorder, and after the reset a launch is correct again."""
+    rng = np.random.default_rng(7)
+    M, H, K1, I, N_next, eps = 16, 512, 512, 1024, 256, 1e-6
+    attn = h16(rng.standard_normal((M, K1)))
+    h_in = rng.standard_normal((M, H)).astype(np.float32)
+    wo, wd, wn = (h16(0.02 * rng.standard_normal(s)) for s in ((H, K1), (H, I), (N_next, H)))
+    wgu = h16(0.02 * rng.standard_normal((2 * I, H)))
+    ones = np.ones(H, np.float32)
+    want = _oracle(attn, h_in, wo, ones, wgu, wd, ones, wn, eps)
+    l = gu.lib()
+    d_attn, d_h, d_w = gu.dev(attn), gu.dev(h_in), gu.dev(ones)
+    p_o, p_gu, p_d, p_n = _pack(wo), _pack(wgu, glu=True), _pack(wd), _pack(wn)
+    wsb = l.axhip_decode_layer_tail_workspace_bytes(H, I)
+    ws = gu.DeviceBuffer(wsb)
+    h_out, y = (gu.DeviceBuffer(n) for n in (M * H * 4, M * N_next * 4))
+    failed = C.c_uint(0)
+    assert l.axhip_decode_layer_tail_status(1, C.byref(failed)) == 0
+
+    def launch():
+        gu._run("axhip_decode_layer_tail", d_attn.ptr, d_h.ptr, p_o.ptr, d_w.ptr, p_gu.ptr, p_d.ptr, d_w.ptr, p_n.ptr,
+                h_out.ptr, y.ptr, ws.ptr, wsb, M, H, K1, I, N_next, eps, None)
+        gu.synchronize()
+        assert l.axhip_decode_layer_tail_status(0, C.byref(failed)) == 0
+        return failed.value
+
+    try:
+        l.axhip_decode_layer_tail_tune(256)
+        print("tail: launch with a spin limit of one look", flush=True)
+        first = launch()
+        assert first > 0
+        l.axhip_decode_layer_tail_tune(0)
+        print("tail: launch on the state that launch left behind", flush=True)
+        assert launch() == first            # gave up at once: no new wait ran out, nothing was waited for
+    finally:
+        l.axhip_decode_layer_tail_tune(0)
+        assert l.axhip_decode_layer_tail_status(1, C.byref(failed)) == 0
+    print("tail: launch after the reset", flush=True)
+    assert launch() == 0
+    np.testing.assert_allclose(y.download(np.float32, (M, N_next)), want[1], rtol=0, atol=2e-3)

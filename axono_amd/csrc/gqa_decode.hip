@@ -1044,7 +1044,8 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
 //       touches, and every slot streams the same number of keys.  A sequence without keys gets its
 //       zeros from the slot that holds its place on the line.
 template <typename T, int D, int G, int U, bool QKV, bool MFMA = false, bool PAGED = false>
-__global__ __launch_bounds__(kThreads, MFMA ? 1 : 4) void gqa_decode_split_kernel(DecodeArgs a) {
+// (the decode-step form needs 161 registers: at four workgroups per CU, 128 registers, it spills 37 of them)
+__global__ __launch_bounds__(kThreads, MFMA ? 1 : (QKV ? 3 : 4)) void gqa_decode_split_kernel(DecodeArgs a) {
   // the piece to work on: keys [s0, s1) of sequence b, range `split` of its n_valid ranges
   int b, hg, split, n_valid, s0, s1;
   bool direct_ok = true;

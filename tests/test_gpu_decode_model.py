@@ -21,6 +21,12 @@ CFG4 = TextConfig(num_hidden_layers=2, hidden_size=256, num_attention_heads=8, n
                   intermediate_size=512, vocab_size=1000)
 
 
+# the small widths the fused layer launch is built for (hidden 512 = 4 heads of 128, intermediate 1024, 4 + 2 * 2 heads
+# of q / k / v): every layer but the last runs behind its attention as one persistent launch
+CFG_FUSED = TextConfig(num_hidden_layers=4, hidden_size=512, num_attention_heads=4, num_key_value_heads=2, head_dim=128,
+                       intermediate_size=1024, vocab_size=1000)
+
+
 def _setup(B=3, S=21, max_len=64, seed=0, CFG=CFG):
     w = random_weights(CFG, seed)
     # non-trivial norm weights so a dropped weight would show
@@ -95,6 +101,62 @@ def test_decode_steps_match_oracle(use_graph):
     # cache rows written by the decode steps
     for i in range(CFG.num_hidden_layers):
         assert_cache_rows(gpu.cache.get(i)[0].numpy()[:, :, S:S + n_steps], cpu.k[i][:, :, S:S + n_steps], i, 5e-4)
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_decode_steps_with_the_fused_layer_launch_match_oracle(use_graph):
+    """The same comparison at widths the fused layer launch is built for: three such launches per step hand the
+    residual stream and the next q/k/v projection to each other, the fourth layer runs as single operators; three
+    sequences (rows 3 to 15 of the launch's 16 are unused), eager and captured; and the tokens equal those of the
+    same model run as single operators."""
+    from axono_amd import libaxono as L
+    gpu, cpu, ids = _setup(seed=11, CFG=CFG_FUSED)
+    assert gpu._fused_tail
+    B, S = ids.shape
+    _, g_next = gpu.prefill(ids)
+    cpu.prefill(ids)
+    first = g_next.to_numpy()
+    pos = np.full((3, B), S, np.int64)
+    n_steps = 6
+    gpu.start_decode(first, pos, n_steps)
+    if use_graph:
+        g = gpu.capture()
+        assert g.num_nodes == 2 * 3 + 7 + 4
+    toks = gpu.generate(n_steps, use_graph=use_graph)
+    assert L.decode_layer_tail_failed_waits() == 0
+    cur = first
+    for s in range(n_steps):
+        logits, _ = cpu.decode_step(cur, pos + s)
+        chosen = logits[np.arange(B), toks[s]]
+        assert np.all(chosen >= logits.max(-1) - 4e-3), (s, chosen, logits.max(-1))
+        cur = toks[s]
+    np.testing.assert_array_equal(gpu.cache.seq_lens.to_numpy(), [S + n_steps] * B)
+    for i in range(CFG_FUSED.num_hidden_layers):
+        assert_cache_rows(gpu.cache.get(i)[0].numpy()[:, :, S:S + n_steps], cpu.k[i][:, :, S:S + n_steps], i, 5e-4)
+
+    # the same model as single operators
+    w = random_weights(CFG_FUSED, 11)
+    rng = np.random.default_rng(12)
+    for k in w:
+        if k.endswith("norm.weight") or k.endswith("layernorm.weight"):
+            w[k] = (1 + 0.1 * rng.standard_normal(w[k].shape)).astype(np.float32)
+    plain = Qwen3VLTextDecoder(CFG_FUSED, w, B, 64, "hip:0", fused_tail=False)
+    _, p_next = plain.prefill(ids)
+    np.testing.assert_array_equal(p_next.to_numpy(), first)
+    plain.start_decode(first, pos, n_steps)
+    if use_graph:
+        plain.capture()
+    toks_plain = plain.generate(n_steps, use_graph=use_graph)
+    cur = first
+    for s in range(n_steps):   # (a near-tie may be broken differently: both must be maximisers for the oracle)
+        if not np.array_equal(toks_plain[s], toks[s]):
+            logits, _ = cpu.decode_step(cur, pos + s)
+            break
+        cur = toks[s]
+    else:
+        return
+    chosen = logits[np.arange(B), toks_plain[s]]
+    assert np.all(chosen >= logits.max(-1) - 4e-3)
 
 
 def test_compiled_decode_loop_matches_the_captured_step():

@@ -48,6 +48,8 @@ PROTOTYPES = {
     "axhip_graph_replay": (c_i, [c_vp]),
     "axhip_set_ticket_lane": (c_i, [c_i]),
     "axhip_ticket_lane": (c_i, []),
+    "axhip_set_plan_reuse": (c_i, [c_i]),
+    "axhip_plan_reuse": (c_i, []),
     "axhip_reset_tickets": (c_i, []),
     "axhip_graph_sync": (c_i, [c_vp]),
     "axhip_graph_destroy": (c_i, [c_vp]),

@@ -49,6 +49,10 @@ Tuning g_tuning;
 // side by side) come from different ticket lanes: a lane is a region of its own in this array.
 constexpr int kTicketSlots = 1 << 16;  // per ticket lane
 __device__ unsigned int g_tickets[AXHIP_TICKET_LANES * kTicketSlots];
+// What the slots of a length-dealt launch found, kept for the later launches of the same step
+// (axhip_set_plan_reuse): 8 ints per slot, per ticket lane.
+constexpr int kPlanSlots = 4096;
+__device__ int g_plan_cache[AXHIP_TICKET_LANES * kPlanSlots * 8];
 
 // Atomics on one 128-byte line are served one after the other (about 10 ns each on MI355X), and the workgroups
 // of a launch finish together: neighbouring (sequence, head group) pairs therefore take counters 128 bytes
@@ -255,6 +259,11 @@ struct DecodeArgs {
   const int32_t *page_table;
   int max_pages, n_pages;
   int64_t page_stride;  // elements per page: Hkv * kPageKeys * D
+  // Decode-step form with lengths dealt in the kernel: the 28 attention launches of a step deal the same lengths
+  // the same way.  plan_mode 1: a launch leaves what every slot found (8 ints per slot) in plan_cache; 2: a launch
+  // reads that instead of the lengths and the dealing.  plan_check marks the entries of a launch of this shape.
+  int *plan_cache;
+  int plan_mode, plan_check;
 };
 
 // Split partials travel between workgroups that may sit on different XCDs, whose L2 caches are not
@@ -274,6 +283,7 @@ __device__ __forceinline__ void st_agent(float *p, float v) {
 // finish together whatever its current length is; a range cut from the host-side upper bound would
 // leave the last split short (4100 keys in 4 splits: 1040/1040/1040/980 instead of 1152/1152/1152/644).
 constexpr int kMinDevChunk = 128;
+constexpr int kNoLength = INT32_MIN;  // "read the length yourself"
 __device__ __forceinline__ int balanced_chunk(int len, int n_splits) {
   int c = (len + n_splits - 1) / n_splits;
   c = (c + 15) & ~15;
@@ -501,7 +511,7 @@ __device__ __forceinline__ float merge_ranges(const float *ml, const float *pa, 
 // the caller puts a barrier between two calls, because the LDS arrays are the same.
 template <typename T, int D, int G, int U, bool QKV, bool HOIST, bool PAGED = false>
 __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg, int split, int n_valid,
-                                              bool direct_ok, int s0, int s1) {
+                                              bool direct_ok, int s0, int s1, int p_raw = kNoLength) {
   constexpr int LPR = D / 8;
   constexpr int RG = kThreads / LPR;
   int tid = threadIdx.x;
@@ -552,7 +562,7 @@ __device__ __forceinline__ void process_range(const DecodeArgs &a, int b, int hg
   int kv_end = s1;  // keys [s0, kv_end) come from the cache
   Frag8<T> kr0[QKV && HOIST ? U : 1], vr0[QKV && HOIST ? U : 1];
   if constexpr (QKV) {
-    int p_new = a.seq_lens[b];
+    int p_new = p_raw != kNoLength ? p_raw : a.seq_lens[b];  // (the caller may have it from the plan cache)
     p_new = p_new < 0 ? 0 : p_new;
     mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
     if (mine) kv_end = p_new;
@@ -801,7 +811,7 @@ constexpr int mfma_lds_bytes() {
 
 template <int D, bool QKV, bool PAGED = false>
 __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, int hg, int split, int n_valid,
-                                                   bool direct_ok, int s0, int s1) {
+                                                   bool direct_ok, int s0, int s1, int p_raw = kNoLength) {
   constexpr int KK = D / 32;   // MFMA steps over d for S^T
   constexpr int DT = D / 16;   // d tiles of O^T
   constexpr int UPR = D / 8;   // 16-byte units per K/V row
@@ -822,7 +832,7 @@ __device__ __forceinline__ void process_range_mfma(const DecodeArgs &a, int b, i
   int kv_end = s1;  // keys [s0, kv_end) come from the cache
   int p_new = 0;
   if constexpr (QKV) {
-    p_new = a.seq_lens[b];
+    p_new = p_raw != kNoLength ? p_raw : a.seq_lens[b];
     p_new = p_new < 0 ? 0 : p_new;
     mine = p_new < a.max_len && p_new < a.cache_rows && p_new >= s0 && p_new < s1;  // then p_new == s1 - 1
     if (mine) kv_end = p_new;
@@ -1047,7 +1057,7 @@ template <typename T, int D, int G, int U, bool QKV, bool MFMA = false, bool PAG
 // (the decode-step form needs 161 registers: at four workgroups per CU, 128 registers, it spills 37 of them)
 __global__ __launch_bounds__(kThreads, MFMA ? 1 : (QKV ? 3 : 4)) void gqa_decode_split_kernel(DecodeArgs a) {
   // the piece to work on: keys [s0, s1) of sequence b, range `split` of its n_valid ranges
-  int b, hg, split, n_valid, s0, s1;
+  int b, hg, split, n_valid, s0, s1, p_raw = kNoLength;
   bool direct_ok = true;
   if (!a.dynamic) {
     split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
@@ -1067,6 +1077,38 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : (QKV ? 3 : 4)) void gqa_decode
     const int lane = threadIdx.x & 63;
     const int j = static_cast<int>(blockIdx.x) / a.n_hg;
     hg = static_cast<int>(blockIdx.x) % a.n_hg;
+    // What an earlier launch of the same step found for slot j, if the caller keeps a plan cache: kind (0 nothing
+    // to do, 1 one range, 2 "deal again": ranges laid end to end, or rows of zeros to write), sequence, range,
+    // ranges of the sequence, first key, end, the sequence's length before the append, the mark of the launch.
+    // (not for four heads per workgroup on the vector units: the second way in costs that form registers it does
+    // not have to spare at three workgroups per CU)
+    constexpr bool kPlanTable = QKV && (MFMA || G <= 2);
+    bool planned = false;
+    if constexpr (kPlanTable) {
+      if (a.plan_mode == 2) {
+        // the same words in every lane; a launch that records stores to the table, so the loads are vector loads
+        // whatever the address: say that the values are uniform, so that what follows lives in scalar registers
+        const int4 *e = reinterpret_cast<const int4 *>(a.plan_cache + 8 * j);
+        const int4 lo = e[0], hi = e[1];
+        const int kind = uni(lo.x), mark = uni(hi.w);
+        if (mark == a.plan_check && kind == 0) return;
+        if (mark == a.plan_check && kind == 1) {
+          b = uni(lo.y), split = uni(lo.z), n_valid = uni(lo.w), s0 = uni(hi.x), s1 = uni(hi.y), p_raw = uni(hi.z);
+          planned = true;
+        }
+      }
+    }
+    if (!planned) {
+    auto record = [&](int kind, int rb, int rsplit, int rn, int rs0, int rs1) {
+      if constexpr (kPlanTable) {
+        if (a.plan_mode == 1 && hg == 0 && threadIdx.x == 0) {
+          int *e = a.plan_cache + 8 * j;
+          e[0] = kind, e[1] = rb, e[2] = rsplit, e[3] = rn, e[4] = rs0, e[5] = rs1;
+          e[6] = kind == 1 ? a.seq_lens[rb] : 0;
+          e[7] = a.plan_check;
+        }
+      }
+    };
     const bool live = lane < a.B;
     const int len = live ? clamped_len(a.seq_lens, lane, a.max_len, a.len_add) : 0;
     // sum of lengths in units of 64 keys (rounded up per sequence): fits an int for any supported size
@@ -1088,6 +1130,7 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : (QKV ? 3 : 4)) void gqa_decode
     // a slot can leave at most one piece per sequence, so `active` partial slots per sequence suffice
     const bool end_to_end = a.active <= a.split_stride && total64 < (1 << 24) && longest - c_even > slack;
     if (end_to_end) {
+      record(2, 0, 0, 0, 0, 0);
       const int start = wave_prefix_i(len, lane) - len;  // where this lane's sequence begins on the line
       const int total = __builtin_amdgcn_readlane(start + len, 63);
       int cc = (total + a.active - 1) / a.active;
@@ -1124,7 +1167,10 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : (QKV ? 3 : 4)) void gqa_decode
     }
     const int first = wave_prefix_i(n, lane) - n;
     const unsigned long long hit = __ballot(j >= first && j < first + n);
-    if (hit == 0ull) return;  // a slot the lengths of this launch leave unused
+    if (hit == 0ull) {  // a slot the lengths of this launch leave unused
+      record(0, 0, 0, 0, 0, 0);
+      return;
+    }
     // the same in every lane: say so, so that everything derived from it lives in scalar registers
     b = uni(__ffsll(hit) - 1);
     split = j - __builtin_amdgcn_readlane(first, b);
@@ -1135,14 +1181,18 @@ __global__ __launch_bounds__(kThreads, MFMA ? 1 : (QKV ? 3 : 4)) void gqa_decode
     s0 = split * chunk;
     s1 = min(s0 + chunk, len_b);
     if (s0 >= len_b) {
+      record(len_b == 0 && split == 0 ? 2 : 0, 0, 0, 0, 0, 0);
       if (len_b == 0 && split == 0) write_zero_rows<T, D, G, MFMA>(a, b, hg);
       return;
     }
+    record(1, b, split, n_valid, s0, s1);
+    }
+    b = uni(b), split = uni(split), n_valid = uni(n_valid), s0 = uni(s0), s1 = uni(s1), p_raw = uni(p_raw);
   }
   if constexpr (MFMA)
-    process_range_mfma<D, QKV, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+    process_range_mfma<D, QKV, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1, p_raw);
   else
-    process_range<T, D, G, U, QKV, true, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1);
+    process_range<T, D, G, U, QKV, true, PAGED>(a, b, hg, split, n_valid, direct_ok, s0, s1, p_raw);
 }
 
 // Cross-split merge: one workgroup of D threads per (sequence, query head).
@@ -1295,6 +1345,31 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
   a.scale_log2e = 1.4426950408889634f / sqrtf(static_cast<float>(D));
   a.part_acc = nullptr;
   a.part_ml = nullptr;
+  a.plan_mode = 0;
+  if (plan.dynamic && axhip_plan_reuse() != 0 && plan.active <= kPlanSlots && (mfma || G <= 2)) {
+    static std::atomic<int *> cache[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return AXHIP_DEVICE_ERROR;
+    int *p = cache[dev].load(std::memory_order_acquire);
+    if (!p) {
+      if (hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_plan_cache)) != hipSuccess || !p) {
+        (void)hipGetLastError();
+        return AXHIP_DEVICE_ERROR;
+      }
+      cache[dev].store(p, std::memory_order_release);
+    }
+    a.plan_cache = p + static_cast<size_t>(axhip_ticket_lane()) * kPlanSlots * 8;
+    a.plan_mode = axhip_plan_reuse();
+    // entries left by a launch of another shape, or dealt for other lengths storage, are not taken
+    unsigned h = 2166136261u;
+    for (const long long v : {static_cast<long long>(B), static_cast<long long>(Hq), static_cast<long long>(G),
+                              static_cast<long long>(max_len), static_cast<long long>(plan.active),
+                              static_cast<long long>(plan.stride), static_cast<long long>(a.len_add),
+                              static_cast<long long>(a.cache_rows),
+                              static_cast<long long>(reinterpret_cast<uintptr_t>(a.seq_lens))})
+      for (int i = 0; i < 8; ++i) h = (h ^ static_cast<unsigned>((v >> (8 * i)) & 255)) * 16777619u;
+    a.plan_check = static_cast<int>(h | 1u);  // (never 0, which a cache nobody has written holds)
+  }
   // the length-dealt plan always merges in the kernel (a second kernel could not be skipped when no
   // sequence needs it); the static plan does unless the two-kernel form was asked for
   a.fused_merge = ((plan.dynamic || !g_tuning.separate_merge) && static_cast<long>(B) * (Hq / G) <= kTicketSlots) ? 1 : 0;

@@ -144,6 +144,7 @@ void *acquire_locked(int dev, size_t rounded) {
 
 hipStream_t current_stream() { return t_capturing ? t_capture_stream : nullptr; }
 thread_local int t_ticket_lane = 0;
+thread_local int t_plan_reuse = 0;
 
 }  // namespace
 }  // namespace axhip
@@ -338,6 +339,12 @@ AXHIP_API int axhip_set_ticket_lane(int lane) {
   return AXHIP_OK;
 }
 AXHIP_API int axhip_ticket_lane(void) { return t_ticket_lane; }
+AXHIP_API int axhip_set_plan_reuse(int mode) {
+  if (mode < 0 || mode > 2) return AXHIP_INVALID_ARGUMENT;
+  t_plan_reuse = mode;
+  return AXHIP_OK;
+}
+AXHIP_API int axhip_plan_reuse(void) { return t_plan_reuse; }
 AXHIP_API int axhip_is_capturing(void) { return t_capturing ? 1 : 0; }
 
 AXHIP_API int axhip_synchronize(void) {

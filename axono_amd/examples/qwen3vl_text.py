@@ -146,7 +146,7 @@ class Qwen3VLTextDecoder(nn.Module):
     prefill of a sequence then runs over one dense scratch block and is copied into the sequence's pages."""
 
     def __init__(self, cfg: TextConfig, weights: dict, batch: int, max_len: int, device: str = "hip", paged: bool = False,
-                 n_pages: int | None = None, fused_tail: bool | None = None):
+                 n_pages: int | None = None, fused_tail: bool | None = None, plan_reuse: bool = True):
         super().__init__()
         self._cfg = cfg
         self._device = device
@@ -188,6 +188,8 @@ class Qwen3VLTextDecoder(nn.Module):
         if fused_tail and not can:
             raise ValueError("decode_layer_tail is not built for these widths")
         self._fused_tail = can if fused_tail is None else bool(fused_tail)
+        # the attention launches of a step deal the same lengths: layer 0 deals, the others take its table
+        self._plan_reuse = bool(plan_reuse)
         if self._fused_tail:
             nbytes = self._lib.axhip_decode_layer_tail_workspace_bytes(cfg.hidden_size, cfg.intermediate_size)
             self._tail_ws = Tensor(DataType.INT8, [nbytes], device)
@@ -205,10 +207,14 @@ class Qwen3VLTextDecoder(nn.Module):
         cfg, cache = self._cfg, self._cache
         args = (qkv, self._w(p + "self_attn.q_norm.weight"), self._w(p + "self_attn.k_norm.weight"), cfg.rms_norm_eps, pos,
                 self._inv_freq, cfg.mrope_section, cache.seq_lens, *cache.get(i))
-        if self._paged:
-            return L.gqa_decode_attention_qkv_paged(*args, cache.page_table, cfg.num_attention_heads, max_len,
-                                                    workspace=self._attn_ws)
-        return L.gqa_decode_attention_qkv(*args, cfg.num_attention_heads, max_len, workspace=self._attn_ws)
+        L.set_plan_reuse((1 if i == 0 else 2) if self._plan_reuse else 0)
+        try:
+            if self._paged:
+                return L.gqa_decode_attention_qkv_paged(*args, cache.page_table, cfg.num_attention_heads, max_len,
+                                                        workspace=self._attn_ws)
+            return L.gqa_decode_attention_qkv(*args, cfg.num_attention_heads, max_len, workspace=self._attn_ws)
+        finally:
+            L.set_plan_reuse(0)
 
     def _linear(self, x, name):
         """x @ W^T over the packed copy of the weight (skinny kernels in decode, MFMA GEMM in prefill)."""

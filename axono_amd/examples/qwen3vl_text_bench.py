@@ -130,7 +130,7 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
 
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
         cpu_step_hook=None, cfg: TextConfig | None = None, kernel_table: bool = True, paged: bool = False,
-        fused_tail: bool | None = None) -> dict:
+        fused_tail: bool | None = None, plan_reuse: bool = True) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
     after the prefill with the model positioned at the first decode step (the benchmark passes a
     hook that times and compares a CPU restatement of one step); its dict is merged into the result."""
@@ -140,7 +140,8 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     log(f"[decode] random weights: {sum(w.size for w in weights.values()) / 1e9:.2f} G params in {time.perf_counter() - t0:.1f} s")
     max_len = context + decode_steps + 1
     max_len = (max_len + 127) // 128 * 128
-    model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0", paged=paged, fused_tail=fused_tail)
+    model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0", paged=paged, fused_tail=fused_tail,
+                               plan_reuse=plan_reuse)
     rng = np.random.default_rng(seed + 1)
     ids = rng.integers(0, cfg.vocab_size, (batch, context)).astype(np.int64)
 
@@ -216,6 +217,9 @@ def main(argv=None):
     ap.add_argument("--paged", action="store_true", help="keep the KV cache in pages of 128 keys (nn.PagedKVCache)")
     ap.add_argument("--no-fused-tail", action="store_true",
                     help="run the part of a layer behind its attention as six launches instead of one persistent launch")
+    ap.add_argument("--no-plan-reuse", action="store_true",
+                    help="every attention launch of a step deals the key ranges itself (default: the first layer's "
+                         "launch deals, the others take its table)")
     ap.add_argument("--no-kernel-table", action="store_true",
                     help="skip the per-kernel table (its extra launches would mix into a profiler's kernel statistics)")
     args = ap.parse_args(argv)
@@ -224,7 +228,7 @@ def main(argv=None):
         _lib.load().axhip_gqa_decode_tune(-1, args.gqa_two_kernels)
     res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
               kernel_table=not args.no_kernel_table, paged=args.paged,
-              fused_tail=False if args.no_fused_tail else None)
+              fused_tail=False if args.no_fused_tail else None, plan_reuse=not args.no_plan_reuse)
     print(json.dumps(res), flush=True)
 
 

@@ -857,6 +857,14 @@ def set_ticket_lane(lane: int) -> None:
     check(_lib_().axhip_set_ticket_lane(int(lane)), "set_ticket_lane")
 
 
+def set_plan_reuse(mode: int) -> None:
+    """The attention launches of one decode step deal the same lengths the same way: mode 1 makes the next
+    gqa_decode_qkv launches of this thread leave what they dealt in a device table, mode 2 makes them take it
+    from there, mode 0 (default) is every launch for itself.  A mode-2 launch must follow a mode-1 launch of the
+    same lengths (same seq_lens tensor and contents) and shape on the same stream."""
+    check(_lib_().axhip_set_plan_reuse(int(mode)), "set_plan_reuse")
+
+
 class HIPGraph:
     """The binding-level graph object (the reference's CUDAGraph class, nanobind_module.cpp:1228-1324):
     capture(fn) = reset the capture pool, run fn once with pool recording on, begin capture, run fn

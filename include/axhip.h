@@ -493,6 +493,17 @@ AXHIP_API int axhip_gqa_decode_qkv(const float *q, int64_t q_stride, const float
                                    size_t workspace_bytes, int cache_dtype, int B, int Hq, int Hkv, int D,
                                    int cache_rows, int max_len, axhip_stream stream);
 
+/* The attention launches of one decode step (one per layer) are given the same seq_lens, and each deals the key
+ * ranges to its workgroups from them in the same way.  With mode 1 set on the calling thread, an
+ * axhip_gqa_decode_qkv[_paged] launch also leaves what each workgroup slot found in a table on the device (per
+ * ticket lane); with mode 2 a launch takes its ranges from that table instead of dealing again.  Mode 0
+ * (default): every launch deals for itself.  A captured launch keeps the mode it was captured under.  The
+ * caller promises, for a mode-2 launch: the mode-1 launch before it on the same stream had the same seq_lens
+ * pointer and contents, B, heads, max_len and cache_rows.  A mode-2 launch whose shape or seq_lens pointer
+ * differs from the table's deals for itself; same results either way.  No reference counterpart. */
+AXHIP_API int axhip_set_plan_reuse(int mode);
+AXHIP_API int axhip_plan_reuse(void);
+
 /* axhip_gqa_decode_qkv over a paged cache (pools, page table, max_pages, n_pages as for
  * axhip_gqa_decode_paged; FLOAT16 caches): the new token's k / v row goes to row seq_lens[b] % 128 of page
  * page_table[b, seq_lens[b] / 128] - that page must already be in the table - when seq_lens[b] < max_len, and

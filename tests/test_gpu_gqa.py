@@ -402,6 +402,32 @@ def _check_decode_step_form(Hq, Hkv, D, lens, rows, max_len, forced=(0, 5), seed
                                               gv.astype(np.float32), attended)
         got = out.download(np.float16, (B, Hq, D)).astype(np.float32)
         assert np.abs(got - want).max() <= 2e-3, (force_splits, np.abs(got - want).max())
+        if force_splits == 0:
+            # the launches of one step share what the first dealt: a launch that leaves its table, launches that take
+            # it (twice: the table must survive being read), and one of another max_len, which the table is not for
+            def launch(mode, ml):
+                dkc.upload(kc.reshape(-1))
+                dvc.upload(vc.reshape(-1))
+                out.upload(np.full(B * Hq * D // 2, np.nan, np.float32))
+                assert l.axhip_set_plan_reuse(mode) == 0
+                try:
+                    gu._run("axhip_gqa_decode_qkv", dq.ptr, width, dq.ptr + Hq * D * 4, width, dq.ptr + (Hq + Hkv) * D * 4,
+                            width, dqw.ptr, dkw.ptr, gu.F32, 1e-6, dp.ptr, di.ptr, hw, hw, dl.ptr, dkc.ptr, dvc.ptr, out.ptr,
+                            ws.ptr, wsb, gu.F16, B, Hq, Hkv, D, rows, ml, None)
+                finally:
+                    l.axhip_set_plan_reuse(0)
+                gu.synchronize()
+                return (out.download(np.uint16, (B, Hq, D)), dkc.download(np.uint16, kc.shape),
+                        dvc.download(np.uint16, vc.shape))
+            plain = launch(0, max_len)
+            np.testing.assert_array_equal(plain[0], got.astype(np.float16).view(np.uint16))
+            for mode in (1, 2, 2):
+                for a_, b_ in zip(launch(mode, max_len), plain):
+                    np.testing.assert_array_equal(a_, b_)
+            if max_len > 300:
+                shorter = launch(0, max_len - 128)
+                for a_, b_ in zip(launch(2, max_len - 128), shorter):
+                    np.testing.assert_array_equal(a_, b_)
     l.axhip_gqa_decode_tune(0, 0)
     return dq, dp, di, dl, dkc, dvc, out, ws, wsb, width, hw
 

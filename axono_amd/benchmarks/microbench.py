@@ -453,7 +453,7 @@ def main(argv=None):
     ap.add_argument("--waves", type=int, default=0, help="linear: wavefronts (K slices) per workgroup (4, 8, 16)")
     ap.add_argument("--M", type=int, default=0, help="linear: only this row count")
     ap.add_argument("--gemm-rows", type=int, default=0, help="linear: rows of x per GEMM workgroup (64 or 128)")
-    ap.add_argument("--rot", type=int, default=0, help="linear: number of weight copies rotated through (1 = cache-hot)")
+    ap.add_argument("--rot", type=int, default=0, help="linear, gqa-step: number of weight / cache copies rotated through (1 = cache-hot)")
     args = ap.parse_args(argv)
     global ZERO_DATA
     ZERO_DATA = bool(args.zero_data)
@@ -483,7 +483,7 @@ def main(argv=None):
         bench_gqa_paged(lib, 32, 32768, 20, np.random.default_rng(0).integers(512, 32769, 32))
     elif args.what == "gqa-step":
         bench_gqa_step_form(lib, args.B if args.B != 32 else 16, args.L if args.L != 8192 else 4160, args.steps,
-                            rows=args.rows or None)
+                            rows=args.rows or None, n_rot=args.rot or 4)
     elif args.what == "gqa-single":
         # the reference's own call: one sequence, q (1,Hq,D), K/V (L,Hkv,D) token-major, fp32 (and the same in fp16)
         for fp32 in (True, False):

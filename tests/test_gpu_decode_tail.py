@@ -2,7 +2,8 @@
 layer's q/k/v Linear in one persistent launch) against the CPU oracle's single operators with the same fp16
 storage points: the activation entering each Linear and `act` are fp16, everything else fp32.  Tolerances: the
 residual stream differs by fp32 summation order and, behind a norm, by activations that round to the neighbouring
-fp16 value (2e-3 + 1e-3 |value|, the fp16 bound of the other decode-path tests)."""
+fp16 value (1e-3 in all; values up to 14); and, tighter, the device may be no
+farther from the same composition evaluated in float64 (same storage points) than 1.5 x what the fp32 oracle is."""
 import ctypes as C
 
 import numpy as np
@@ -10,6 +11,7 @@ import pytest
 
 import gpu_util as gu
 from oracle import port
+from oracle.f64_ops import F64Ops
 
 pytestmark = pytest.mark.gpu
 
@@ -28,16 +30,17 @@ def _pack(w, glu=False):
     return p
 
 
-def _oracle(attn, h_in, wo, w_post, wgu, wd, w_next, wn, eps):
-    f = lambda a: np.asarray(a, np.float32)
+def _oracle(attn, h_in, wo, w_post, wgu, wd, w_next, wn, eps, ops=port, f=np.float32):
+    """The composition with the oracle's operators (ops=port, fp32) or in float64 (ops=F64Ops(), f=np.float64)."""
+    c = lambda a: np.asarray(a, f)
     inter = wd.shape[1]
-    h_mid = port.linear(f(attn), f(wo)) + h_in
-    xn2 = f(h16(port.rms_norm(h_mid, w_post, eps)))
-    gu_ = port.linear(xn2, f(wgu))
-    act = h16(port.silu_mul(np.ascontiguousarray(gu_[:, :inter]), np.ascontiguousarray(gu_[:, inter:])))
-    h_out = port.linear(f(act), f(wd)) + h_mid
-    xn = f(h16(port.rms_norm(h_out, w_next, eps)))
-    return h_out, port.linear(xn, f(wn))
+    h_mid = ops.linear(c(attn), c(wo)) + c(h_in)
+    xn2 = c(h16(ops.rms_norm(h_mid, w_post, eps)))
+    gu_ = ops.linear(xn2, c(wgu))
+    act = h16(ops.silu_mul(np.ascontiguousarray(gu_[:, :inter]), np.ascontiguousarray(gu_[:, inter:])))
+    h_out = ops.linear(c(act), c(wd)) + h_mid
+    xn = c(h16(ops.rms_norm(h_out, w_next, eps)))
+    return h_out, ops.linear(xn, c(wn))
 
 
 @pytest.mark.parametrize("M,H,K1,I,N_next", [(16, 512, 512, 1024, 512), (5, 512, 512, 1024, 1024), (1, 512, 512, 1024, 16),
@@ -64,6 +67,7 @@ def test_layer_tail_matches_operator_composition(M, H, K1, I, N_next):
         attn_i = h16(attn * (1.0 + 0.5 * it))
         h_i = (h_in * (1.0 - 0.3 * it)).astype(np.float32)
         want = _oracle(attn_i, h_i, wo, w_post, wgu, wd, w_next, wn, eps)
+        exact = _oracle(attn_i, h_i, wo, w_post, wgu, wd, w_next, wn, eps, ops=F64Ops(), f=np.float64)
         d_attn, d_h = gu.dev(attn_i), gu.dev(h_i)
         print(f"tail M={M} H={H} I={I} N_next={N_next} launch {it}", flush=True)
         gu._run("axhip_decode_layer_tail", d_attn.ptr, d_h.ptr, p_o.ptr, d_wp.ptr, p_gu.ptr, p_d.ptr, d_wn.ptr,
@@ -71,12 +75,17 @@ def test_layer_tail_matches_operator_composition(M, H, K1, I, N_next):
         gu.synchronize()
         assert l.axhip_decode_layer_tail_status(0, C.byref(failed)) == 0 and failed.value == 0
         got = (h_out.download(np.float32, (M, H)), y.download(np.float32, (M, N_next)))
-        for name, g_, w_ in (("h_out", got[0], want[0]), ("y", got[1], want[1])):
+        for name, g_, w_, e_ in (("h_out", got[0], want[0], exact[0]), ("y", got[1], want[1], exact[1])):
             err = np.abs(g_ - w_)
-            print(f"  {name}: max abs err {float(err.max()):.3e} (max |value| {float(np.abs(w_).max()):.3f})", flush=True)
-            # 2e-3, plus one part in a thousand where a value is large enough for its fp16 spacing to matter
-            excess = float((err - (2e-3 + 1e-3 * np.abs(w_))).max())
-            assert excess <= 0.0, (name, excess)
+            d_dev, d_cpu = float(np.abs(g_ - e_).max()), float(np.abs(w_ - e_).max())
+            print(f"  {name}: max abs err {float(err.max()):.3e} (max |value| {float(np.abs(w_).max()):.3f}); against float64: "
+                  f"device {d_dev:.3e}, fp32 oracle {d_cpu:.3e}", flush=True)
+            # a few activations that round to the other fp16 neighbour behind a norm (each moves a sum by about
+            # 2^-11 x |activation| x |weight| <= 2e-4): 1e-3 holds with a factor of two to spare at the large widths
+            assert float(err.max()) <= 1e-3, (name, float(err.max()))
+            # no farther from the float64 evaluation than 1.5 x the fp32 oracle (floor: what one activation that rounds
+            # to the other fp16 neighbour moves a sum, 2^-11 x |activation| x |weight| ~ 5e-4 x 4 x 0.08)
+            assert d_dev <= max(1.5 * d_cpu, 2e-4), (name, d_dev, d_cpu)
         # poison the outputs so that a launch that did nothing cannot pass
         for b in (h_out, y):
             b.upload(np.full(b.nbytes // 4, np.nan, np.float32))

@@ -111,6 +111,8 @@ PROTOTYPES = {
     "axhip_decode_layer_tail_workspace_bytes": (c_sz, [c_i, c_i]),
     "axhip_decode_layer_tail": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz,
                                       c_i, c_i, c_i, c_i, c_i, c_f, c_vp]),
+    "axhip_decode_layer_tail_last": (c_i, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_sz,
+                                           c_i, c_i, c_i, c_i, c_f, c_vp]),
     "axhip_decode_layer_tail_status": (c_i, [c_i, c_vp]),
     "axhip_decode_layer_tail_tune": (None, [c_i]),
     "axhip_decode_layer_tail_trace": (None, [c_vp]),

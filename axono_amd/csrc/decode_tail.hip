@@ -125,6 +125,7 @@ struct TailArgs {
   unsigned char *act;    // activations in MFMA fragment order: 1 KiB per 32 columns, lane (r, g) = 8 halves of row r
   float *h_out;          // [M, H]  out, row-major
   float *y;              // [M, N_next] out, row-major
+  __half *xn;            // N_next == 0 (nothing behind the last norm in this launch): [M, H] out, the normalised rows
   int M, H, K1, I, N_next;
   float eps;
   unsigned long long *dbg;  // measurement: 32 timestamps per workgroup (axhip_decode_layer_tail_trace), or null
@@ -351,6 +352,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
 
   // ---- phase 2: post-attention norm, gate + up, SiLU-mul -------------------------------------------------------------
   half8_t wC[CI], wD[CH];
+  const bool lin4 = a.N_next > 0;  // a Linear behind the last norm (else the launch ends with the normalised rows)
   const __half *pd = a.w_nl + (static_cast<int64_t>(on4 ? wg : 0) * (a.H / 32) + wave * CH) * 512 + lane * 8;
   const __half *pc = a.w_down + (static_cast<int64_t>(on1 ? wg >> 1 : 0) * (a.I / 32) + wave * CI) * 512 + src_lane * 8;
   {
@@ -431,7 +433,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
       for (int j = 0; j < CI; ++j) acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wC[j], bf[j], acc[0], 0, 0, 0);
     }
     STAMP(8);
-    if (wave != 0) {
+    if (wave != 0 && lin4) {
 #pragma unroll
       for (int j = 0; j < CH; ++j) wD[j] = ld_w(pd + j * 512);
     }
@@ -442,6 +444,7 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
   }
   {
     auto pf = [&] {
+      if (!lin4) return;
 #pragma unroll
       for (int j = 0; j < CH; ++j) wD[j] = ld_w(pd + j * 512);
     };
@@ -465,14 +468,24 @@ __global__ __launch_bounds__(kTailThreads) void decode_tail_kernel(TailArgs a) {
       half8_t bf[CH];
 #pragma unroll
       for (int j = 0; j < CH; ++j) bf[j] = norm_frag(hv[j], s_wn + a.H, (wave * CH + j) * 32 + g * 8, rs);
+      if (lin4) {
 #pragma unroll
-      for (int j = 0; j < CH; ++j) acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wD[j], bf[j], acc[0], 0, 0, 0);
+        for (int j = 0; j < CH; ++j) acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wD[j], bf[j], acc[0], 0, 0, 0);
+      } else if (wg < kTailWaves && wave == wg && r < a.M) {
+        // every workgroup holds all the normalised rows, 32 * CH columns per wavefront: workgroup w writes the
+        // columns of its wavefront w
+#pragma unroll
+        for (int j = 0; j < CH; ++j)
+          *reinterpret_cast<half8_t *>(a.xn + static_cast<int64_t>(r) * a.H + (wave * CH + j) * 32 + g * 8) = bf[j];
+      }
     }
     STAMP(11);
-    total<1>(acc, wave, lane);
-    if (wave == 0) {
-      if (on4 && r < a.M)
-        *reinterpret_cast<float4_t *>(a.y + static_cast<int64_t>(r) * a.N_next + wg * 16 + 4 * g) = acc[0];
+    if (lin4) {
+      total<1>(acc, wave, lane);
+      if (wave == 0) {
+        if (on4 && r < a.M)
+          *reinterpret_cast<float4_t *>(a.y + static_cast<int64_t>(r) * a.N_next + wg * 16 + 4 * g) = acc[0];
+      }
     }
     STAMP(12);
   }
@@ -497,7 +510,7 @@ int launch_tail(const TailArgs &a, int wgs, hipStream_t st) {
 // 1 = <4,4,12,3> (K1 = H = 2048, I = 6144), 2 = <1,1,2,1> (K1 = H = 512, I = 1024).  Every phase must have at most
 // one unit per resident workgroup (one workgroup per compute unit, 256 at most).
 int tail_instance(int M, int H, int K1, int I, int N_next, int *wgs_out) {
-  if (M < 0 || M > kTailRows || H <= 0 || K1 <= 0 || I <= 0 || N_next <= 0) return 0;
+  if (M < 0 || M > kTailRows || H <= 0 || K1 <= 0 || I <= 0 || N_next < 0) return 0;  // N_next 0: no Linear behind
   if (H % 512 != 0 || K1 % 512 != 0 || I % 512 != 0 || N_next % 16 != 0 || H > kTailMaxH) return 0;
   const int cus = device_cu_count();
   const int wgs = cus < kTailMaxWgs ? cus : kTailMaxWgs;
@@ -510,6 +523,7 @@ int tail_instance(int M, int H, int K1, int I, int N_next, int *wgs_out) {
       break;
     }
   if (nt2 == 0 || H / 8 > wgs || N_next / 16 > wgs) return 0;
+  if (N_next == 0 && wgs < kTailWaves) return 0;  // one workgroup per wavefront's columns writes the normalised rows
   if (ck1 == 4 && ch == 4 && ci == 12 && nt2 == 3) return 1;
   if (ck1 == 1 && ch == 1 && ci == 2 && nt2 == 1) return 2;
   return 0;
@@ -517,6 +531,56 @@ int tail_instance(int M, int H, int K1, int I, int N_next, int *wgs_out) {
 
 size_t tail_workspace_bytes(int H, int I) {
   return 2 * static_cast<size_t>(H / 8) * kHBlockBytes + static_cast<size_t>(I) * 32;
+}
+
+// The launch behind both entry points: N_next > 0 ends with y = norm(h_out) . w_next_linear^T, N_next == 0 with
+// xn = norm(h_out) as fp16 rows.
+int tail_entry(const void *attn, const float *h_in, const void *w_o, const float *w_post, const void *w_gate_up,
+               const void *w_down, const float *w_next, const void *w_next_linear, float *h_out, float *y, void *xn,
+               void *workspace, size_t workspace_bytes, int M, int H, int K1, int I, int N_next, float eps,
+               axhip_stream stream) {
+  int wgs = 0;
+  const int instance = tail_instance(M, H, K1, I, N_next, &wgs);
+  if (instance == 0) return AXHIP_INVALID_ARGUMENT;  // widths this launch is not built for: use the single operators
+  if (M == 0) return AXHIP_OK;
+  if (!attn || !h_in || !w_o || !w_post || !w_gate_up || !w_down || !w_next || !h_out || !workspace)
+    return AXHIP_INVALID_PTR;
+  if (N_next > 0 ? (!w_next_linear || !y) : !xn) return AXHIP_INVALID_PTR;
+  if (h_in == h_out) return AXHIP_INVALID_ARGUMENT;  // lines of h_in are in the L2s when h_out is written
+  const uintptr_t all = reinterpret_cast<uintptr_t>(attn) | reinterpret_cast<uintptr_t>(h_in) |
+                        reinterpret_cast<uintptr_t>(w_post) | reinterpret_cast<uintptr_t>(w_next) |
+                        reinterpret_cast<uintptr_t>(h_out) | reinterpret_cast<uintptr_t>(y) |
+                        reinterpret_cast<uintptr_t>(xn) | reinterpret_cast<uintptr_t>(w_o) |
+                        reinterpret_cast<uintptr_t>(w_gate_up) | reinterpret_cast<uintptr_t>(w_down) |
+                        reinterpret_cast<uintptr_t>(w_next_linear);
+  if (all & 15) return AXHIP_INVALID_PTR;
+  if (reinterpret_cast<uintptr_t>(workspace) & 127) return AXHIP_INVALID_PTR;
+  if (workspace_bytes < tail_workspace_bytes(H, I)) return AXHIP_INVALID_ARGUMENT;
+  TailArgs a;
+  a.attn = static_cast<const __half *>(attn);
+  a.h_in = h_in;
+  a.w_o = static_cast<const __half *>(w_o);
+  a.w_post = w_post;
+  a.w_gu = static_cast<const __half *>(w_gate_up);
+  a.w_down = static_cast<const __half *>(w_down);
+  a.w_next = w_next;
+  a.w_nl = static_cast<const __half *>(w_next_linear);
+  a.hmid = static_cast<unsigned char *>(workspace);
+  a.hout = a.hmid + static_cast<size_t>(H / 8) * kHBlockBytes;
+  a.act = a.hout + static_cast<size_t>(H / 8) * kHBlockBytes;
+  a.h_out = h_out;
+  a.y = y;
+  a.xn = static_cast<__half *>(xn);
+  a.M = M;
+  a.H = H;
+  a.K1 = K1;
+  a.I = I;
+  a.N_next = N_next;
+  a.eps = eps;
+  a.skip = g_tail_skip;
+  a.dbg = g_tail_dbg;
+  hipStream_t st = as_stream(stream);
+  return instance == 1 ? launch_tail<4, 4, 12, 3>(a, wgs, st) : launch_tail<1, 1, 2, 1>(a, wgs, st);
 }
 
 }  // namespace
@@ -536,46 +600,17 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
                                       const void *w_next_linear, float *h_out, float *y, void *workspace,
                                       size_t workspace_bytes, int M, int H, int K1, int I, int N_next, float eps,
                                       axhip_stream stream) {
-  int wgs = 0;
-  const int instance = tail_instance(M, H, K1, I, N_next, &wgs);
-  if (instance == 0) return AXHIP_INVALID_ARGUMENT;  // widths this launch is not built for: use the single operators
-  if (M == 0) return AXHIP_OK;
-  if (!attn || !h_in || !w_o || !w_post || !w_gate_up || !w_down || !w_next || !w_next_linear || !h_out || !y ||
-      !workspace)
-    return AXHIP_INVALID_PTR;
-  if (h_in == h_out) return AXHIP_INVALID_ARGUMENT;  // lines of h_in are in the L2s when h_out is written
-  const uintptr_t all = reinterpret_cast<uintptr_t>(attn) | reinterpret_cast<uintptr_t>(h_in) |
-                        reinterpret_cast<uintptr_t>(w_post) | reinterpret_cast<uintptr_t>(w_next) |
-                        reinterpret_cast<uintptr_t>(h_out) | reinterpret_cast<uintptr_t>(y) |
-                        reinterpret_cast<uintptr_t>(w_o) | reinterpret_cast<uintptr_t>(w_gate_up) |
-                        reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(w_next_linear);
-  if (all & 15) return AXHIP_INVALID_PTR;
-  if (reinterpret_cast<uintptr_t>(workspace) & 127) return AXHIP_INVALID_PTR;
-  if (workspace_bytes < tail_workspace_bytes(H, I)) return AXHIP_INVALID_ARGUMENT;
-  TailArgs a;
-  a.attn = static_cast<const __half *>(attn);
-  a.h_in = h_in;
-  a.w_o = static_cast<const __half *>(w_o);
-  a.w_post = w_post;
-  a.w_gu = static_cast<const __half *>(w_gate_up);
-  a.w_down = static_cast<const __half *>(w_down);
-  a.w_next = w_next;
-  a.w_nl = static_cast<const __half *>(w_next_linear);
-  a.hmid = static_cast<unsigned char *>(workspace);
-  a.hout = a.hmid + static_cast<size_t>(H / 8) * kHBlockBytes;
-  a.act = a.hout + static_cast<size_t>(H / 8) * kHBlockBytes;
-  a.h_out = h_out;
-  a.y = y;
-  a.M = M;
-  a.H = H;
-  a.K1 = K1;
-  a.I = I;
-  a.N_next = N_next;
-  a.eps = eps;
-  a.skip = g_tail_skip;
-  a.dbg = g_tail_dbg;
-  hipStream_t st = as_stream(stream);
-  return instance == 1 ? launch_tail<4, 4, 12, 3>(a, wgs, st) : launch_tail<1, 1, 2, 1>(a, wgs, st);
+  if (N_next <= 0) return AXHIP_INVALID_ARGUMENT;
+  return tail_entry(attn, h_in, w_o, w_post, w_gate_up, w_down, w_next, w_next_linear, h_out, y, nullptr, workspace,
+                    workspace_bytes, M, H, K1, I, N_next, eps, stream);
+}
+
+AXHIP_API int axhip_decode_layer_tail_last(const void *attn, const float *h_in, const void *w_o, const float *w_post,
+                                           const void *w_gate_up, const void *w_down, const float *w_final_norm,
+                                           float *h_out, void *xn_out, void *workspace, size_t workspace_bytes, int M,
+                                           int H, int K1, int I, float eps, axhip_stream stream) {
+  return tail_entry(attn, h_in, w_o, w_post, w_gate_up, w_down, w_final_norm, nullptr, h_out, nullptr, xn_out, workspace,
+                    workspace_bytes, M, H, K1, I, 0, eps, stream);
 }
 
 AXHIP_API int axhip_decode_layer_tail_supported(int M, int H, int K1, int I, int N_next) {

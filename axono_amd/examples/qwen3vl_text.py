@@ -146,7 +146,8 @@ class Qwen3VLTextDecoder(nn.Module):
     prefill of a sequence then runs over one dense scratch block and is copied into the sequence's pages."""
 
     def __init__(self, cfg: TextConfig, weights: dict, batch: int, max_len: int, device: str = "hip", paged: bool = False,
-                 n_pages: int | None = None, fused_tail: bool | None = None, plan_reuse: bool = True):
+                 n_pages: int | None = None, fused_tail: bool | None = None, plan_reuse: bool = True,
+                 fused_last: bool = True):
         super().__init__()
         self._cfg = cfg
         self._device = device
@@ -190,6 +191,8 @@ class Qwen3VLTextDecoder(nn.Module):
         self._fused_tail = can if fused_tail is None else bool(fused_tail)
         # the attention launches of a step deal the same lengths: layer 0 deals, the others take its table
         self._plan_reuse = bool(plan_reuse)
+        # the last layer through the same launch, closed by the final norm (False: as single operators)
+        self._fused_last = bool(fused_last)
         if self._fused_tail:
             nbytes = self._lib.axhip_decode_layer_tail_workspace_bytes(cfg.hidden_size, cfg.intermediate_size)
             self._tail_ws = Tensor(DataType.INT8, [nbytes], device)
@@ -270,6 +273,14 @@ class Qwen3VLTextDecoder(nn.Module):
                                              self._w(n + "input_layernorm.weight"),
                                              self._packed[n + "self_attn.qkv_proj.weight"], n_qkv, cfg.rms_norm_eps,
                                              self._tail_ws)
+                continue
+            if self._fused_tail and self._fused_last:
+                # the last layer: the same launch, closed by the final norm (the rows the lm_head reads)
+                h, xn = L.decode_layer_tail_last(attn.reshape([B, nqd]), h, self._packed[p + "self_attn.o_proj.weight"],
+                                                 self._w(p + "post_attention_layernorm.weight"),
+                                                 self._packed[p + "mlp.gate_up_proj.weight"],
+                                                 self._packed[p + "mlp.down_proj.weight"], self._w("norm.weight"),
+                                                 cfg.rms_norm_eps, self._tail_ws)
                 continue
             attn_out = self._linear(attn.reshape([B, nqd]), p + "self_attn.o_proj.weight")
             h, xn2 = L.add_rms_norm(attn_out, h, self._w(p + "post_attention_layernorm.weight"), cfg.rms_norm_eps,

@@ -73,17 +73,17 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
         return 2 * K * N + 2 * B * K + out_b * B * N
 
     fused = model._fused_tail
-    per = (lambda n: 1 if fused else n)   # with the fused launch only one layer runs these as single launches
+    per = (lambda n: 0 if fused else n)   # with the fused launch no layer runs these as single launches
     n_qkv = (nq + 2 * nkv) * D
     kinds = [
-        ("qkv Linear 2048->4096", nl, per(nl), lin_bytes(H, n_qkv, 4),
+        ("qkv Linear 2048->4096", nl, 1 if fused else nl, lin_bytes(H, n_qkv, 4),
          layers(lambda p, i: model._linear(xn, p + "self_attn.qkv_proj.weight"))),
         ("attention (qk-norm + M-RoPE + KV append + split-K decode + merge)", nl, nl,
          2 * nkv * D * 2 * B * (context + 1) + B * n_qkv * 4 + B * nq * D * 2,
          layers(lambda p, i: model._attention_step(qkv, p, i, model._pos, model._decode_bound))),
         ("o_proj Linear 2048->2048", nl, per(nl), lin_bytes(nq * D, H, 4),
          layers(lambda p, i: model._linear(attn, p + "self_attn.o_proj.weight"))),
-        ("add + RMSNorm (fp32 residual, fp16 out)", 2 * nl, 2 if fused else 2 * nl, B * H * (4 + 4 + 4 + 2) + 4 * H,
+        ("add + RMSNorm (fp32 residual, fp16 out)", 2 * nl, 0 if fused else 2 * nl, B * H * (4 + 4 + 4 + 2) + 4 * H,
          lambda: [L.add_rms_norm(o32, h, W(f"layers.{i // 2}.post_attention_layernorm.weight"), cfg.rms_norm_eps,
                                  DataType.FLOAT16) for i in range(2 * nl)]),
         ("gate+up Linear 2048->12288 + SiLU-mul", nl, per(nl), lin_bytes(H, 2 * I, 1),
@@ -109,6 +109,19 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
         kinds.insert(2, ("layer tail: o_proj + norm + gate/up + SiLU-mul + down + norm + next qkv, one persistent launch",
                          nl - 1, nl - 1, 2 * (nq * D * H + 2 * I * H + H * I + n_qkv * H) + B * (nq * D * 2 + 2 * H * 4 + n_qkv * 4),
                          tails))
+
+        def last_tails():
+            hh = h
+            for i in range(nl):
+                p = f"layers.{i}."
+                hh, _ = L.decode_layer_tail_last(attn, hh, model._packed[p + "self_attn.o_proj.weight"],
+                                                 W(p + "post_attention_layernorm.weight"),
+                                                 model._packed[p + "mlp.gate_up_proj.weight"],
+                                                 model._packed[p + "mlp.down_proj.weight"], W("norm.weight"), cfg.rms_norm_eps,
+                                                 model._tail_ws)
+        kinds.insert(3, ("last layer's tail: the same launch closed by the final norm", nl, 1,
+                         2 * (nq * D * H + 2 * I * H + H * I) + B * (nq * D * 2 + 2 * H * 4 + H * 2), last_tails))
+        # the single operators below are not part of the fused step: listed for comparison
     rows = []
     for name, graph_calls, calls, nbytes, fn in kinds:
         g = HIPGraph()
@@ -130,7 +143,8 @@ def per_kernel_table(model: Qwen3VLTextDecoder, context: int, reps: int = 10, on
 
 def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int = 0, log=print,
         cpu_step_hook=None, cfg: TextConfig | None = None, kernel_table: bool = True, paged: bool = False,
-        fused_tail: bool | None = None, plan_reuse: bool = True) -> dict:
+        fused_tail: bool | None = None, plan_reuse: bool = True,
+        fused_last: bool = True) -> dict:
     """cpu_step_hook(cfg, weights, model, first_ids, pos, batch, max_len, log) -> dict, if given, runs
     after the prefill with the model positioned at the first decode step (the benchmark passes a
     hook that times and compares a CPU restatement of one step); its dict is merged into the result."""
@@ -141,7 +155,7 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     max_len = context + decode_steps + 1
     max_len = (max_len + 127) // 128 * 128
     model = Qwen3VLTextDecoder(cfg, weights, batch, max_len, "hip:0", paged=paged, fused_tail=fused_tail,
-                               plan_reuse=plan_reuse)
+                               plan_reuse=plan_reuse, fused_last=fused_last)
     rng = np.random.default_rng(seed + 1)
     ids = rng.integers(0, cfg.vocab_size, (batch, context)).astype(np.int64)
 
@@ -220,6 +234,8 @@ def main(argv=None):
     ap.add_argument("--no-plan-reuse", action="store_true",
                     help="every attention launch of a step deals the key ranges itself (default: the first layer's "
                          "launch deals, the others take its table)")
+    ap.add_argument("--no-fused-last", action="store_true",
+                    help="the last layer as single operators (default: the persistent launch closed by the final norm)")
     ap.add_argument("--no-kernel-table", action="store_true",
                     help="skip the per-kernel table (its extra launches would mix into a profiler's kernel statistics)")
     args = ap.parse_args(argv)
@@ -228,7 +244,8 @@ def main(argv=None):
         _lib.load().axhip_gqa_decode_tune(-1, args.gqa_two_kernels)
     res = run(args.steps, args.batch, args.context, log=lambda *a: print(*a, file=sys.stderr, flush=True),
               kernel_table=not args.no_kernel_table, paged=args.paged,
-              fused_tail=False if args.no_fused_tail else None, plan_reuse=not args.no_plan_reuse)
+              fused_tail=False if args.no_fused_tail else None, plan_reuse=not args.no_plan_reuse,
+              fused_last=not args.no_fused_last)
     print(json.dumps(res), flush=True)
 
 

@@ -625,6 +625,32 @@ def decode_layer_tail(attn: Tensor, h_in: Tensor, w_o: Tensor, w_post: Tensor, w
     return h_out, y
 
 
+def decode_layer_tail_last(attn: Tensor, h_in: Tensor, w_o: Tensor, w_post: Tensor, w_gate_up: Tensor, w_down: Tensor,
+                           w_final_norm: Tensor, eps: float, workspace: Tensor, h_out: Tensor | None = None):
+    """decode_layer_tail for a model's last layer: ends with the final norm instead of a next projection.  Returns
+    (h_out FLOAT32 [M,H], xn FLOAT16 [M,H] = rms_norm(h_out, w_final_norm), the rows the lm_head reads)."""
+    op = "decode_layer_tail_last"
+    _need_hip(op, attn, h_in, w_o, w_post, w_gate_up, w_down, w_final_norm, workspace)
+    if attn.dtype != DataType.FLOAT16 or h_in.dtype != DataType.FLOAT32 or w_post.dtype != DataType.FLOAT32 or \
+            w_final_norm.dtype != DataType.FLOAT32:
+        raise AxhipError(op, Status.UNSUPPORTED_TYPE)
+    m, hidden = h_in.shape
+    k1 = attn.num_elements // m
+    inter = w_down.num_elements // hidden
+    lib = _lib_()
+    need = lib.axhip_decode_layer_tail_workspace_bytes(hidden, inter)
+    if workspace.num_bytes < need or w_post.num_elements != hidden or w_final_norm.num_elements != hidden:
+        raise AxhipError(op, Status.SHAPE_MISMATCH)
+    if h_out is None:
+        h_out = _new(DataType.FLOAT32, [m, hidden], h_in)
+    xn = _new(DataType.FLOAT16, [m, hidden], h_in)
+    check(lib.axhip_decode_layer_tail_last(attn.data_ptr, h_in.data_ptr, w_o.data_ptr, w_post.data_ptr, w_gate_up.data_ptr,
+                                           w_down.data_ptr, w_final_norm.data_ptr, h_out.data_ptr, xn.data_ptr,
+                                           workspace.data_ptr, workspace.num_bytes, m, hidden, k1, inter, float(eps),
+                                           current_stream()), op)
+    return h_out, xn
+
+
 def decode_layer_tail_failed_waits(reset: bool = False) -> int:
     """Barrier waits of decode_layer_tail that ran out since the last reset (0 in a healthy process)."""
     n = C.c_uint(0)

@@ -558,6 +558,14 @@ AXHIP_API int axhip_decode_layer_tail(const void *attn, const float *h_in, const
                                       const void *w_next_linear, float *h_out, float *y, void *workspace,
                                       size_t workspace_bytes, int M, int H, int K1, int I, int N_next, float eps,
                                       axhip_stream stream);
+/* The same launch for the last layer of a model: nothing follows the closing norm, and the launch ends with
+ * xn_out = rmsnorm(h_out, w_final_norm) as FLOAT16 [M, H] (the rows the lm_head reads) instead of y.  Supported
+ * where axhip_decode_layer_tail_supported(M, H, K1, I, 0) is 1.  Replaces the same operator sequence followed by the
+ * model's final norm (examples/vlm/qwen3vl/model.py:408-436, 760-761). */
+AXHIP_API int axhip_decode_layer_tail_last(const void *attn, const float *h_in, const void *w_o, const float *w_post,
+                                           const void *w_gate_up, const void *w_down, const float *w_final_norm,
+                                           float *h_out, void *xn_out, void *workspace, size_t workspace_bytes, int M,
+                                           int H, int K1, int I, float eps, axhip_stream stream);
 /* Barrier waits of axhip_decode_layer_tail that ran out since the last reset (0 in a healthy process); reset != 0
  * also puts the barrier counters back to zero (only while no such launch is in flight). */
 AXHIP_API int axhip_decode_layer_tail_status(int reset, unsigned *failed_waits);

@@ -106,7 +106,7 @@ def test_decode_steps_match_oracle(use_graph):
 @pytest.mark.parametrize("use_graph", [False, True])
 def test_decode_steps_with_the_fused_layer_launch_match_oracle(use_graph):
     """The same comparison at widths the fused layer launch is built for: three such launches per step hand the
-    residual stream and the next q/k/v projection to each other, the fourth layer runs as single operators; three
+    residual stream and the next q/k/v projection to each other, the fourth layer's closes with the final norm; three
     sequences (rows 3 to 15 of the launch's 16 are unused), eager and captured; and the tokens equal those of the
     same model run as single operators."""
     from axono_amd import libaxono as L
@@ -121,7 +121,8 @@ def test_decode_steps_with_the_fused_layer_launch_match_oracle(use_graph):
     gpu.start_decode(first, pos, n_steps)
     if use_graph:
         g = gpu.capture()
-        assert g.num_nodes == 2 * 3 + 7 + 4
+        # embedding + first norm, first q/k/v, (attention, fused launch) x 4, lm_head, argmax, state advance
+        assert g.num_nodes == 2 + 2 * 4 + 3
     toks = gpu.generate(n_steps, use_graph=use_graph)
     assert L.decode_layer_tail_failed_waits() == 0
     cur = first
@@ -399,7 +400,8 @@ def test_captured_step_at_the_real_widths_of_the_2b_shape(fused_tail, n_layers):
     g = gpu.capture()
     # single operators: 7 launches per layer; fused: attention + one launch per layer but the last, whose q/k/v
     # projection the launch before it has already run
-    assert g.num_nodes == (2 * (n_layers - 1) + 7 + 4 if fused_tail else 7 * n_layers + 4)
+    # fused: embedding + first norm, first q/k/v, (attention, fused launch) per layer, lm_head, argmax, state advance
+    assert g.num_nodes == (2 + 2 * n_layers + 3 if fused_tail else 7 * n_layers + 4)
     g.replay()
     h_gpu = [t.to_numpy().copy() for t in trace]
     logits = gpu._graph_out[0].to_numpy().copy()

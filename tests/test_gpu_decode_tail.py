@@ -91,6 +91,53 @@ def test_layer_tail_matches_operator_composition(M, H, K1, I, N_next):
             b.upload(np.full(b.nbytes // 4, np.nan, np.float32))
 
 
+@pytest.mark.parametrize("M,H,K1,I", [(16, 512, 512, 1024), (3, 512, 512, 1024), (16, 2048, 2048, 6144), (9, 2048, 2048, 6144)])
+def test_last_layer_form_ends_with_the_final_norm(M, H, K1, I):
+    """axhip_decode_layer_tail_last: h_out has the bits of the launch with a projection behind it (same phases 1-3),
+    and xn is the RMSNorm of exactly that h_out, rounded once to fp16 (the norm's sum runs over per-unit partial sums:
+    1 ulp of fp16 where the fp32 value sits next to a rounding boundary)."""
+    rng = np.random.default_rng(300 + M + H)
+    eps = 1e-6
+    attn = h16(rng.standard_normal((M, K1)))
+    h_in = rng.standard_normal((M, H)).astype(np.float32) * 3
+    wo, wd, wn = (h16(0.02 * rng.standard_normal(s)) for s in ((H, K1), (H, I), (64, H)))
+    wgu = h16(0.02 * rng.standard_normal((2 * I, H)))
+    w_post = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    w_fin = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    l = gu.lib()
+    assert l.axhip_decode_layer_tail_supported(M, H, K1, I, 0) == 1
+    d_attn, d_h, d_wp, d_wf = (gu.dev(a) for a in (attn, h_in, w_post, w_fin))
+    p_o, p_gu, p_d, p_n = _pack(wo), _pack(wgu, glu=True), _pack(wd), _pack(wn)
+    wsb = l.axhip_decode_layer_tail_workspace_bytes(H, I)
+    ws = gu.DeviceBuffer(wsb)
+    h_a, h_b, y, xn = (gu.DeviceBuffer(n) for n in (M * H * 4, M * H * 4, M * 64 * 4, M * H * 2))
+    failed = C.c_uint(0)
+    assert l.axhip_decode_layer_tail_status(1, C.byref(failed)) == 0
+    print(f"tail M={M} H={H}: with a projection behind it", flush=True)
+    gu._run("axhip_decode_layer_tail", d_attn.ptr, d_h.ptr, p_o.ptr, d_wp.ptr, p_gu.ptr, p_d.ptr, d_wf.ptr, p_n.ptr,
+            h_a.ptr, y.ptr, ws.ptr, wsb, M, H, K1, I, 64, eps, None)
+    gu.synchronize()
+    for it in range(2):
+        xn.upload(np.full(M * H // 2, np.nan, np.float32))
+        print(f"tail M={M} H={H}: last-layer form, launch {it}", flush=True)
+        gu._run("axhip_decode_layer_tail_last", d_attn.ptr, d_h.ptr, p_o.ptr, d_wp.ptr, p_gu.ptr, p_d.ptr, d_wf.ptr, h_b.ptr,
+                xn.ptr, ws.ptr, wsb, M, H, K1, I, eps, None)
+        gu.synchronize()
+        assert l.axhip_decode_layer_tail_status(0, C.byref(failed)) == 0 and failed.value == 0
+        ha, hb = h_a.download(np.float32, (M, H)), h_b.download(np.float32, (M, H))
+        np.testing.assert_array_equal(ha.view(np.uint32), hb.view(np.uint32))
+        got = xn.download(np.float16, (M, H))
+        want = port.rms_norm(hb, w_fin, eps)
+        assert np.all(np.isfinite(got))
+        ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float32)
+        assert np.all(np.abs(got.astype(np.float32) - want) <= 0.5 * ulp + 2e-6 * np.abs(want) + 1e-7)
+    # against the oracle's whole composition as well (a few fp16 flips behind the first norm: the bound of the test above)
+    ref_h, _ = _oracle(attn, h_in, wo, w_post, wgu, wd, w_fin, wn, eps)
+    assert float(np.abs(hb - ref_h).max()) <= 1e-3
+    assert l.axhip_decode_layer_tail_last(d_attn.ptr, d_h.ptr, p_o.ptr, d_wp.ptr, p_gu.ptr, p_d.ptr, d_wf.ptr, h_b.ptr,
+                                          None, ws.ptr, wsb, M, H, K1, I, eps, None) == 7
+
+
 def test_layer_tail_argument_checks():
     l = gu.lib()
     b = gu.DeviceBuffer(1 << 22)
@@ -105,6 +152,7 @@ def test_layer_tail_argument_checks():
     assert l.axhip_decode_layer_tail(*same, 16, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # h_out is h_in
     assert l.axhip_decode_layer_tail(*args[:11], 1024, 16, 2048, 2048, 6144, 4096, 1e-6, None) == 1   # workspace too small
     assert l.axhip_decode_layer_tail(*args, 0, 2048, 2048, 6144, 4096, 1e-6, None) == 0
+    assert l.axhip_decode_layer_tail(*args, 16, 2048, 2048, 6144, 0, 1e-6, None) == 1      # no projection: the _last form
     # the question a caller asks before it chooses between this launch and the single operators
     assert l.axhip_decode_layer_tail_supported(16, 2048, 2048, 6144, 4096) == 1
     assert l.axhip_decode_layer_tail_supported(16, 512, 512, 1024, 48) == 1

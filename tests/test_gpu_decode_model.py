@@ -356,6 +356,35 @@ def test_paged_decoder_gives_the_tokens_and_logits_of_the_dense_one():
         cur = outs["paged"][2][s]
 
 
+@pytest.mark.parametrize("paged", [False, True])
+def test_one_dealing_of_the_key_ranges_per_step_changes_no_bit(paged):
+    """The captured step whose attention launches of layers 1.. take their key ranges from the table layer 0's launch
+    leaves (the default) against the same model with every launch dealing for itself: same tokens and the same logits
+    of the last replay, bit for bit, over replays in which the lengths grow (ragged start: prefill of the longest,
+    then the lengths set by hand), dense and paged."""
+    n_steps = 7
+    shared, cpu, ids = _setup(seed=29, S=100, max_len=160)
+    B, S = ids.shape
+    each = Qwen3VLTextDecoder(CFG, cpu.w, B, 160, "hip:0", paged=paged, plan_reuse=False)
+    if paged:
+        shared = Qwen3VLTextDecoder(CFG, cpu.w, B, 160, "hip:0", paged=True)
+    assert shared._plan_reuse and not each._plan_reuse
+    outs = []
+    for m in (shared, each):
+        _, nxt = m.prefill(ids)
+        first = nxt.to_numpy().copy()
+        # sequences of different lengths: the rows beyond a sequence's length stay in the cache and are not attended
+        lens = np.array([S, S - 37, 5][:B], np.int32)
+        m.cache.set_lengths(lens)
+        m.start_decode(first, np.tile(lens.astype(np.int64), (3, 1)), n_steps)
+        m.capture()
+        toks = m.generate(n_steps)
+        outs.append((toks, m._graph_out[0].to_numpy().copy(), m.cache.seq_lens.to_numpy().copy()))
+    for a, b in zip(*outs):
+        np.testing.assert_array_equal(a, b)
+    np.testing.assert_array_equal(outs[0][2], [S + n_steps, S - 37 + n_steps, 5 + n_steps][:B])
+
+
 @pytest.mark.parametrize("fused_tail,n_layers", [(False, 2), (True, 3)])
 def test_captured_step_at_the_real_widths_of_the_2b_shape(fused_tail, n_layers):
     """The launches of the benchmark's decode step at their real sizes, two or three layers deep (three with the

@@ -203,7 +203,8 @@ def run(decode_steps: int = 128, batch: int = 16, context: int = 4096, seed: int
     log(f"[decode]   sum of the per-kind graphs {in_kernels:.0f} us of the {ms_step * 1e3:.0f} us step")
     result.update({
         "per_kernel": {"how": "each kind of launch captured for all layers (own weights / caches) and replayed back to "
-                              "back; host clock around 10 replays; bytes are algorithmic",
+                              "back; host clock around 10 replays; bytes are algorithmic; a kind with 0 calls per step is "
+                              "not part of this step (the single operators the fused layer launch replaces), timed for comparison",
                        "cols": ["kernel", "calls_per_step", "us_per_call", "us_per_step", "bytes_per_call", "frac_hbm_peak"],
                        "rows": [[r["kernel"], r["calls_per_step"], r["us_per_call"], r["us_per_step"], r["bytes_per_call"],
                                  r["frac_hbm_peak"]] for r in table],

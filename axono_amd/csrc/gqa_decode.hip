@@ -259,8 +259,8 @@ struct DecodeArgs {
   const int32_t *page_table;
   int max_pages, n_pages;
   int64_t page_stride;  // elements per page: Hkv * kPageKeys * D
-  // Decode-step form with lengths dealt in the kernel: the 28 attention launches of a step deal the same lengths
-  // the same way.  plan_mode 1: a launch leaves what every slot found (8 ints per slot) in plan_cache; 2: a launch
+  // Decode-step form with lengths dealt in the kernel: the attention launches of a step (one per layer) deal the
+  // same lengths the same way.  plan_mode 1: a launch leaves what every slot found (8 ints per slot) in plan_cache; 2: a launch
   // reads that instead of the lengths and the dealing.  plan_check marks the entries of a launch of this shape.
   int *plan_cache;
   int plan_mode, plan_check;
@@ -1360,7 +1360,7 @@ int plan_and_launch(DecodeArgs &a, void *workspace, size_t workspace_bytes, int 
     }
     a.plan_cache = p + static_cast<size_t>(axhip_ticket_lane()) * kPlanSlots * 8;
     a.plan_mode = axhip_plan_reuse();
-    // entries left by a launch of another shape, or dealt for other lengths storage, are not taken
+    // entries left by a launch of another shape, or dealt from another lengths array, are not taken
     unsigned h = 2166136261u;
     for (const long long v : {static_cast<long long>(B), static_cast<long long>(Hq), static_cast<long long>(G),
                               static_cast<long long>(max_len), static_cast<long long>(plan.active),
